@@ -1,0 +1,192 @@
+/*
+ * q8mi.h — C ABI of the MI355X (gfx950) Q8_0 x Q8_1 quantized-linear library.
+ *
+ * This is the drop-in boundary for qw3's Q8_0 linear hot path: every entry
+ * point below replaces one `qw3::ported::launch_*` launcher (declared by the
+ * reference at src/kernels_cuda.cu:56-125) or one of the argmax kernels the
+ * reference's CUDA backend launches itself.  Paths in comments are relative to
+ * the reference checkout.
+ *
+ * Conventions
+ *   - All data pointers are caller-owned DEVICE pointers unless a parameter is
+ *     documented as host memory.  Nothing here allocates, frees or synchronises
+ *     (src/mmvq_q8.cu:19-22); work is enqueued on `stream` (a hipStream_t passed
+ *     as void*, NULL = the default stream) and is capturable into a HIP graph.
+ *   - Return value: Q8MI_OK, Q8MI_REJECTED (the reference launcher would have
+ *     returned false: nothing was enqueued) or Q8MI_LAUNCH_ERROR (the HIP
+ *     runtime reported an error; text via q8mi_last_error()).
+ *   - Weights use the reference's split-plane row layout
+ *     (src/cuda_helpers.cuh:16-39): row r starts at r*nb*34 bytes and holds
+ *     nb fp16 scales followed by nb*32 int8 quants, nb = cols/32.
+ *   - Activations are Q8_1 blocks of 36 B (src/mmvq_q8.cu:48-52) for the GEMV
+ *     family, or 144-B D4 super-blocks (src/mmvq_q8.cu:60-64) with block index
+ *     (k/128)*batch + j for the MFMA GEMM.
+ *   - Outputs are [batch][stride_dst_row]; element (j, r) lives at
+ *     j*stride_dst_row + r.
+ */
+#ifndef Q8MI_H
+#define Q8MI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define Q8MI_OK 0
+#define Q8MI_REJECTED 1
+#define Q8MI_LAUNCH_ERROR 2
+
+#define Q8MI_MAX_GEMV_BATCH 8
+
+/* Device-visible argmax record; byte-identical to the reference's ArgmaxPair
+ * (src/kernels_cuda.cu:1741-1744), which its device-chained MTP draft loop
+ * reads on the GPU (src/kernels_cuda.cu:2110-2133). */
+typedef struct q8mi_argmax_pair {
+    float value;
+    int32_t index;
+} q8mi_argmax_pair;
+
+/* Thread-local text of the last Q8MI_LAUNCH_ERROR / Q8MI_REJECTED on this thread. */
+const char *q8mi_last_error(void);
+/* Library ABI version (bumped on any signature change). */
+int q8mi_abi_version(void);
+
+/* ---- Q8_1 activation quantizer ------------------------------------------- */
+/* replaces q8_1_scratch_bytes, src/mmvq_q8.cu:613-616 */
+size_t q8mi_q8_1_scratch_bytes(uint32_t batch, uint32_t cols);
+/* replaces launch_quantize_q8_1, src/mmvq_q8.cu:623-640 (kernel :82-112).
+ * Rejects cols % 32 != 0. */
+int q8mi_quantize_q8_1(const float *x, void *y_q8_1, uint32_t batch, uint32_t cols,
+                       uint32_t stride_x_row, void *stream);
+
+/* ---- GEMV family, batch 1..8 --------------------------------------------- */
+/* replaces launch_mmvq_q8_0, src/mmvq_q8.cu:805-811.  Rejects cols % 32 != 0,
+ * batch == 0, batch > 8 (src/mmvq_q8.cu:773-774). */
+int q8mi_gemv(const uint8_t *weight, const void *y_q8_1, float *dst, uint32_t rows, uint32_t cols,
+              uint32_t batch, uint32_t stride_dst_row, void *stream);
+/* replaces launch_mmvq_q8_0_bf16, src/mmvq_q8.cu:813-819 (dst is bf16 bits) */
+int q8mi_gemv_bf16(const uint8_t *weight, const void *y_q8_1, uint16_t *dst, uint32_t rows,
+                   uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
+/* replaces launch_mmvq_q8_0_two, src/mmvq_q8.cu:823-864 */
+int q8mi_gemv_two(const uint8_t *weight0, const uint8_t *weight1, const void *y_q8_1, float *dst0,
+                  float *dst1, uint32_t rows, uint32_t cols, uint32_t batch,
+                  uint32_t stride_dst_row, void *stream);
+/* replaces launch_mmvq_q8_0_silu_mul, src/mmvq_q8.cu:869-909:
+ * dst = silu(Wg x) * (Wu x), silu(g) = g / (1 + exp(-g)) */
+int q8mi_gemv_silu_mul(const uint8_t *weight_gate, const uint8_t *weight_up, const void *y_q8_1,
+                       float *dst, uint32_t rows, uint32_t cols, uint32_t batch,
+                       uint32_t stride_dst_row, void *stream);
+/* replaces launch_mmvq_q8_0_add, src/mmvq_q8.cu:955-961: dst += W x */
+int q8mi_gemv_add(const uint8_t *weight, const void *y_q8_1, float *dst, uint32_t rows,
+                  uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
+/* replaces launch_mmvq_q8_0_add_bf16, src/mmvq_q8.cu:963-969 */
+int q8mi_gemv_add_bf16(const uint8_t *weight, const void *y_q8_1, uint16_t *dst, uint32_t rows,
+                       uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
+/* replaces launch_mmvq_q8_0_fanout4_batch, src/mmvq_q8.cu:1070-1113.  A slot
+ * with a NULL weight, NULL dst or zero rows is skipped; rejects a total of
+ * zero rows. */
+int q8mi_gemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uint8_t *weight2,
+                      const uint8_t *weight3, const void *y_q8_1, float *dst0, float *dst1,
+                      float *dst2, float *dst3, uint32_t rows0, uint32_t rows1, uint32_t rows2,
+                      uint32_t rows3, uint32_t cols, uint32_t batch, uint32_t stride_dst0,
+                      uint32_t stride_dst1, uint32_t stride_dst2, uint32_t stride_dst3,
+                      void *stream);
+
+/* ---- D4 activation quantizer + int8 MFMA GEMM ---------------------------- */
+/* replaces q8_1_mmq_scratch_bytes, src/mmvq_q8.cu:726-729 */
+size_t q8mi_q8_1_d4_scratch_bytes(uint32_t batch, uint32_t cols);
+/* replaces launch_quantize_mmq_q8_1, src/mmvq_q8.cu:736-755 (kernel :668-722).
+ * Rejects cols % 128 != 0. */
+int q8mi_quantize_q8_1_d4(const float *x, void *y_d4, uint32_t batch, uint32_t cols,
+                          uint32_t stride_x_row, void *stream);
+/* replaces launch_mmq_q8_0, src/mmq_q8.cu:2278-2501.  As in the reference the
+ * activation layout is implied by the shape (src/kernels_cuda.cu:14545-14552):
+ * rows >= 128 && cols % 128 == 0 -> y is D4 (144-B super-blocks); otherwise y is
+ * Q8_1 (36-B blocks).  Rejects cols % 32 != 0, rows == 0, batch == 0. */
+int q8mi_gemm(const uint8_t *weight, const void *y, float *dst, uint32_t rows, uint32_t cols,
+              uint32_t batch, uint32_t stride_dst_row, void *stream);
+/* replaces launch_mmq_q8_0_medium, src/mmq_q8.cu:2512-2548: y is always D4.
+ * Rejects cols % 128 != 0, rows == 0, batch == 0, batch > 64. */
+int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *dst, uint32_t rows,
+                     uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
+
+/* Checker hook (no counterpart in the reference): writes the int32 block dots
+ * S[row][j][kb] = sum_t q_w*q_x for n sampled (row, j, kb) triples, computed on
+ * the GPU with the same int8 dot instruction the kernels use.  y_layout:
+ * 0 = Q8_1, 1 = D4.  sample arrays and out are device pointers. */
+int q8mi_block_dots(const uint8_t *weight, const void *y, int y_layout, uint32_t rows,
+                    uint32_t cols, uint32_t batch, const uint32_t *sample_row,
+                    const uint32_t *sample_j, const uint32_t *sample_kb, uint32_t n, int32_t *out,
+                    void *stream);
+
+/* ---- argmax -------------------------------------------------------------- */
+/* replaces argmax_kernel, src/kernels_cuda.cu:1693-1734 (launched at :20759):
+ * out2[0] = index (-1 if no element is above -inf), out2[1] = bits of the max. */
+int q8mi_argmax(const float *x, uint64_t n, int32_t *out2, void *stream);
+/* replaces argmax_pair_kernel, src/kernels_cuda.cu:1804-1857 (launched :20787) */
+int q8mi_argmax_to_pair(const float *x, uint64_t n, q8mi_argmax_pair *out, uint32_t out_index,
+                     void *stream);
+/* replaces argmax_rows_block_kernel + argmax_rows_finalize_kernel,
+ * src/kernels_cuda.cu:1773-1802, 1859-1888 (launched :20814-20836).  Rejects
+ * row_stride == 0 and rows wider than 1024*256 (the reference falls back to a
+ * host scan there).  scratch: q8mi_argmax_rows_scratch_bytes() device bytes. */
+size_t q8mi_argmax_rows_scratch_bytes(uint32_t batch, uint32_t row_stride);
+int q8mi_argmax_rows(const float *x, uint32_t batch, uint32_t row_stride, void *scratch,
+                     q8mi_argmax_pair *result, void *stream);
+
+/* ---- fused LM head ------------------------------------------------------- */
+/* No single counterpart in the reference: fuses the verify tail
+ * q8_0_matmul(W_out) -> argmax_batch -> greedy accept
+ * (src/qwen_executor.cpp:6779-6821, src/kernels_cuda.cu:20814-20850,
+ * src/qwen_native_backend.cpp:15948-15960, 16048-16052) into one pass over the
+ * LM-head weights that never materialises the batch x vocab logits.
+ *   rows        vocabulary size (weight rows), cols = hidden size
+ *   batch       1..8 verify rows; row i gates drafts[i]; n_drafts = batch - 1
+ *   drafts      batch-1 draft token ids; host memory when drafts_on_device == 0
+ *               (they are passed by value), device memory otherwise
+ *   row_out     device, batch pairs {max logit, token} (ties -> lowest token)
+ *   accept_out  device int32[2]: {accept length, next token} where next token =
+ *               row_out[accept].index, or eos if that index is negative
+ *   logits      optional device [batch][stride_logits] fp32 copy of the logits
+ *               (NULL = do not write them)
+ *   scratch     q8mi_lm_head_scratch_bytes(rows, cols, batch) device bytes
+ */
+size_t q8mi_lm_head_scratch_bytes(uint32_t rows, uint32_t cols, uint32_t batch);
+int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y_q8_1, uint32_t rows,
+                               uint32_t cols, uint32_t batch, const int32_t *drafts,
+                               int drafts_on_device, int32_t eos, q8mi_argmax_pair *row_out,
+                               int32_t *accept_out, float *logits, uint32_t stride_logits,
+                               void *scratch, void *stream);
+
+/* ---- weight upload (host side) ------------------------------------------- */
+/* replaces the repack loop of the CudaWeight constructor,
+ * src/kernels_cuda.cu:1566-1594: interleaved GGUF Q8_0 blocks (34 B: fp16 d,
+ * 32 int8) -> split-plane rows.  Both pointers are HOST memory. */
+int q8mi_repack_q8_0_split_host(const void *gguf_blocks, uint64_t rows, uint64_t cols,
+                                void *split_out);
+/* Same repack done on the GPU (both pointers device memory; in != out). */
+int q8mi_repack_q8_0_split(const void *gguf_blocks, uint64_t rows, uint64_t cols, void *split_out,
+                           void *stream);
+
+/* ---- synthetic inputs (host side, for benches and tests) ----------------- */
+/* Counter-based generator: element i of stream `seed` depends only on
+ * (seed, i), so any thread split gives the same bytes.
+ *   kind 0: N(0,1) * scale
+ *   kind 1: Student-t(nu=3)/sqrt(3) * scale, with every column whose hash
+ *           (seed, col) falls in the lowest `outlier_ppm` millionths multiplied
+ *           by outlier_gain (BASELINE config 4: 1000 ppm, gain 20).
+ * out: host fp32 [rows][cols]. */
+int q8mi_synth_f32(float *out, uint64_t rows, uint64_t cols, uint64_t seed, int kind, float scale,
+                   uint32_t outlier_ppm, float outlier_gain, int threads);
+/* N(0, sigma^2) weights quantized to Q8_0 (tests/mmq_parity.cu:54-80 rule:
+ * d = amax/127 stored fp16, q = clamp(lrintf(w * (1/d)), +-127)) and written
+ * straight into split-plane rows.  out: host, rows*cols/32*34 bytes. */
+int q8mi_synth_q8_0_weight(uint8_t *split_out, uint64_t rows, uint64_t cols, uint64_t seed,
+                           float sigma, int threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* Q8MI_H */

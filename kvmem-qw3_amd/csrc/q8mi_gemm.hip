@@ -1,0 +1,297 @@
+// Prefill GEMM: Q8_0 weights x D4-quantized activations on the gfx950 int8
+// matrix cores (v_mfma_i32_32x32x32_i8; K = 32 is exactly one Q8 block, so each
+// instruction yields the int32 dot of one block for a 32 x 32 patch of outputs).
+// Reference semantics: src/mmq_q8.cu:2164-2273 — one int32 sum per 32-block,
+// rescaled by d_w * d_y in fp32 and accumulated in ascending block order.
+//
+// Tiling
+//   workgroup  128 weight rows x 128 activation rows (batch), 4 waves
+//   wave       32 activation rows x 128 weight rows = four 32x32 MFMA patches
+//   K step     one 128-element super-block (4 Q8 blocks), double-buffered in LDS
+// The MFMA "A" operand is the activation patch and "B" the weight patch, so a
+// lane owns ONE weight row (lane % 32) and 16 activation rows per patch.  That
+// makes the fp16 weight scale a per-lane constant and the output stores
+// contiguous along the weight-row axis (dst is [batch][rows]).
+//
+// LDS record (144 B, both operands): [4 x fp32 scales][128 x int8].  The 144-B
+// pitch is what the D4 activation blocks already have in memory, and it spreads
+// the 16-byte fragment reads of 8 consecutive rows over all banks.  Activation
+// scales are kept a second time, transposed ([sub-block][row]), so a lane can
+// fetch the four scales of four consecutive activation rows with one 16-B read.
+//
+// Rescale without an int->float conversion: the MFMA accumulator is seeded with
+// the bit pattern of 1.5*2^23, so the int32 result reinterpreted as fp32 is
+// F = 12582912 + S exactly (|S| <= 516128 < 2^22).  g = fma(F, d_w, -12582912*d_w)
+// is then the correctly rounded d_w*S (12582912*d_w is exact: d_w has 11
+// significant bits), and acc = fma(g, d_y, acc): two FMAs per (output, block).
+#include "q8mi_device.hpp"
+#include "q8mi_internal.hpp"
+
+namespace q8mi {
+
+// GEMV-based route for shapes the MFMA tile does not cover (defined in
+// q8mi_gemv.hip): y is Q8_1, any batch, processed eight activation rows at a time.
+int gemv_any_batch(const uint8_t *w, const void *y_q8_1, float *dst, uint32_t rows, uint32_t cols,
+                   uint32_t batch, uint32_t stride_dst_row, hipStream_t stream);
+
+namespace {
+
+constexpr int kTileRows = 128;   // weight rows per workgroup
+constexpr int kTileCols = 128;   // activation rows (batch) per workgroup
+constexpr int kGemmThreads = 256;
+constexpr int kRec = 144;        // LDS record pitch in bytes
+constexpr int kStageBytes = kTileRows * kRec + kTileCols * kRec + 4 * kTileCols * 4;  // 38912
+constexpr int kLdsBytes = 2 * kStageBytes;                                             // 77824
+constexpr uint32_t kMagicBits = 0x4B400000u;  // 1.5 * 2^23
+constexpr float kMagic = 12582912.0f;
+
+struct Prefetch {
+    v4i wq[4];   // 4 x 16 B of weight quants
+    uint2 wd;    // 4 fp16 weight scales (threads 0..127)
+    v4i yq[5];   // up to 5 x 16 B of activation records
+};
+
+// 16 bytes from an address that is 16-byte aligned (A16) or only 8-byte aligned
+// (rows of cols/32 % 8 == 4 start on an odd multiple of 8).
+template <bool A16>
+__device__ __forceinline__ v4i load16(const uint8_t *p) {
+    if (A16) return *reinterpret_cast<const v4i *>(p);
+    const uint2 lo = *reinterpret_cast<const uint2 *>(p);
+    const uint2 hi = *reinterpret_cast<const uint2 *>(p + 8);
+    v4i v;
+    v.x = static_cast<int>(lo.x); v.y = static_cast<int>(lo.y);
+    v.z = static_cast<int>(hi.x); v.w = static_cast<int>(hi.y);
+    return v;
+}
+
+template <bool CHECK, bool A16>
+__device__ __forceinline__ void prefetch_load(Prefetch &pf, const uint8_t *__restrict__ w,
+                                              const uint8_t *__restrict__ y, uint32_t rows, uint32_t nb,
+                                              uint32_t batch, uint32_t row0, uint32_t col0, uint32_t sb,
+                                              uint32_t tid) {
+    const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t c = tid + kGemmThreads * p;
+        const uint32_t r = c >> 3, piece = c & 7u;
+        v4i v = {0, 0, 0, 0};
+        if (!CHECK || row0 + r < rows) {
+            v = load16<A16>(w + (row0 + r) * row_bytes + 2 * nb + sb * 128 + piece * 16);
+        }
+        pf.wq[p] = v;
+    }
+    pf.wd = make_uint2(0u, 0u);
+    if (tid < kTileRows && (!CHECK || row0 + tid < rows)) {
+        pf.wd = *reinterpret_cast<const uint2 *>(w + (row0 + tid) * row_bytes + sb * 8);
+    }
+    const uint8_t *ysrc = y + (static_cast<uint64_t>(sb) * batch + col0) * kRec;
+#pragma unroll
+    for (int p = 0; p < 5; ++p) {
+        const uint32_t c = tid + kGemmThreads * p;
+        v4i v = {0, 0, 0, 0};
+        if (c < kTileCols * 9 && (!CHECK || col0 + c / 9 < batch)) {
+            v = *reinterpret_cast<const v4i *>(ysrc + static_cast<uint64_t>(c) * 16);
+        }
+        pf.yq[p] = v;
+    }
+}
+
+__device__ __forceinline__ void prefetch_store(const Prefetch &pf, uint8_t *stage, uint32_t tid) {
+    uint8_t *lw = stage;
+    uint8_t *ly = stage + kTileRows * kRec;
+    float *ysc = reinterpret_cast<float *>(stage + kTileRows * kRec + kTileCols * kRec);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t c = tid + kGemmThreads * p;
+        const uint32_t r = c >> 3, piece = c & 7u;
+        *reinterpret_cast<v4i *>(lw + r * kRec + 16 + piece * 16) = pf.wq[p];
+    }
+    if (tid < kTileRows) {
+        float4 d;
+        d.x = half_bits_to_float(static_cast<uint16_t>(pf.wd.x & 0xffffu));
+        d.y = half_bits_to_float(static_cast<uint16_t>(pf.wd.x >> 16));
+        d.z = half_bits_to_float(static_cast<uint16_t>(pf.wd.y & 0xffffu));
+        d.w = half_bits_to_float(static_cast<uint16_t>(pf.wd.y >> 16));
+        *reinterpret_cast<float4 *>(lw + tid * kRec) = d;
+    }
+#pragma unroll
+    for (int p = 0; p < 5; ++p) {
+        const uint32_t c = tid + kGemmThreads * p;
+        if (c < kTileCols * 9) {
+            *reinterpret_cast<v4i *>(ly + c * 16) = pf.yq[p];
+            if (c % 9 == 0) {  // record header: the four fp32 scales, also kept transposed
+                const uint32_t j = c / 9;
+                ysc[0 * kTileCols + j] = as_f32(pf.yq[p].x);
+                ysc[1 * kTileCols + j] = as_f32(pf.yq[p].y);
+                ysc[2 * kTileCols + j] = as_f32(pf.yq[p].z);
+                ysc[3 * kTileCols + j] = as_f32(pf.yq[p].w);
+            }
+        }
+    }
+}
+
+template <bool CHECK, bool A16>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_kernel(
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles,
+        uint32_t col_tiles) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid % kWave;
+    const uint32_t wave = tid / kWave;
+    const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
+
+    // Tile order: consecutive workgroup ids land on different XCDs (8 of them,
+    // each with its own L2).  Give every XCD whole row tiles, and walk the
+    // column tiles of one row tile back to back so its weights stay in that L2.
+    const uint32_t id = blockIdx.x;
+    const uint32_t xcd = id % 8u, seq = id / 8u;
+    const uint32_t rt_local = seq / col_tiles, ct = seq % col_tiles;
+    const uint32_t rt = rt_local * 8u + xcd;
+    if (rt >= row_tiles) return;  // uniform for the workgroup
+    const uint32_t row0 = rt * kTileRows, col0 = ct * kTileCols;
+
+    const uint32_t nsb = nb / 4;
+    v16i zero_c;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) zero_c[i] = static_cast<int>(kMagicBits);
+
+    float acc[4][16];
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
+
+    Prefetch pf;
+    prefetch_load<CHECK, A16>(pf, w, y, rows, nb, batch, row0, col0, 0, tid);
+    prefetch_store(pf, smem, tid);
+    __syncthreads();
+
+    for (uint32_t sb = 0; sb < nsb; ++sb) {
+        uint8_t *cur = smem + (sb & 1u) * kStageBytes;
+        uint8_t *nxt = smem + ((sb + 1u) & 1u) * kStageBytes;
+        const bool more = sb + 1 < nsb;
+        if (more) prefetch_load<CHECK, A16>(pf, w, y, rows, nb, batch, row0, col0, sb + 1, tid);
+
+        const uint8_t *lw = cur;
+        const uint8_t *ly = cur + kTileRows * kRec;
+        const float *ysc = reinterpret_cast<const float *>(cur + kTileRows * kRec + kTileCols * kRec);
+
+        // one Q8 block (K = 32) per trip; kept rolled so that only the four
+        // 32x32 result patches of one block are live at a time
+#pragma unroll 1
+        for (uint32_t sub = 0; sub < 4; ++sub) {
+            const uint32_t frag_off = 16 + sub * 32 + lhalf * 16;
+            const v4i a = *reinterpret_cast<const v4i *>(ly + (wave * 32 + l32) * kRec + frag_off);
+            float dy[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 t = *reinterpret_cast<const float4 *>(
+                    ysc + sub * kTileCols + wave * 32 + 8 * g + 4 * lhalf);
+                dy[4 * g + 0] = t.x; dy[4 * g + 1] = t.y; dy[4 * g + 2] = t.z; dy[4 * g + 3] = t.w;
+            }
+            v16i r[4];
+            float dw[4];
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const uint8_t *rec = lw + (rb * 32 + l32) * kRec;
+                const v4i b = *reinterpret_cast<const v4i *>(rec + frag_off);
+                dw[rb] = *reinterpret_cast<const float *>(rec + sub * 4);
+                r[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero_c, 0, 0, 0);
+            }
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const float cw = -kMagic * dw[rb];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float g = fmaf(as_f32(r[rb][v]), dw[rb], cw);
+                    acc[rb][v] = fmaf(g, dy[v], acc[rb][v]);
+                }
+            }
+        }
+
+        if (more) prefetch_store(pf, nxt, tid);
+        __syncthreads();
+    }
+
+    // D[i][n]: n = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (activation row)
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+        const uint32_t r = row0 + rb * 32 + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t j = col0 + wave * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
+            if (!CHECK || (r < rows && j < batch)) {
+                dst[static_cast<uint64_t>(j) * stride_dst + r] = acc[rb][v];
+            }
+        }
+    }
+}
+
+template <bool CHECK, bool A16>
+int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb,
+                   uint32_t batch, uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid,
+                   hipStream_t stream) {
+    // more than 64 KiB of dynamic LDS has to be granted per kernel, once per process
+    static bool granted = false;
+    if (!granted) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_kernel<CHECK, A16>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", kLdsBytes);
+        }
+        granted = true;
+    }
+    gemm_d4_kernel<CHECK, A16><<<grid, kGemmThreads, kLdsBytes, stream>>>(
+        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
+    return check_launch("gemm");
+}
+
+int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,
+                   uint32_t batch, uint32_t stride, hipStream_t stream) {
+    const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
+    const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
+    const uint32_t rt_padded = (row_tiles + 7u) / 8u * 8u;
+    const uint64_t grid64 = static_cast<uint64_t>(rt_padded) * col_tiles;
+    if (grid64 > 0x7fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    const uint32_t grid = static_cast<uint32_t>(grid64);
+    const bool check = (rows % kTileRows != 0) || (batch % kTileCols != 0);
+    const uint32_t nb = cols / kQK;
+    const bool a16 = nb % 8 == 0;
+    const auto *yb = static_cast<const uint8_t *>(y);
+    if (check) {
+        return a16 ? launch_variant<true, true>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
+                   : launch_variant<true, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
+    }
+    return a16 ? launch_variant<false, true>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
+               : launch_variant<false, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
+}
+
+}  // namespace
+}  // namespace q8mi
+
+using namespace q8mi;
+
+extern "C" int q8mi_gemm(const uint8_t *weight, const void *y, float *dst, uint32_t rows, uint32_t cols,
+                         uint32_t batch, uint32_t stride_dst_row, void *stream) {
+    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "gemm: cols %u not a multiple of 32", cols);
+    if (batch == 0 || rows == 0) return fail(Q8MI_REJECTED, "gemm: empty shape");
+    if (cols == 0) return fail(Q8MI_REJECTED, "gemm: cols is zero");
+    if (reinterpret_cast<uintptr_t>(weight) % 16 != 0)
+        return fail(Q8MI_REJECTED, "gemm: weight pointer not 16-byte aligned");
+    if (rows >= 128 && cols % 128 == 0) {
+        return launch_gemm_d4(weight, y, dst, rows, cols, batch, stride_dst_row, as_stream(stream));
+    }
+    return gemv_any_batch(weight, y, dst, rows, cols, batch, stride_dst_row, as_stream(stream));
+}
+
+extern "C" int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *dst, uint32_t rows,
+                                uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream) {
+    if (cols % 128 != 0) return fail(Q8MI_REJECTED, "gemm_medium: cols %u not a multiple of 128", cols);
+    if (batch == 0 || rows == 0) return fail(Q8MI_REJECTED, "gemm_medium: empty shape");
+    if (batch > 64) return fail(Q8MI_REJECTED, "gemm_medium: batch %u above 64", batch);
+    if (cols == 0) return fail(Q8MI_REJECTED, "gemm_medium: cols is zero");
+    if (reinterpret_cast<uintptr_t>(weight) % 16 != 0)
+        return fail(Q8MI_REJECTED, "gemm_medium: weight pointer not 16-byte aligned");
+    return launch_gemm_d4(weight, y_d4, dst, rows, cols, batch, stride_dst_row, as_stream(stream));
+}

@@ -1,0 +1,246 @@
+// Host-side pieces of the library: error text, device queries, the weight
+// repack (host and device), the block-dot checker hook and the synthetic input
+// generator.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <thread>
+#include <vector>
+
+#include "q8mi_device.hpp"
+#include "q8mi_internal.hpp"
+
+namespace q8mi {
+
+namespace {
+thread_local char g_err[256] = "";
+}
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return Q8MI_OK;
+    return fail(Q8MI_LAUNCH_ERROR, "%s: %s", what, hipGetErrorString(e));
+}
+
+int device_cu_count() {
+    static thread_local int cached_dev = -1;
+    static thread_local int cached_cus = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev != cached_dev) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        cached_dev = dev;
+        cached_cus = cus;
+    }
+    return cached_cus;
+}
+
+namespace {
+
+// ---- device repack: interleaved 34-B blocks -> split-plane rows ------------
+// One thread moves one block: 2 scale bytes + 32 quant bytes (the source block
+// is only 2-byte aligned, so it is read as 17 halfwords).
+__global__ __launch_bounds__(256) void repack_kernel(const uint16_t *__restrict__ in,
+                                                     uint8_t *__restrict__ out, uint64_t rows,
+                                                     uint64_t nb) {
+    const uint64_t b = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (b >= rows * nb) return;
+    const uint64_t row = b / nb, kb = b % nb;
+    const uint16_t *src = in + b * 17;
+    uint8_t *row_out = out + row * nb * 34;
+    reinterpret_cast<uint16_t *>(row_out)[kb] = src[0];
+    uint16_t *q = reinterpret_cast<uint16_t *>(row_out + 2 * nb + kb * 32);
+#pragma unroll
+    for (int t = 0; t < 16; ++t) q[t] = src[1 + t];
+}
+
+// ---- checker hook: int32 block dots on the GPU -------------------------------
+__global__ __launch_bounds__(256) void block_dots_kernel(const uint8_t *__restrict__ w,
+                                                         const uint8_t *__restrict__ y, int layout,
+                                                         uint32_t nb, uint32_t batch,
+                                                         const uint32_t *__restrict__ sr,
+                                                         const uint32_t *__restrict__ sj,
+                                                         const uint32_t *__restrict__ sk, uint32_t n,
+                                                         int32_t *__restrict__ out) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t row = sr[i], j = sj[i], kb = sk[i];
+    const uint16_t *wq = reinterpret_cast<const uint16_t *>(w + static_cast<uint64_t>(row) * nb * 34 + 2 * nb +
+                                                            static_cast<uint64_t>(kb) * 32);
+    const uint8_t *xq8 = layout == 0
+        ? y + (static_cast<uint64_t>(j) * nb + kb) * kQ81Bytes + 4
+        : y + (static_cast<uint64_t>(kb / 4) * batch + j) * kD4Bytes + 16 + (kb % 4) * 32;
+    const int *xq = reinterpret_cast<const int *>(xq8);
+    int s = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const int a = static_cast<int>(wq[2 * t]) | (static_cast<int>(wq[2 * t + 1]) << 16);
+        s = __builtin_amdgcn_sdot4(a, xq[t], s, false);
+    }
+    out[i] = s;
+}
+
+// ---- synthetic inputs --------------------------------------------------------
+inline uint64_t splitmix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+inline uint64_t draw(uint64_t seed, uint64_t stream, uint64_t i) {
+    return splitmix64(splitmix64(seed * 0xD1342543DE82EF95ull + stream) + i);
+}
+
+// uniform in (0, 1): 53 random bits, never 0
+inline double unit(uint64_t bits) { return (static_cast<double>(bits >> 11) + 0.5) * (1.0 / 9007199254740992.0); }
+
+// standard normal from two independent draws (Box-Muller, cosine branch)
+inline double normal(uint64_t seed, uint64_t stream, uint64_t i) {
+    const double u1 = unit(draw(seed, stream, 2 * i));
+    const double u2 = unit(draw(seed, stream, 2 * i + 1));
+    return sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2);
+}
+
+template <typename F>
+void parallel_rows(uint64_t rows, int threads, F fn) {
+    if (threads < 1) threads = 1;
+    if (static_cast<uint64_t>(threads) > rows) threads = rows ? static_cast<int>(rows) : 1;
+    if (threads == 1) {
+        fn(0, rows);
+        return;
+    }
+    std::vector<std::thread> pool;
+    const uint64_t chunk = (rows + threads - 1) / threads;
+    for (int t = 0; t < threads; ++t) {
+        const uint64_t lo = chunk * t, hi = lo + chunk < rows ? lo + chunk : rows;
+        if (lo >= hi) break;
+        pool.emplace_back([=] { fn(lo, hi); });
+    }
+    for (auto &th : pool) th.join();
+}
+
+inline uint16_t f32_to_f16_host(float f) { return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); }
+
+}  // namespace
+}  // namespace q8mi
+
+using namespace q8mi;
+
+extern "C" const char *q8mi_last_error(void) { return g_err; }
+
+extern "C" int q8mi_abi_version(void) { return 1; }
+
+extern "C" int q8mi_repack_q8_0_split_host(const void *gguf_blocks, uint64_t rows, uint64_t cols,
+                                           void *split_out) {
+    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "repack: cols %llu not a multiple of 32", (unsigned long long)cols);
+    const uint64_t nb = cols / kQK;
+    const uint8_t *in = static_cast<const uint8_t *>(gguf_blocks);
+    uint8_t *out = static_cast<uint8_t *>(split_out);
+    for (uint64_t r = 0; r < rows; ++r) {
+        const uint8_t *src = in + r * nb * 34;
+        uint8_t *d_plane = out + r * nb * 34;
+        uint8_t *q_plane = d_plane + 2 * nb;
+        for (uint64_t b = 0; b < nb; ++b, src += 34) {
+            memcpy(d_plane + 2 * b, src, 2);
+            memcpy(q_plane + 32 * b, src + 2, 32);
+        }
+    }
+    return Q8MI_OK;
+}
+
+extern "C" int q8mi_repack_q8_0_split(const void *gguf_blocks, uint64_t rows, uint64_t cols,
+                                      void *split_out, void *stream) {
+    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "repack: cols %llu not a multiple of 32", (unsigned long long)cols);
+    if (gguf_blocks == split_out) return fail(Q8MI_REJECTED, "repack: in-place repack is not supported");
+    const uint64_t nb = cols / kQK;
+    const uint64_t blocks = rows * nb;
+    if (blocks == 0) return Q8MI_OK;
+    const uint64_t grid = (blocks + 255) / 256;
+    if (grid > 0x7fffffffull) return fail(Q8MI_REJECTED, "repack: tensor too large for one launch");
+    repack_kernel<<<static_cast<uint32_t>(grid), 256, 0, as_stream(stream)>>>(
+        static_cast<const uint16_t *>(gguf_blocks), static_cast<uint8_t *>(split_out), rows, nb);
+    return check_launch("repack");
+}
+
+extern "C" int q8mi_block_dots(const uint8_t *weight, const void *y, int y_layout, uint32_t rows,
+                               uint32_t cols, uint32_t batch, const uint32_t *sample_row,
+                               const uint32_t *sample_j, const uint32_t *sample_kb, uint32_t n,
+                               int32_t *out, void *stream) {
+    (void)rows;
+    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "block_dots: cols %u not a multiple of 32", cols);
+    if (y_layout != 0 && y_layout != 1) return fail(Q8MI_REJECTED, "block_dots: unknown layout %d", y_layout);
+    if (y_layout == 1 && cols % 128 != 0) return fail(Q8MI_REJECTED, "block_dots: D4 needs cols %% 128 == 0");
+    if (n == 0) return Q8MI_OK;
+    block_dots_kernel<<<(n + 255) / 256, 256, 0, as_stream(stream)>>>(
+        weight, static_cast<const uint8_t *>(y), y_layout, cols / kQK, batch, sample_row, sample_j,
+        sample_kb, n, out);
+    return check_launch("block_dots");
+}
+
+extern "C" int q8mi_synth_f32(float *out, uint64_t rows, uint64_t cols, uint64_t seed, int kind,
+                              float scale, uint32_t outlier_ppm, float outlier_gain, int threads) {
+    if (kind != 0 && kind != 1) return fail(Q8MI_REJECTED, "synth_f32: unknown kind %d", kind);
+    parallel_rows(rows, threads, [=](uint64_t lo, uint64_t hi) {
+        for (uint64_t r = lo; r < hi; ++r) {
+            for (uint64_t c = 0; c < cols; ++c) {
+                const uint64_t i = r * cols + c;
+                double v;
+                if (kind == 0) {
+                    v = normal(seed, 0, i);
+                } else {
+                    // Student-t(3) = Z / sqrt(chi2_3 / 3); unit variance after / sqrt(3)
+                    const double z = normal(seed, 0, i);
+                    const double a = normal(seed, 1, i), b = normal(seed, 2, i), d = normal(seed, 3, i);
+                    const double chi2 = a * a + b * b + d * d;
+                    v = z / sqrt(chi2 / 3.0) / 1.7320508075688772;
+                    if (outlier_ppm != 0 && draw(seed, 4, c) % 1000000ull < outlier_ppm) v *= outlier_gain;
+                }
+                out[i] = static_cast<float>(v * scale);
+            }
+        }
+    });
+    return Q8MI_OK;
+}
+
+extern "C" int q8mi_synth_q8_0_weight(uint8_t *split_out, uint64_t rows, uint64_t cols, uint64_t seed,
+                                      float sigma, int threads) {
+    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "synth_q8_0_weight: cols %llu not a multiple of 32", (unsigned long long)cols);
+    const uint64_t nb = cols / kQK;
+    parallel_rows(rows, threads, [=](uint64_t lo, uint64_t hi) {
+        float blk[kQK];
+        for (uint64_t r = lo; r < hi; ++r) {
+            uint8_t *d_plane = split_out + r * nb * 34;
+            int8_t *q_plane = reinterpret_cast<int8_t *>(d_plane + 2 * nb);
+            for (uint64_t kb = 0; kb < nb; ++kb) {
+                float amax = 0.0f;
+                for (int t = 0; t < kQK; ++t) {
+                    blk[t] = static_cast<float>(normal(seed, 0, r * cols + kb * kQK + t) * sigma);
+                    amax = fmaxf(amax, fabsf(blk[t]));
+                }
+                const float d = amax / 127.0f;
+                const float d_inv = d == 0.0f ? 0.0f : 1.0f / d;
+                const uint16_t hd = f32_to_f16_host(d);
+                memcpy(d_plane + 2 * kb, &hd, 2);
+                for (int t = 0; t < kQK; ++t) {
+                    long q = lrintf(blk[t] * d_inv);
+                    q = q < -127 ? -127 : (q > 127 ? 127 : q);
+                    q_plane[kb * kQK + t] = static_cast<int8_t>(q);
+                }
+            }
+        }
+    });
+    return Q8MI_OK;
+}

@@ -1,0 +1,167 @@
+"""Minimal ctypes view of the HIP runtime: device memory, streams, events.
+
+Used by the tests and the bench to own device buffers and to time launches on
+the stream the kernels run on.  It binds the same libamdhip64 the C-ABI library
+is linked against, so there is exactly one HIP runtime in the process.
+"""
+import ctypes as C
+
+import numpy as np
+
+_rt = None
+
+hipMemcpyHostToDevice = 1
+hipMemcpyDeviceToHost = 2
+hipMemcpyDeviceToDevice = 3
+
+
+class HipError(RuntimeError):
+    pass
+
+
+def rt():
+    global _rt
+    if _rt is None:
+        last = None
+        for name in ("libamdhip64.so.7", "libamdhip64.so", "/opt/rocm/lib/libamdhip64.so"):
+            try:
+                _rt = C.CDLL(name, mode=C.RTLD_GLOBAL)
+                break
+            except OSError as e:  # pragma: no cover - depends on the box
+                last = e
+        if _rt is None:
+            raise HipError(f"cannot load the HIP runtime: {last}")
+        _rt.hipGetErrorString.restype = C.c_char_p
+        _rt.hipGetErrorString.argtypes = [C.c_int]
+    return _rt
+
+
+def check(code, what=""):
+    if code != 0:
+        msg = rt().hipGetErrorString(code)
+        raise HipError(f"{what}: HIP error {code}: {msg.decode() if msg else '?'}")
+
+
+def device_count():
+    n = C.c_int(0)
+    try:
+        code = rt().hipGetDeviceCount(C.byref(n))
+    except HipError:
+        return 0
+    return n.value if code == 0 else 0
+
+
+def set_device(i):
+    check(rt().hipSetDevice(C.c_int(i)), "hipSetDevice")
+
+
+def synchronize():
+    check(rt().hipDeviceSynchronize(), "hipDeviceSynchronize")
+
+
+def device_name():
+    # hipDeviceGetName(char*, int, hipDevice_t)
+    buf = C.create_string_buffer(256)
+    check(rt().hipDeviceGetName(buf, C.c_int(256), C.c_int(0)), "hipDeviceGetName")
+    return buf.value.decode()
+
+
+class DeviceBuffer:
+    """Owning device allocation."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        self._ptr = C.c_void_p(0)
+        check(rt().hipMalloc(C.byref(self._ptr), C.c_size_t(max(self.nbytes, 1))), "hipMalloc")
+
+    @property
+    def ptr(self):
+        return self._ptr.value
+
+    def at(self, offset):
+        return C.c_void_p(self._ptr.value + int(offset))
+
+    def free(self):
+        if self._ptr is not None and self._ptr.value:
+            rt().hipFree(self._ptr)
+            self._ptr = C.c_void_p(0)
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:  # interpreter shutdown
+            pass
+
+    # -- transfers (synchronous) --
+    def upload(self, arr, offset=0):
+        a = np.ascontiguousarray(arr)
+        assert offset + a.nbytes <= self.nbytes, "upload past the end of the buffer"
+        if a.nbytes:
+            check(rt().hipMemcpy(self.at(offset), a.ctypes.data_as(C.c_void_p), C.c_size_t(a.nbytes),
+                                 C.c_int(hipMemcpyHostToDevice)), "hipMemcpy H2D")
+        return self
+
+    def download(self, dtype, count=None, offset=0):
+        dtype = np.dtype(dtype)
+        if count is None:
+            count = (self.nbytes - offset) // dtype.itemsize
+        out = np.empty(count, dtype)
+        assert offset + out.nbytes <= self.nbytes, "download past the end of the buffer"
+        if out.nbytes:
+            check(rt().hipMemcpy(out.ctypes.data_as(C.c_void_p), self.at(offset), C.c_size_t(out.nbytes),
+                                 C.c_int(hipMemcpyDeviceToHost)), "hipMemcpy D2H")
+        return out
+
+    def fill(self, byte=0):
+        check(rt().hipMemset(self._ptr, C.c_int(byte), C.c_size_t(self.nbytes)), "hipMemset")
+        return self
+
+
+def to_device(arr):
+    a = np.ascontiguousarray(arr)
+    return DeviceBuffer(a.nbytes).upload(a)
+
+
+class Stream:
+    def __init__(self):
+        self._s = C.c_void_p(0)
+        check(rt().hipStreamCreate(C.byref(self._s)), "hipStreamCreate")
+
+    @property
+    def handle(self):
+        return self._s
+
+    def synchronize(self):
+        check(rt().hipStreamSynchronize(self._s), "hipStreamSynchronize")
+
+    def __del__(self):
+        try:
+            if self._s.value:
+                rt().hipStreamDestroy(self._s)
+        except Exception:
+            pass
+
+
+class Event:
+    def __init__(self):
+        self._e = C.c_void_p(0)
+        check(rt().hipEventCreate(C.byref(self._e)), "hipEventCreate")
+
+    def record(self, stream=None):
+        s = stream.handle if stream is not None else C.c_void_p(0)
+        check(rt().hipEventRecord(self._e, s), "hipEventRecord")
+
+    def synchronize(self):
+        check(rt().hipEventSynchronize(self._e), "hipEventSynchronize")
+
+    def elapsed_ms(self, end):
+        ms = C.c_float(0)
+        check(rt().hipEventElapsedTime(C.byref(ms), self._e, end._e), "hipEventElapsedTime")
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self._e.value:
+                rt().hipEventDestroy(self._e)
+        except Exception:
+            pass

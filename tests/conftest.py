@@ -1,0 +1,34 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "kvmem-qw3_amd"), os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    """The CPU oracle (built on demand from oracle/q8_oracle.c)."""
+    from oracle import q8_oracle
+    q8_oracle.lib()
+    return q8_oracle
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """Loaded C-ABI library + HIP runtime on device 0.  Fails (not skips) when the
+    library is not built: GPU tests must never pass without the native code."""
+    import q8mi
+    from q8mi import hip
+    if hip.device_count() < 1:
+        pytest.fail("GPU test selected but no HIP device is visible")
+    hip.set_device(0)
+    q8mi.lib()
+    return q8mi

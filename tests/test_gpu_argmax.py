@@ -1,0 +1,176 @@
+"""GPU parity: argmax kernels and the fused LM head + greedy accept, bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import q8mi
+from gpu_common import NULL, dev, quantize_q8_1
+from q8mi import hip, ok, synth
+
+pytestmark = pytest.mark.gpu
+
+PAIR = np.dtype([("value", np.float32), ("index", np.int32)])
+
+
+def adversarial_rows(n, seed):
+    rng = np.random.default_rng(seed)
+    rows = []
+    r = rng.standard_normal(n).astype(np.float32)
+    rows.append(r.copy())
+    t = r.copy(); m = t.max(); t[[n // 3, n // 2, n - 1]] = m + 1.0     # ties of the maximum
+    rows.append(t)
+    rows.append(np.full(n, -np.inf, np.float32))                          # nothing above -inf
+    t = np.full(n, -np.inf, np.float32); t[n - 1] = -1e30
+    rows.append(t)
+    rows.append(np.zeros(n, np.float32))                                  # all equal
+    t = np.zeros(n, np.float32); t[1::2] = -0.0
+    rows.append(t)
+    t = r.copy(); t[::5] = np.nan                                         # NaN never wins a `>`
+    rows.append(t)
+    t = r.copy(); t[0] = np.nan; t[n - 1] = np.nan; t[255 % n] = np.nan
+    rows.append(t)
+    t = r.copy(); t[n // 2] = np.inf
+    rows.append(t)
+    return np.stack(rows)
+
+
+@pytest.mark.parametrize("n", [1, 31, 256, 1024, 1025, 248320])
+def test_argmax_single_row(gpu, oracle, n):
+    rows = adversarial_rows(n, seed=n)
+    L = q8mi.lib()
+    out2 = hip.DeviceBuffer(8)
+    pairs = hip.DeviceBuffer(8 * 4)
+    for i, r in enumerate(rows):
+        dx = dev(r)
+        ok(L.q8mi_argmax(dx.ptr, n, out2.ptr, NULL), "argmax")
+        ok(L.q8mi_argmax_to_pair(dx.ptr, n, pairs.ptr, i % 4, NULL), "argmax_to_pair")
+        hip.synchronize()
+        got = out2.download(np.int32)
+        v, idx = oracle.argmax_row(r)
+        assert got[0] == idx, f"row {i}: index {got[0]} != {idx}"
+        assert got[1] == np.float32(v).view(np.int32), f"row {i}: value bits differ"
+        p = pairs.download(PAIR)[i % 4]
+        assert p["index"] == idx and p["value"].view(np.int32) == np.float32(v).view(np.int32)
+
+
+def test_argmax_empty_row(gpu):
+    out2 = hip.DeviceBuffer(8)
+    ok(q8mi.lib().q8mi_argmax(out2.ptr, 0, out2.ptr, NULL), "argmax")
+    hip.synchronize()
+    got = out2.download(np.int32)
+    assert got[0] == -1 and got[1] == np.float32(-np.inf).view(np.int32)
+
+
+@pytest.mark.parametrize("row_stride", [1, 255, 256, 257, 5000, 248320])
+def test_argmax_rows_matches_reference_network(gpu, oracle, row_stride):
+    rows = adversarial_rows(row_stride, seed=row_stride + 1)
+    batch = rows.shape[0]
+    L = q8mi.lib()
+    scratch = hip.DeviceBuffer(L.q8mi_argmax_rows_scratch_bytes(batch, row_stride))
+    res = hip.DeviceBuffer(8 * batch)
+    dx = dev(rows)
+    ok(L.q8mi_argmax_rows(dx.ptr, batch, row_stride, scratch.ptr, res.ptr, NULL), "argmax_rows")
+    hip.synchronize()
+    got = res.download(PAIR)
+    rc, ref = oracle.argmax_rows(rows, batch, row_stride)
+    assert rc == 0
+    assert np.array_equal(got["index"], ref["index"])
+    assert np.array_equal(got["value"].view(np.int32), ref["value"].view(np.int32))
+
+
+def test_argmax_rows_rejections(gpu):
+    L = q8mi.lib()
+    b = hip.DeviceBuffer(64)
+    assert L.q8mi_argmax_rows(b.ptr, 2, 0, b.ptr, b.ptr, NULL) == q8mi.REJECTED
+    assert L.q8mi_argmax_rows(b.ptr, 2, 1024 * 256 + 1, b.ptr, b.ptr, NULL) == q8mi.REJECTED
+
+
+def run_lm_head(w_dev, y_dev, vocab, cols, batch, drafts, eos, want_logits=False, on_device=False):
+    L = q8mi.lib()
+    scratch = hip.DeviceBuffer(L.q8mi_lm_head_scratch_bytes(vocab, cols, batch))
+    row_out = hip.DeviceBuffer(8 * batch)
+    acc = hip.DeviceBuffer(8)
+    logits = hip.DeviceBuffer(4 * batch * vocab) if want_logits else None
+    d = np.ascontiguousarray(drafts, np.int32)
+    if on_device:
+        dd = dev(d) if d.size else None
+        dptr = dd.ptr if dd is not None else None
+    else:
+        dptr = d.ctypes.data_as(C.c_void_p) if d.size else None
+    ok(L.q8mi_lm_head_argmax_accept(w_dev.ptr, y_dev.ptr, vocab, cols, batch, dptr, 1 if on_device else 0,
+                                    eos, row_out.ptr, acc.ptr, logits.ptr if logits else None, vocab,
+                                    scratch.ptr, NULL), "lm_head")
+    hip.synchronize()
+    pairs = row_out.download(PAIR)
+    a = acc.download(np.int32)
+    lg = logits.download(np.float32).reshape(batch, vocab) if want_logits else None
+    return pairs, int(a[0]), int(a[1]), lg
+
+
+@pytest.mark.parametrize("batch", [1, 2, 4, 6, 8])
+def test_lm_head_fused_matches_unfused_and_oracle(gpu, oracle, batch):
+    vocab, cols = 20000, 1024
+    w = synth.q8_0_weight(vocab, cols, seed=500)
+    x = synth.normal(batch, cols, seed=600 + batch)
+    dw = dev(w)
+    dy, y = quantize_q8_1(x)
+    rc, ref_logits = oracle.gemv(w, y, vocab, cols, batch)
+    ref_pairs = oracle.argmax_rows_scan(ref_logits, batch, vocab)
+    ref_tokens = ref_pairs["index"]
+    rng = np.random.default_rng(batch)
+    for prefix in range(batch):            # forced-match prefix of every possible length
+        drafts = rng.integers(0, vocab, batch - 1).astype(np.int32)
+        drafts[:prefix] = ref_tokens[:prefix]
+        if prefix < batch - 1 and drafts[prefix] == ref_tokens[prefix]:
+            drafts[prefix] = (drafts[prefix] + 1) % vocab
+        exp_len, exp_next = oracle.accept(ref_tokens, drafts, eos=2)
+        assert exp_len == prefix
+        for on_device in (False, True):
+            pairs, n_acc, nxt, lg = run_lm_head(dw, dy, vocab, cols, batch, drafts, 2,
+                                                want_logits=(prefix == 0), on_device=on_device)
+            assert np.array_equal(pairs["index"], ref_tokens), "row argmax tokens differ"
+            assert n_acc == exp_len and nxt == exp_next
+            # winning logits are the GPU's own fp32 values: within tolerance of the oracle's
+            assert np.allclose(pairs["value"], ref_pairs["value"], rtol=1e-5, atol=1e-6)
+            if lg is not None:
+                # the fused kernel's optional logits equal the plain GEMV's bit for bit
+                out = hip.DeviceBuffer(4 * batch * vocab)
+                ok(q8mi.lib().q8mi_gemv(dw.ptr, dy.ptr, out.ptr, vocab, cols, batch, vocab, NULL), "gemv")
+                hip.synchronize()
+                plain = out.download(np.float32).reshape(batch, vocab)
+                assert np.array_equal(lg.view(np.uint32), plain.view(np.uint32))
+                assert np.array_equal(pairs["value"].view(np.uint32),
+                                      plain[np.arange(batch), pairs["index"]].view(np.uint32))
+
+
+def test_lm_head_ties_and_eos(gpu, oracle):
+    """Duplicate weight rows give exactly equal logits: the lowest token id must win,
+    whichever workgroup met it first."""
+    vocab, cols, batch = 6000, 512, 3
+    w = synth.q8_0_weight(vocab, cols, seed=9)
+    x = synth.normal(batch, cols, seed=10)
+    dy, y = quantize_q8_1(x)
+    rc, logits = oracle.gemv(w, y, vocab, cols, batch)
+    top = int(np.argmax(logits[0]))
+    for dup in (5, 4097, 5999):
+        if dup != top:
+            w[dup] = w[top]
+    dw = dev(w)
+    rc, logits = oracle.gemv(w, y, vocab, cols, batch)
+    ref = oracle.argmax_rows_scan(logits, batch, vocab)
+    assert ref["index"][0] == min(top, 5)
+    pairs, n_acc, nxt, _ = run_lm_head(dw, dy, vocab, cols, batch, ref["index"][:2], eos=7)
+    assert np.array_equal(pairs["index"], ref["index"])
+    assert n_acc == 2 and nxt == ref["index"][2]
+
+
+def test_lm_head_rejections(gpu):
+    L = q8mi.lib()
+    b = hip.DeviceBuffer(1 << 16)
+    d = np.zeros(8, np.int32).ctypes.data_as(C.c_void_p)
+    args = lambda rows, cols, batch: (b.ptr, b.ptr, rows, cols, batch, d, 0, 0, b.ptr, b.ptr, None, rows, b.ptr, NULL)
+    assert L.q8mi_lm_head_argmax_accept(*args(100, 500, 2)) == q8mi.REJECTED
+    assert L.q8mi_lm_head_argmax_accept(*args(100, 512, 0)) == q8mi.REJECTED
+    assert L.q8mi_lm_head_argmax_accept(*args(100, 512, 9)) == q8mi.REJECTED
+    assert L.q8mi_lm_head_argmax_accept(*args(0, 512, 2)) == q8mi.REJECTED

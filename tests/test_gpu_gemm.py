@@ -1,0 +1,172 @@
+"""GPU parity: D4 quantizer + int8 MFMA GEMM through the C ABI vs the CPU oracle."""
+import numpy as np
+import pytest
+
+import q8mi
+from gpu_common import NULL, assert_close_fp32, dev, quantize_d4, quantize_q8_1
+from q8mi import hip, ok, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gemm(dw, dy, rows, cols, batch, stride=None, medium=False):
+    stride = rows if stride is None else stride
+    out = hip.DeviceBuffer(4 * batch * stride).fill(0xff)
+    fn = q8mi.lib().q8mi_gemm_medium if medium else q8mi.lib().q8mi_gemm
+    ok(fn(dw.ptr, dy.ptr, out.ptr, rows, cols, batch, stride, NULL), "gemm")
+    hip.synchronize()
+    return out.download(np.float32).reshape(batch, stride)
+
+
+def d4_block_dots(oracle, dw, w, dy, y, rows, cols, batch, seed, n=2048):
+    rng = np.random.default_rng(seed)
+    sr = rng.integers(0, rows, n, dtype=np.uint32)
+    sj = rng.integers(0, batch, n, dtype=np.uint32)
+    sk = rng.integers(0, cols // 32, n, dtype=np.uint32)
+    out = hip.DeviceBuffer(4 * n)
+    a, b, c = dev(sr), dev(sj), dev(sk)
+    ok(q8mi.lib().q8mi_block_dots(dw.ptr, dy.ptr, 1, rows, cols, batch, a.ptr, b.ptr, c.ptr, n, out.ptr, NULL),
+       "block_dots")
+    hip.synchronize()
+    got = out.download(np.int32)
+    ref = np.array([oracle.block_dot(w, y, 1, cols, batch, int(r), int(j), int(k))
+                    for r, j, k in zip(sr, sj, sk)], np.int32)
+    assert np.array_equal(got, ref)
+    assert np.abs(got).max() <= 516128
+
+
+# (rows M, batch N, cols K): the reference's own parity shapes (tests/mmq_parity.cu:275-295)
+REFERENCE_SHAPES = [
+    (128, 128, 256), (128, 128, 1024), (128, 128, 2048), (256, 128, 2048), (128, 256, 2048),
+    (256, 256, 1024), (384, 256, 2048), (2048, 2048, 2048), (2304, 2048, 2304), (640, 2048, 2304),
+    (2048, 2048, 2304), (2304, 2271, 2304), (2048, 2271, 2304), (2304, 223, 2304),
+    (2048, 223, 2304), (640, 223, 2304),
+]
+
+
+@pytest.mark.parametrize("rows,batch,cols", REFERENCE_SHAPES)
+def test_gemm_reference_shapes(gpu, oracle, rows, batch, cols):
+    w = synth.q8_0_weight(rows, cols, seed=rows + cols)
+    x = synth.normal(batch, cols, seed=batch + cols + 1)
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    rc, yref = oracle.quantize_q8_1_d4(x)
+    assert np.array_equal(y, yref), "quantized activations must be bit-exact"
+    got = run_gemm(dw, dy, rows, cols, batch)
+    big = rows * batch > 512 * 512
+    if not big:
+        rc, ref = oracle.gemm_d4(w, y, rows, cols, batch, threads=8)
+        rr, jj = np.meshgrid(np.arange(rows, dtype=np.uint32), np.arange(batch, dtype=np.uint32))
+        rc, ref_s, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr.reshape(-1), jj.reshape(-1))
+        assert np.array_equal(ref_s.reshape(batch, rows), ref)
+        assert_close_fp32(got, ref, absum, f"gemm {rows}x{batch}x{cols}")
+    else:
+        rng = np.random.default_rng(rows)
+        n = 20000
+        sr = rng.integers(0, rows, n, dtype=np.uint32)
+        sj = rng.integers(0, batch, n, dtype=np.uint32)
+        # always include the corners and the last row / column of every tile edge
+        sr[:4] = [0, rows - 1, 0, rows - 1]
+        sj[:4] = [0, 0, batch - 1, batch - 1]
+        rc, ref_s, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, sr, sj)
+        assert_close_fp32(got[sj, sr], ref_s, absum, f"gemm {rows}x{batch}x{cols} (sampled)")
+    assert np.isfinite(got).all()
+    d4_block_dots(oracle, dw, w, dy, y, rows, cols, batch, seed=cols, n=512)
+
+
+def test_gemm_reference_tolerance_restated(gpu):
+    """tests/mmq_parity.cu:246-254 restated: output vs fp32 dot of the dequantised
+    operands within 5e-3 abs or 1e-3 rel, U(-0.5,0.5) weights and U(-1,1) activations."""
+    rows, batch, cols = 256, 256, 1024
+    rng = np.random.default_rng(0x5EED)
+    wf = rng.uniform(-0.5, 0.5, (rows, cols)).astype(np.float32)
+    x = rng.uniform(-1, 1, (batch, cols)).astype(np.float32)
+    from oracle import q8_oracle as o   # only to build the Q8_0 weight bytes (test input)
+    w = o.make_weight(wf)
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    got = run_gemm(dw, dy, rows, cols, batch)
+    nb = cols // 32
+    dq_w = (w[:, 2 * nb:].view(np.int8).reshape(rows, nb, 32).astype(np.float32)
+            * w[:, :2 * nb].copy().view(np.float16).astype(np.float32)[:, :, None]).reshape(rows, cols)
+    yb = y.reshape(cols // 128, batch, 144)
+    d4 = yb[:, :, :16].copy().view(np.float32)                      # [sb, j, 4]
+    qs = yb[:, :, 16:].view(np.int8).reshape(cols // 128, batch, 4, 32).astype(np.float32)
+    dq_x = (qs * d4[..., None]).transpose(1, 0, 2, 3).reshape(batch, cols)
+    ref = dq_x @ dq_w.T
+    d = np.abs(got - ref)
+    assert np.all((d <= 5e-3) | (d <= 1e-3 * np.maximum(np.abs(ref), 1e-6)))
+
+
+@pytest.mark.parametrize("rows,batch,cols", [(128, 1, 128), (129, 9, 384), (200, 33, 640), (500, 64, 1152),
+                                             (1000, 12, 5120)])
+def test_gemm_ragged_and_medium(gpu, oracle, rows, batch, cols):
+    """Tile-edge handling (rows, batch not multiples of 128; cols/32 % 8 == 4) and the
+    medium-batch entry point."""
+    w = synth.q8_0_weight(rows, cols, seed=rows * 7 + cols)
+    x = synth.normal(batch, cols, seed=batch * 13 + cols)
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    rc, ref = oracle.gemm_d4(w, y, rows, cols, batch, threads=8)
+    rr, jj = np.meshgrid(np.arange(rows, dtype=np.uint32), np.arange(batch, dtype=np.uint32))
+    rc, _, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr.reshape(-1), jj.reshape(-1))
+    stride = rows + 3
+    got = run_gemm(dw, dy, rows, cols, batch, stride=stride)
+    assert_close_fp32(got[:, :rows], ref, absum, "gemm ragged")
+    assert np.all(got[:, rows:].view(np.uint32) == 0xffffffff), "stores must stay inside the rows"
+    got_m = run_gemm(dw, dy, rows, cols, batch, medium=True)
+    assert np.array_equal(got_m.view(np.uint32), got[:, :rows].view(np.uint32))
+
+
+def test_gemm_small_shapes_take_q8_1(gpu, oracle):
+    """rows < 128 or cols % 128 != 0: the entry point expects Q8_1 activations, as the
+    reference's launcher does for those shapes (src/kernels_cuda.cu:14545-14552)."""
+    for rows, batch, cols in [(64, 20, 256), (300, 11, 160), (16, 32, 96)]:
+        w = synth.q8_0_weight(rows, cols, seed=rows)
+        x = synth.normal(batch, cols, seed=batch)
+        dw = dev(w)
+        dy, y = quantize_q8_1(x)
+        got = run_gemm(dw, dy, rows, cols, batch)
+        ref = np.zeros((batch, rows), np.float32)
+        absum = np.zeros((batch, rows), np.float32)
+        for j0 in range(0, batch, 8):
+            m = min(8, batch - j0)
+            ysl = y.reshape(batch, -1)[j0:j0 + m].reshape(-1)
+            rc, r = oracle.gemv(w, ysl, rows, cols, m)
+            rc, a = oracle.gemv_abs(w, ysl, rows, cols, m)
+            ref[j0:j0 + m] = r
+            absum[j0:j0 + m] = a
+        assert_close_fp32(got, ref, absum, f"gemm small {rows}x{batch}x{cols}")
+
+
+def test_gemm_equals_gemv_at_block_level(gpu, oracle):
+    """Same int8 inputs through GEMV (Q8_1) and GEMM (D4) give the same int32 block
+    dots whenever both quantizers agree on q (they do when x/d and x*(127/amax)
+    round alike); here both are compared with the oracle instead of each other."""
+    rows, batch, cols = 256, 8, 1024
+    w = synth.q8_0_weight(rows, cols, seed=1)
+    x = synth.normal(batch, cols, seed=2)
+    dw = dev(w)
+    dy1, y1 = quantize_q8_1(x)
+    dy4, y4 = quantize_d4(x)
+    q1 = y1.reshape(batch, cols // 32, 36)[:, :, 4:]
+    q4 = y4.reshape(cols // 128, batch, 144)[:, :, 16:].reshape(cols // 128, batch, 4, 32)
+    q4 = q4.transpose(1, 0, 2, 3).reshape(batch, cols // 32, 32)
+    same = (q1 == q4).all(axis=2)
+    assert same.mean() > 0.9
+    for j, kb in zip(*np.nonzero(same)):
+        if (j + kb) % 37:
+            continue
+        a = oracle.block_dot(w, y1, 0, cols, batch, 3, int(j), int(kb))
+        b = oracle.block_dot(w, y4, 1, cols, batch, 3, int(j), int(kb))
+        assert a == b
+
+
+def test_gemm_rejections(gpu):
+    L = q8mi.lib()
+    b = hip.DeviceBuffer(1 << 16)
+    assert L.q8mi_gemm(b.ptr, b.ptr, b.ptr, 128, 100, 4, 128, NULL) == q8mi.REJECTED
+    assert L.q8mi_gemm(b.ptr, b.ptr, b.ptr, 0, 128, 4, 128, NULL) == q8mi.REJECTED
+    assert L.q8mi_gemm(b.ptr, b.ptr, b.ptr, 128, 128, 0, 128, NULL) == q8mi.REJECTED
+    assert L.q8mi_gemm_medium(b.ptr, b.ptr, b.ptr, 128, 160, 4, 128, NULL) == q8mi.REJECTED
+    assert L.q8mi_gemm_medium(b.ptr, b.ptr, b.ptr, 128, 128, 65, 128, NULL) == q8mi.REJECTED
