@@ -1,0 +1,293 @@
+#!/usr/bin/env python3
+"""Bench of the Q8_0 quantized-linear hot path on one MI355X.
+
+One "step" = one pass over the decode GEMV set of one 27B-style layer at M=1
+(BASELINE config 1), through the C ABI exactly as the executor would drive it:
+
+    quantize_q8_1(x[5120])   -> gemv_fanout4  Q 5120x6144, K 5120x1024, V 5120x1024
+    quantize_q8_1(a[6144])   -> gemv_add      O 6144x5120   (residual add)
+    quantize_q8_1(x[5120])   -> gemv_silu_mul gate, up 5120x17408 each
+    quantize_q8_1(f[17408])  -> gemv_add      down 17408x5120
+
+`value` is algorithmic bytes per step / time per step with all inputs resident
+in HBM, cycling through several distinct copies of the layer's weights so that
+no copy can be served from the 256 MB last-level cache ("streaming").  The same
+loop on a single copy is reported as `resident_gbps`.
+
+Prints ONE JSON line (see the keys at the bottom).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "kvmem-qw3_amd"))
+
+HBM_PEAK_GBPS = 8000.0        # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0       # MI355X published dense int8 MFMA rate (TOP/s)
+
+HIDDEN, QDIM, KVDIM, ATTN_OUT, FFN, VOCAB = 5120, 24 * 256, 4 * 256, 6144, 17408, 248320
+
+
+def w_bytes(rows, cols):
+    return rows * (cols // 32) * 34
+
+
+def q81_bytes(m, cols):
+    return m * (cols // 32) * 36
+
+
+class Layer:
+    """Device-resident Q8_0 weights of one layer (one seed)."""
+
+    def __init__(self, synth, hip, seed):
+        shapes = {"q": (QDIM, HIDDEN), "k": (KVDIM, HIDDEN), "v": (KVDIM, HIDDEN), "o": (HIDDEN, ATTN_OUT),
+                  "gate": (FFN, HIDDEN), "up": (FFN, HIDDEN), "down": (HIDDEN, FFN)}
+        self.w = {}
+        for i, (name, (rows, cols)) in enumerate(shapes.items()):
+            host = synth.q8_0_weight(rows, cols, seed=seed * 16 + i, sigma=0.02)
+            self.w[name] = hip.to_device(host)
+        self.bytes = sum(w_bytes(r, c) for r, c in shapes.values())
+
+
+class DecodeStep:
+    """Buffers + the launch sequence of one layer's decode GEMVs for batch m."""
+
+    def __init__(self, q8mi, hip, m, seed=1):
+        from q8mi import synth
+        self.L = q8mi.lib()
+        self.ok = q8mi.ok
+        self.m = m
+        f32 = lambda n: hip.DeviceBuffer(4 * n)
+        self.x = hip.to_device(synth.normal(m, HIDDEN, seed=seed))          # normed hidden state
+        self.attn = hip.to_device(synth.normal(m, ATTN_OUT, seed=seed + 1))  # attention output
+        self.h = hip.to_device(synth.normal(m, HIDDEN, seed=seed + 2))       # residual stream
+        self.q, self.k, self.v = f32(m * QDIM), f32(m * KVDIM), f32(m * KVDIM)
+        self.ffn = f32(m * FFN)
+        self.y5120 = hip.DeviceBuffer(q81_bytes(m, HIDDEN))
+        self.y6144 = hip.DeviceBuffer(q81_bytes(m, ATTN_OUT))
+        self.y17408 = hip.DeviceBuffer(q81_bytes(m, FFN))
+
+    def algorithmic_bytes(self, layer_bytes):
+        m = self.m
+        act = 2 * q81_bytes(m, HIDDEN) + q81_bytes(m, ATTN_OUT) + q81_bytes(m, FFN)
+        outs = 4 * m * (QDIM + 2 * KVDIM + HIDDEN + FFN + HIDDEN)
+        return layer_bytes + act + outs
+
+    def run(self, layer, stream=None):
+        L, m, w = self.L, self.m, layer.w
+        ok = self.ok
+        ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize")
+        ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.y5120.ptr,
+                               self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
+                               HIDDEN, m, QDIM, KVDIM, KVDIM, 0, stream), "fanout4")
+        ok(L.q8mi_quantize_q8_1(self.attn.ptr, self.y6144.ptr, m, ATTN_OUT, ATTN_OUT, stream), "quantize")
+        ok(L.q8mi_gemv_add(w["o"].ptr, self.y6144.ptr, self.h.ptr, HIDDEN, ATTN_OUT, m, HIDDEN, stream), "o")
+        ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize")
+        self.run_silu(layer, stream)
+        ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, m, FFN, FFN, stream), "quantize")
+        ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, m, HIDDEN, stream), "down")
+
+    def run_silu(self, layer, stream=None):
+        self.ok(self.L.q8mi_gemv_silu_mul(layer.w["gate"].ptr, layer.w["up"].ptr, self.y5120.ptr, self.ffn.ptr,
+                                          FFN, HIDDEN, self.m, FFN, stream), "silu_mul")
+
+    def silu_bytes(self):
+        return 2 * w_bytes(FFN, HIDDEN) + q81_bytes(self.m, HIDDEN) + 4 * self.m * FFN
+
+
+def time_loop(hip, fn, steps, warmup):
+    """Device time of `steps` calls of fn(i), HIP events on the (default) stream."""
+    for i in range(warmup):
+        fn(i)
+    hip.synchronize()
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record()
+    for i in range(steps):
+        fn(warmup + i)
+    e1.record()
+    e1.synchronize()
+    hip.synchronize()
+    return e0.elapsed_ms(e1) / steps
+
+
+def time_each_launch(hip, fn, n, warmup=5):
+    """Average duration of single launches, one event pair per launch."""
+    for i in range(warmup):
+        fn(i)
+    hip.synchronize()
+    pairs = [(hip.Event(), hip.Event()) for _ in range(n)]
+    for i, (a, b) in enumerate(pairs):
+        a.record()
+        fn(warmup + i)
+        b.record()
+    hip.synchronize()
+    ds = np.array([a.elapsed_ms(b) for a, b in pairs])
+    return float(ds.mean()), float(np.median(ds)), float(ds.min())
+
+
+def cpu_baseline(seconds=12.0):
+    """The oracle's scalar GEMV (oracle/q8_oracle.c) on BASELINE config 0
+    (5120x5120, M=1), timed on this host: once on one core, once row-parallel."""
+    sys.path.insert(0, ROOT)
+    from oracle import q8_oracle as o
+    from q8mi import synth
+    rows = cols = HIDDEN
+    w = synth.q8_0_weight(rows, cols, seed=12345)
+    x = synth.normal(1, cols, seed=54321)
+    rc, y = o.quantize_q8_1(x)
+    nbytes = w_bytes(rows, cols) + q81_bytes(1, cols) + 4 * rows
+
+    def run(threads, budget):
+        o.gemv(w, y, rows, cols, 1, threads=threads)     # warm
+        n, t0 = 0, time.perf_counter()
+        while True:
+            o.gemv(w, y, rows, cols, 1, threads=threads)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt >= budget:
+                return nbytes * n / dt / 1e9, n
+
+    cores = min(16, os.cpu_count() or 1)
+    one, n1 = run(1, seconds / 2)
+    many, nm = run(cores, seconds / 2)
+    return {"value": round(many, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"oracle q8o_gemv, config 0 (5120x5120, M=1), {nm} calls row-parallel on {cores} threads "
+                      f"(~{seconds / 2:.0f} s); single core: {one:.3f} GB/s over {n1} calls",
+            "value_1core": round(one, 3)}
+
+
+def bench_gemm(q8mi, hip, synth, reps=10):
+    """Prefill GEMM (D4 quantize + MFMA GEMM) at M=2048 on the two FFN shapes."""
+    L, ok = q8mi.lib(), q8mi.ok
+    out = {}
+    m = 2048
+    for name, rows, cols in (("k5120_n17408", FFN, HIDDEN), ("k17408_n5120", HIDDEN, FFN)):
+        w = hip.to_device(synth.q8_0_weight(rows, cols, seed=rows + 7))
+        x = hip.to_device(synth.normal(m, cols, seed=cols + 9))
+        y = hip.DeviceBuffer(L.q8mi_q8_1_d4_scratch_bytes(m, cols))
+        dst = hip.DeviceBuffer(4 * m * rows)
+        ok(L.q8mi_quantize_q8_1_d4(x.ptr, y.ptr, m, cols, cols, None), "quantize_d4")
+        gemm = lambda i: ok(L.q8mi_gemm(w.ptr, y.ptr, dst.ptr, rows, cols, m, rows, None), "gemm")
+        quant = lambda i: ok(L.q8mi_quantize_q8_1_d4(x.ptr, y.ptr, m, cols, cols, None), "quantize_d4")
+        t_gemm = time_loop(hip, gemm, reps, 3)
+        t_quant = time_loop(hip, quant, reps, 3)
+        ops = 2.0 * m * rows * cols
+        out[name] = {"gemm_ms": round(t_gemm, 4), "quantize_ms": round(t_quant, 4),
+                     "tops": round(ops / (t_gemm * 1e-3) / 1e12, 2),
+                     "frac_of_int8_peak": round(ops / (t_gemm * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
+                     "tops_with_quantize": round(ops / ((t_gemm + t_quant) * 1e-3) / 1e12, 2)}
+        for b in (w, x, y, dst):
+            b.free()
+    return out
+
+
+def bench_lm_head(q8mi, hip, synth, reps=10):
+    """Fused LM head (5120 x 248320) + argmax + accept at M = 1, 2, 4, 6, 8."""
+    L, ok = q8mi.lib(), q8mi.ok
+    w = hip.to_device(synth.q8_0_weight(VOCAB, HIDDEN, seed=4242))
+    out = {}
+    for m in (1, 2, 4, 6, 8):
+        x = hip.to_device(synth.normal(m, HIDDEN, seed=m))
+        y = hip.DeviceBuffer(q81_bytes(m, HIDDEN))
+        ok(L.q8mi_quantize_q8_1(x.ptr, y.ptr, m, HIDDEN, HIDDEN, None), "quantize")
+        scratch = hip.DeviceBuffer(L.q8mi_lm_head_scratch_bytes(VOCAB, HIDDEN, m))
+        rows_out, acc = hip.DeviceBuffer(8 * m), hip.DeviceBuffer(8)
+        drafts = np.zeros(8, np.int32)
+        fn = lambda i: ok(L.q8mi_lm_head_argmax_accept(w.ptr, y.ptr, VOCAB, HIDDEN, m,
+                                                       drafts.ctypes.data_as(C.c_void_p), 0, 0, rows_out.ptr,
+                                                       acc.ptr, None, VOCAB, scratch.ptr, None), "lm_head")
+        t = time_loop(hip, fn, reps, 3)
+        nbytes = w_bytes(VOCAB, HIDDEN) + q81_bytes(m, HIDDEN) + 8 * m
+        out[f"m{m}"] = {"ms": round(t, 4), "gbps": round(nbytes / (t * 1e-3) / 1e9, 1)}
+    w.free()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
+    ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU's throughput; run with --gpus 1 "
+                 "(the path shards by weight rows, see DESIGN.md)")
+
+    import q8mi
+    from q8mi import hip, synth
+    if hip.device_count() < 1:
+        sys.exit("bench.py: no HIP device visible")
+    hip.set_device(0)
+    q8mi.lib()
+
+    layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
+    step = DecodeStep(q8mi, hip, m=1)
+    step_bytes = step.algorithmic_bytes(layers[0].bytes)
+
+    # headline: K timed steps over rotating weight copies
+    ms_stream = time_loop(hip, lambda i: step.run(layers[i % len(layers)]), args.steps, args.warmup)
+    value = step_bytes / (ms_stream * 1e-3) / 1e9
+    ms_resident = time_loop(hip, lambda i: step.run(layers[0]), args.steps, args.warmup)
+
+    # dominant kernel: the fused gate/up SwiGLU GEMV (52 % of the step's bytes)
+    n_each = min(max(args.steps, 50), 400)
+    mean_ms, med_ms, min_ms = time_each_launch(hip, lambda i: step.run_silu(layers[i % len(layers)]), n_each)
+    back_ms = time_loop(hip, lambda i: step.run_silu(layers[i % len(layers)]), n_each, 5)
+    silu_bytes = step.silu_bytes()
+    achieved = silu_bytes / (mean_ms * 1e-3) / 1e9
+    result = {
+        "metric": "Q8_0 GEMV HBM GB/s at M=1 (decode GEMV set of one 27B-style layer)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_stream, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 x int8 -> int32 dots, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "BASELINE config 1: decode GEMV set of one layer, M=1 "
+                               "(QKV 5120x8192 fan-out, O 6144x5120 +residual, gate/up 5120x17408 SwiGLU, "
+                               "down 17408x5120 +residual), Q8_0 N(0,0.02) weights, Q8_1 N(0,1) activations",
+                   "weight_copies_cycled": args.copies, "bytes_per_step": step_bytes,
+                   "launches_per_step": 8},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "resident_gbps": round(step_bytes / (ms_resident * 1e-3) / 1e9, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "gemv_kernel<1, SiluMul, x-in-LDS> (gate+up 2 x 5120x17408)",
+                     "bytes_per_launch": silu_bytes, "launch_ms_mean": round(mean_ms, 5),
+                     "launch_ms_median": round(med_ms, 5), "launch_ms_min": round(min_ms, 5),
+                     "back_to_back_ms": round(back_ms, 5), "launches_timed": n_each},
+    }
+
+    if not args.quick:
+        sweep = {}
+        for m in (1, 2, 4, 6, 8):
+            st = step if m == 1 else DecodeStep(q8mi, hip, m=m)
+            b = st.algorithmic_bytes(layers[0].bytes)
+            t = time_loop(hip, lambda i: st.run(layers[i % len(layers)]), max(args.steps // 2, 20), 5)
+            sweep[f"m{m}"] = {"ms_per_step": round(t, 5), "gbps": round(b / (t * 1e-3) / 1e9, 1)}
+        result["gemv_layer_gbps_by_m"] = sweep
+    for l in layers[1:]:
+        for b in l.w.values():
+            b.free()
+    if not args.quick:
+        result["gemm_int8_m2048"] = bench_gemm(q8mi, hip, synth)
+        result["lm_head_fused"] = bench_lm_head(q8mi, hip, synth)
+    if not (args.quick or args.no_cpu):
+        result["cpu_baseline"] = cpu_baseline()
+    else:
+        result["cpu_baseline"] = None
+    try:
+        result["device"] = hip.device_name()
+    except Exception:
+        pass
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
