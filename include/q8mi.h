@@ -170,6 +170,14 @@ int q8mi_repack_q8_0_split_host(const void *gguf_blocks, uint64_t rows, uint64_t
 int q8mi_repack_q8_0_split(const void *gguf_blocks, uint64_t rows, uint64_t cols, void *split_out,
                            void *stream);
 
+/* ---- measurement helper --------------------------------------------------- */
+/* Plain streaming read of `bytes` device bytes (16-byte loads, grid-stride,
+ * wgs_per_cu workgroups of 256 per CU): the practical HBM read ceiling that
+ * the GEMV's achieved bandwidth is compared with.  No counterpart in the
+ * reference.  sink: one device uint32 (never written in practice). */
+int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per_cu, uint32_t *sink,
+                    void *stream);
+
 /* ---- synthetic inputs (host side, for benches and tests) ----------------- */
 /* Counter-based generator: element i of stream `seed` depends only on
  * (seed, i), so any thread split gives the same bytes.

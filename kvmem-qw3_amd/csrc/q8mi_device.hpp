@@ -58,6 +58,53 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// xor-D lane exchange, D = 1, 2 by DPP, 4..16 by ds_swizzle (bit-mask mode, no
+// LDS memory touched), 32 by ds_bpermute.
+template <int D>
+__device__ __forceinline__ float lane_xor(float v) {
+    if (D == 1) return dpp_f32<kDppXor1>(v);
+    if (D == 2) return dpp_f32<kDppXor2>(v);
+    if (D == 32) {
+        const int lane = static_cast<int>(threadIdx.x) & 63;
+        return as_f32(__builtin_amdgcn_ds_bpermute(((lane ^ 32) << 2), as_i32(v)));
+    }
+    return as_f32(__builtin_amdgcn_ds_swizzle(as_i32(v), (D << 10) | 0x1f));
+}
+
+// Sums V per-lane values across the wave "transposed": on return, lane l holds
+// the wave-wide total of v[l % VP] (VP = V rounded up to a power of two).  Each
+// stage halves the number of live values by letting the two lanes of an
+// exchange pair keep one value each, so the whole reduction costs about 4*V
+// instructions instead of 12*V for V independent wave sums.  The order of the
+// additions is fixed.
+template <int VP, int D = 1>
+struct TransposeReduce {
+    static __device__ __forceinline__ float run(float (&v)[VP], uint32_t lane) {
+        if constexpr (VP == 1) {
+            float t = v[0];
+            if constexpr (D <= 1) t += lane_xor<1>(t);
+            if constexpr (D <= 2) t += lane_xor<2>(t);
+            if constexpr (D <= 4) t += lane_xor<4>(t);
+            if constexpr (D <= 8) t += lane_xor<8>(t);
+            if constexpr (D <= 16) t += lane_xor<16>(t);
+            if constexpr (D <= 32) t += lane_xor<32>(t);
+            return t;
+        } else {
+            const bool hi = lane & D;
+            float h[VP / 2];
+#pragma unroll
+            for (int i = 0; i < VP / 2; ++i) {
+                const float keep = hi ? v[2 * i + 1] : v[2 * i];
+                const float send = hi ? v[2 * i] : v[2 * i + 1];
+                h[i] = keep + lane_xor<D>(send);
+            }
+            return TransposeReduce<VP / 2, D * 2>::run(h, lane);
+        }
+    }
+};
+
+constexpr int pow2_at_least(int v) { return v <= 1 ? 1 : 2 * pow2_at_least((v + 1) / 2); }
+
 // ---- conversions ----------------------------------------------------------
 __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return static_cast<float>(__builtin_bit_cast(_Float16, h));
@@ -78,7 +125,17 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t h) {
 }
 
 // ---- int8 dot products ------------------------------------------------------
-// 16 int8 x 16 int8 -> int32, four v_dot4_i32_i8.
+// 16 int8 x 16 int8 -> int32, four v_dot4 (the first one in its three-operand
+// form with a literal zero, which saves initialising an accumulator register).
+__device__ __forceinline__ int dot16(const v4i &a, const v4i &b) {
+    int acc;
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(acc) : "v"(a.x), "v"(b.x));
+    acc = __builtin_amdgcn_sdot4(a.y, b.y, acc, false);
+    acc = __builtin_amdgcn_sdot4(a.z, b.z, acc, false);
+    acc = __builtin_amdgcn_sdot4(a.w, b.w, acc, false);
+    return acc;
+}
+
 __device__ __forceinline__ int dot16(const v4i &a, const v4i &b, int acc) {
     acc = __builtin_amdgcn_sdot4(a.x, b.x, acc, false);
     acc = __builtin_amdgcn_sdot4(a.y, b.y, acc, false);

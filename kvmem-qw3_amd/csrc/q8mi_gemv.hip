@@ -2,22 +2,14 @@
 // Reference semantics: src/mmvq_q8.cu:193-280 (plain), :295-399 (two weights),
 // :414-519 (SwiGLU), :528-606 (residual add), :976-1068 (four-weight fan-out).
 //
-// Shape of the work: the weights are read exactly once from HBM and nothing
-// else is large, so the kernel is a stream over the int8 plane of each row.
-//   * One wave owns one weight row at a time; waves stride over rows so that
-//     the waves in flight read adjacent rows (adjacent addresses).
-//   * Inside a row a lane reads 16 contiguous bytes per load, the wave 1 KiB
-//     per load (global_load_dwordx4, fully coalesced).  Two such loads ("A" and
-//     "B", 1 KiB apart) form one step; a lane therefore holds half of block
-//     A_(lane/2) and half of block B_(lane/2).  Lane pairs swap half sums with
-//     one DPP move so that the even lane ends with the full int32 dot of block
-//     A and the odd lane with that of block B: every 32-element block gets one
-//     int32 sum and one fp32 rescale, as the reference's MMQ path does.
-//   * Activations are tiny and re-used by every row: the workgroup stages them
-//     once in LDS (int8 as packed dwords + fp32 scales) when they fit, otherwise
-//     lanes read them from global memory (served by L2).
-//   * Per-lane fp32 partial sums are reduced across the wave with DPP in a
-//     fixed order, so results are deterministic run to run.
+// The weights are read exactly once from HBM and nothing else is large, so the
+// kernel is a stream over the int8 plane of each row (see q8mi_gemv_core.hpp
+// for the streaming core).  This file adds what differs between the entry
+// points: which rows form a unit, and what happens to a finished unit (store,
+// residual add, bf16 rounding, SwiGLU).  All of that is wave-uniform and runs
+// once per unit, so it is a runtime switch rather than a template parameter.
+#include <stdlib.h>
+
 #include "q8mi_gemv_core.hpp"
 
 namespace q8mi {
@@ -37,19 +29,152 @@ struct GemvParams {
     uint32_t row_end[4];  // cumulative row counts of the concatenated row space
     uint32_t stride[4];
     const uint8_t *y;     // Q8_1 blocks, [batch][nb]
-    uint32_t total_rows;
-    uint32_t cols;
+    uint32_t total_rows;  // rows of the concatenated space (SwiGLU: rows of one weight)
+    uint32_t units;
     uint32_t nb;
+    uint32_t x_bytes;     // LDS bytes of the staged activations (0 when they are read from global)
+    int mode;
+    int interleave;
+#ifdef Q8MI_TRACE
+    unsigned long long *trace;   // [grid][4] timestamps (tuning builds only)
+#endif
 };
 
-template <int MODE>
-__device__ __forceinline__ void store_out(void *dst, uint64_t idx, float v) {
-    if (MODE == kStoreF32 || MODE == kSiluMul) {
+// Which of the (up to four) concatenated weights a row belongs to.
+struct RowRef {
+    const uint8_t *w;
+    void *dst;
+    uint32_t stride;
+    uint32_t local;
+};
+
+__device__ __forceinline__ RowRef resolve_row(const GemvParams &p, uint32_t row) {
+    uint32_t seg = 0, base = 0;
+    if (row >= p.row_end[0]) { seg = 1; base = p.row_end[0]; }
+    if (row >= p.row_end[1]) { seg = 2; base = p.row_end[1]; }
+    if (row >= p.row_end[2]) { seg = 3; base = p.row_end[2]; }
+    RowRef r;
+    r.w = p.w[0]; r.dst = p.dst[0]; r.stride = p.stride[0];
+    if (seg == 1) { r.w = p.w[1]; r.dst = p.dst[1]; r.stride = p.stride[1]; }
+    if (seg == 2) { r.w = p.w[2]; r.dst = p.dst[2]; r.stride = p.stride[2]; }
+    if (seg == 3) { r.w = p.w[3]; r.dst = p.dst[3]; r.stride = p.stride[3]; }
+    r.local = row - base;
+    return r;
+}
+
+
+__device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, float v);
+
+// Each wave parks the (possibly partial) sums of the units it touched in LDS;
+// after a barrier the workgroup adds the partials of every unit in wave order and
+// writes the results out, all threads in parallel.
+//
+// Unit u covers rows R*u .. R*u+R-1 of the concatenated row space; for SwiGLU it
+// covers rows (R/2)*u .. of BOTH weights: slots 0..R/2-1 are gate rows, slots
+// R/2..R-1 the matching up rows.
+template <int M, int THREADS, int XMODE>
+__global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int R = RowsPerUnit<M>::value;
+    constexpr uint32_t kPerUnit = M * R;
+    constexpr uint32_t kWaves = THREADS / kWave;
+    const uint32_t lane = threadIdx.x % kWave;
+    // wave index as a scalar, so that row bookkeeping stays in SGPRs
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t nsteps = (p.nb * 2 + 127) / 128;
+    const uint64_t row_bytes = static_cast<uint64_t>(p.nb) * 34;
+#ifdef Q8MI_TRACE
+    const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
+#endif
+    uint32_t ufirst, ucount, ustride;
+    group_units(p.units, blockIdx.x, gridDim.x, p.interleave, ufirst, ucount, ustride);
+    const uint32_t n_items = ucount * nsteps;
+    uint32_t i0, i1;
+    wave_items(n_items, wave, kWaves, i0, i1);
+    float *park_base = reinterpret_cast<float *>(smem + p.x_bytes);   // [wave][kParkFloats]
+    float *my_park = park_base + wave * kParkFloats;
+    const uint32_t last_row = p.total_rows - 1;
+
+    auto rows_of = [&](uint32_t u, RowPtrs<R> &rp) {
+        if (p.mode == kSiluMul) {
+#pragma unroll
+            for (int r = 0; r < R / 2; ++r) {
+                uint32_t row = (R / 2) * u + r;
+                row = row < last_row ? row : last_row;   // ragged tail: re-read the last row
+                rp.p[r] = p.w[0] + row * row_bytes;
+                rp.p[R / 2 + r] = p.w[1] + row * row_bytes;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                uint32_t row = R * u + r;
+                row = row < last_row ? row : last_row;
+                const RowRef a = resolve_row(p, row);
+                rp.p[r] = a.w + a.local * row_bytes;
+            }
+        }
+    };
+    auto park = [&](uint32_t kk, float total) {
+        if (lane < kPerUnit) my_park[kk * kPerUnit + lane] = total;
+    };
+    gemv_stream<M, R, THREADS, XMODE>(smem, p.y, p.nb, ufirst, ustride, i0, i1, rows_of, park);
+#ifdef Q8MI_TRACE
+    const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
+#endif
+    __syncthreads();
+#ifdef Q8MI_TRACE
+    if (p.trace && threadIdx.x == 0) {
+        p.trace[blockIdx.x * 4 + 0] = t_begin;
+        p.trace[blockIdx.x * 4 + 1] = t_stream;
+        p.trace[blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
+    }
+#endif
+
+    // combine + write-out: entry e = (unit ordinal k, activation row m, slot r)
+    auto total_of = [&](uint32_t k, uint32_t mr) {
+        float t = 0.0f;
+        for (uint32_t w = 0; w < kWaves; ++w) {
+            uint32_t a0, a1;
+            wave_items(n_items, w, kWaves, a0, a1);
+            if (a1 <= a0) continue;
+            const uint32_t kf = a0 / nsteps, kl = (a1 - 1) / nsteps;   // units wave w touched
+            if (k >= kf && k <= kl) t += park_base[w * kParkFloats + (k - kf) * kPerUnit + mr];
+        }
+        return t;
+    };
+    if (p.mode == kSiluMul) {
+        constexpr uint32_t kHalf = R / 2;
+        for (uint32_t e = threadIdx.x; e < ucount * M * kHalf; e += THREADS) {
+            const uint32_t k = e / (M * kHalf), m = (e / kHalf) % M, r = e % kHalf;
+            const uint32_t row = kHalf * (ufirst + k * ustride) + r;
+            if (row >= p.total_rows) continue;
+            const float g = total_of(k, m * R + r);
+            const float up = total_of(k, m * R + kHalf + r);
+            const float silu = g / (1.0f + __expf(-g));
+            static_cast<float *>(p.dst[0])[static_cast<uint64_t>(m) * p.stride[0] + row] = silu * up;
+        }
+    } else {
+        for (uint32_t e = threadIdx.x; e < ucount * kPerUnit; e += THREADS) {
+            const uint32_t k = e / kPerUnit, mr = e % kPerUnit;
+            const uint32_t m = mr / R, r = mr % R;
+            const uint32_t row = R * (ufirst + k * ustride) + r;
+            if (row >= p.total_rows) continue;
+            const RowRef ref = resolve_row(p, row);
+            store_out(p.mode, ref.dst, static_cast<uint64_t>(m) * ref.stride + ref.local, total_of(k, mr));
+        }
+    }
+#ifdef Q8MI_TRACE
+    if (p.trace && threadIdx.x == 0) p.trace[blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
+#endif
+}
+
+__device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, float v) {
+    if (mode == kStoreF32) {
         static_cast<float *>(dst)[idx] = v;
-    } else if (MODE == kAddF32) {
+    } else if (mode == kAddF32) {
         float *p = static_cast<float *>(dst) + idx;
         *p = *p + v;
-    } else if (MODE == kStoreBF16) {
+    } else if (mode == kStoreBF16) {
         static_cast<uint16_t *>(dst)[idx] = float_to_bf16_bits(v);
     } else {
         uint16_t *p = static_cast<uint16_t *>(dst) + idx;
@@ -57,82 +182,23 @@ __device__ __forceinline__ void store_out(void *dst, uint64_t idx, float v) {
     }
 }
 
-template <int M, int MODE, bool XLDS>
-__global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvParams p) {
-    extern __shared__ __align__(16) uint8_t smem[];
-    const uint32_t nb = p.nb;
-    const uint32_t nsteps = (nb * 2 + 127) / 128;
-    const int *lds_q = reinterpret_cast<const int *>(smem);
-    const float *lds_d = reinterpret_cast<const float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
-
-    if (XLDS) stage_x_lds<M>(smem, p.y, nb);
-
-    const uint32_t lane = threadIdx.x % kWave;
-    const uint32_t wave = blockIdx.x * kGemvWaves + threadIdx.x / kWave;
-    const uint32_t nwaves = gridDim.x * kGemvWaves;
-    const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
-
-    for (uint32_t row = wave; row < p.total_rows; row += nwaves) {
-        if (MODE == kSiluMul) {
-            float g[M], u[M];
-            row_partial<M, XLDS>(p.w[0] + row * row_bytes, p.y, lds_q, lds_d, nb, lane, g);
-            row_partial<M, XLDS>(p.w[1] + row * row_bytes, p.y, lds_q, lds_d, nb, lane, u);
-#pragma unroll
-            for (int m = 0; m < M; ++m) {
-                const float gs = wave_sum(g[m]);
-                const float us = wave_sum(u[m]);
-                if (lane == 0) {
-                    const float silu = gs / (1.0f + __expf(-gs));
-                    static_cast<float *>(p.dst[0])[static_cast<uint64_t>(m) * p.stride[0] + row] = silu * us;
-                }
-            }
-        } else {
-            // which of the (up to four) concatenated weights this row belongs to
-            uint32_t seg = 0, base = 0;
-            if (row >= p.row_end[0]) { seg = 1; base = p.row_end[0]; }
-            if (row >= p.row_end[1]) { seg = 2; base = p.row_end[1]; }
-            if (row >= p.row_end[2]) { seg = 3; base = p.row_end[2]; }
-            const uint32_t local = row - base;
-            const uint8_t *wbase = p.w[0];
-            void *dst = p.dst[0];
-            uint32_t stride = p.stride[0];
-            if (seg == 1) { wbase = p.w[1]; dst = p.dst[1]; stride = p.stride[1]; }
-            if (seg == 2) { wbase = p.w[2]; dst = p.dst[2]; stride = p.stride[2]; }
-            if (seg == 3) { wbase = p.w[3]; dst = p.dst[3]; stride = p.stride[3]; }
-            float acc[M];
-            row_partial<M, XLDS>(wbase + local * row_bytes, p.y, lds_q, lds_d, nb, lane, acc);
-#pragma unroll
-            for (int m = 0; m < M; ++m) {
-                const float s = wave_sum(acc[m]);
-                if (lane == 0) store_out<MODE>(dst, static_cast<uint64_t>(m) * stride + local, s);
-            }
-        }
-    }
-}
-
 // Fallback for rows whose planes are not 16-byte aligned (cols/32 not a
 // multiple of 8): one lane per 32-element block, 2-byte weight loads.
-template <int MODE>
-__global__ __launch_bounds__(kGemvThreads) void gemv_unaligned_kernel(const GemvParams p, uint32_t batch) {
+__global__ __launch_bounds__(256) void gemv_unaligned_kernel(const GemvParams p, uint32_t batch) {
     const uint32_t nb = p.nb;
     const uint32_t lane = threadIdx.x % kWave;
-    const uint32_t wave = blockIdx.x * kGemvWaves + threadIdx.x / kWave;
-    const uint32_t nwaves = gridDim.x * kGemvWaves;
+    const uint32_t wave = blockIdx.x * 4 + threadIdx.x / kWave;
+    const uint32_t nwaves = gridDim.x * 4;
     const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
-    const uint32_t nw = (MODE == kSiluMul) ? 2 : 1;
+    const uint32_t nw = (p.mode == kSiluMul) ? 2 : 1;
 
     for (uint32_t row = wave; row < p.total_rows; row += nwaves) {
-        uint32_t seg = 0, base = 0;
-        if (MODE != kSiluMul) {
-            if (row >= p.row_end[0]) { seg = 1; base = p.row_end[0]; }
-            if (row >= p.row_end[1]) { seg = 2; base = p.row_end[1]; }
-            if (row >= p.row_end[2]) { seg = 3; base = p.row_end[2]; }
-        }
-        const uint32_t local = row - base;
+        const RowRef ref = resolve_row(p, p.mode == kSiluMul ? 0 : row);
+        const uint32_t local = p.mode == kSiluMul ? row : ref.local;
         for (uint32_t j = 0; j < batch; ++j) {
             float res[2] = {0.0f, 0.0f};
             for (uint32_t wi = 0; wi < nw; ++wi) {
-                const uint8_t *row_w = p.w[MODE == kSiluMul ? wi : seg] + local * row_bytes;
+                const uint8_t *row_w = (p.mode == kSiluMul ? p.w[wi] : ref.w) + local * row_bytes;
                 const uint16_t *scales = reinterpret_cast<const uint16_t *>(row_w);
                 const uint16_t *quants = reinterpret_cast<const uint16_t *>(row_w + 2 * nb);
                 float acc = 0.0f;
@@ -153,58 +219,86 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_unaligned_kernel(const Gemv
                 res[wi] = wave_sum(acc);
             }
             if (lane == 0) {
-                if (MODE == kSiluMul) {
+                if (p.mode == kSiluMul) {
                     const float silu = res[0] / (1.0f + __expf(-res[0]));
                     static_cast<float *>(p.dst[0])[static_cast<uint64_t>(j) * p.stride[0] + row] = silu * res[1];
                 } else {
-                    store_out<MODE>(p.dst[seg], static_cast<uint64_t>(j) * p.stride[seg] + local, res[0]);
+                    store_out(p.mode, ref.dst, static_cast<uint64_t>(j) * ref.stride + local, res[0]);
                 }
             }
         }
     }
 }
 
-template <int M, int MODE>
-int launch_m(const GemvParams &p, hipStream_t stream) {
-    const int cus = device_cu_count();
-    const uint32_t lds = x_lds_bytes(p.nb, M);
-    const uint32_t rows_per_wg_pass = kGemvWaves;
-    uint32_t max_wgs = (p.total_rows + rows_per_wg_pass - 1) / rows_per_wg_pass;
-    if (lds <= kMaxXLdsBytes) {
-        // persistent-style grid: a few workgroups per CU, each stages x once
-        uint32_t per_cu = 160u * 1024u / (lds + 1024u);
-        if (per_cu > 4) per_cu = 4;
-        if (per_cu < 1) per_cu = 1;
-        uint32_t grid = static_cast<uint32_t>(cus) * per_cu;
-        if (grid > max_wgs) grid = max_wgs;
-        gemv_kernel<M, MODE, true><<<grid, kGemvThreads, lds, stream>>>(p);
-    } else {
-        uint32_t grid = static_cast<uint32_t>(cus) * 4;
-        if (grid > max_wgs) grid = max_wgs;
-        gemv_kernel<M, MODE, false><<<grid, kGemvThreads, 0, stream>>>(p);
+// One launch of a given instantiation: geometry is cached per (instantiation, LDS size).
+template <int M, int THREADS, int XMODE>
+int launch_inst(GemvParams p, uint32_t x_bytes, hipStream_t stream) {
+    auto kern = gemv_kernel<M, THREADS, XMODE>;
+    constexpr uint32_t R = RowsPerUnit<M>::value;
+    p.x_bytes = x_bytes;
+    p.units = p.mode == kSiluMul ? (p.total_rows + R / 2 - 1) / (R / 2) : (p.total_rows + R - 1) / R;
+    const uint32_t lds = x_bytes + (THREADS / kWave) * kParkFloats * 4;
+    static thread_local uint32_t cached_lds = 0xffffffffu;
+    static thread_local int cached_occ = 0;
+    if (cached_lds != lds) {
+        if (lds > 64u * 1024u &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds)) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
+        }
+        int occ = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, THREADS, lds) != hipSuccess || occ < 1) {
+            (void)hipGetLastError();
+            occ = 1;
+        }
+        cached_occ = occ;
+        cached_lds = lds;
     }
+    const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+    const GemvTuning tune = gemv_tuning();
+    uint32_t per_cu = static_cast<uint32_t>(cached_occ);
+    if (tune.wgs_per_cu > 0 && static_cast<uint32_t>(tune.wgs_per_cu) < per_cu) per_cu = tune.wgs_per_cu;
+    p.interleave = tune.interleave;
+#ifdef Q8MI_TRACE
+    p.trace = nullptr;
+    if (const char *e = getenv("Q8MI_TRACE_PTR")) p.trace = reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 0));
+#endif
+    const uint32_t grid = pick_grid(p.units, (p.nb * 2 + 127) / 128, M, THREADS / kWave, cus, per_cu);
+    kern<<<grid, THREADS, lds, stream>>>(p);
     return check_launch("gemv");
 }
 
-template <int MODE>
-int launch_mode(const GemvParams &p, uint32_t batch, hipStream_t stream) {
+template <int M>
+int launch_m(const GemvParams &p, hipStream_t stream) {
+    const uint32_t xb = x_lds_bytes(p.nb, M);
+    const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
+    const int forced = gemv_tuning().threads;
+    if (forced == 256 && xb + park_256 <= kLdsLimit) return launch_inst<M, 256, kXLds>(p, xb, stream);
+    if (forced == 1024 && xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds>(p, xb, stream);
+    if (xb + park_256 <= 76u * 1024u) return launch_inst<M, 256, kXLds>(p, xb, stream);   // two per CU fit
+    if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds>(p, xb, stream);
+    return launch_inst<M, 256, kXGlobal>(p, 0, stream);
+}
+
+int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
     if (p.nb % 8 != 0) {
-        const int cus = device_cu_count();
-        uint32_t grid = static_cast<uint32_t>(cus) * 8;
-        const uint32_t max_wgs = (p.total_rows + kGemvWaves - 1) / kGemvWaves;
+        const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+        uint32_t grid = cus * 8;
+        const uint32_t max_wgs = (p.total_rows + 3) / 4;
         if (grid > max_wgs) grid = max_wgs;
-        gemv_unaligned_kernel<MODE><<<grid, kGemvThreads, 0, stream>>>(p, batch);
+        gemv_unaligned_kernel<<<grid, 256, 0, stream>>>(p, batch);
         return check_launch("gemv_unaligned");
     }
     switch (batch) {
-        case 1: return launch_m<1, MODE>(p, stream);
-        case 2: return launch_m<2, MODE>(p, stream);
-        case 3: return launch_m<3, MODE>(p, stream);
-        case 4: return launch_m<4, MODE>(p, stream);
-        case 5: return launch_m<5, MODE>(p, stream);
-        case 6: return launch_m<6, MODE>(p, stream);
-        case 7: return launch_m<7, MODE>(p, stream);
-        case 8: return launch_m<8, MODE>(p, stream);
+        case 1: return launch_m<1>(p, stream);
+        case 2: return launch_m<2>(p, stream);
+        case 3: return launch_m<3>(p, stream);
+        case 4: return launch_m<4>(p, stream);
+        case 5: return launch_m<5>(p, stream);
+        case 6: return launch_m<6>(p, stream);
+        case 7: return launch_m<7>(p, stream);
+        case 8: return launch_m<8>(p, stream);
         default: return Q8MI_REJECTED;
     }
 }
@@ -219,7 +313,7 @@ int shape_gate(const char *what, uint32_t cols, uint32_t batch) {
 bool planes_aligned(const void *w) { return reinterpret_cast<uintptr_t>(w) % 16 == 0; }
 
 GemvParams single(const uint8_t *w, const void *y, void *dst, uint32_t rows, uint32_t cols,
-                  uint32_t stride) {
+                  uint32_t stride, int mode) {
     GemvParams p{};
     p.w[0] = w;
     p.dst[0] = dst;
@@ -227,22 +321,35 @@ GemvParams single(const uint8_t *w, const void *y, void *dst, uint32_t rows, uin
     for (int i = 0; i < 4; ++i) p.row_end[i] = rows;
     p.y = static_cast<const uint8_t *>(y);
     p.total_rows = rows;
-    p.cols = cols;
+    p.units = 0;   // set per batch size at launch
     p.nb = cols / kQK;
+    p.mode = mode;
     return p;
 }
 
-template <int MODE>
-int run_single(const char *what, const uint8_t *w, const void *y, void *dst, uint32_t rows,
+int run_single(const char *what, int mode, const uint8_t *w, const void *y, void *dst, uint32_t rows,
                uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
     if (int rc = shape_gate(what, cols, batch)) return rc;
     if (rows == 0 || cols == 0) return Q8MI_OK;
     if (!planes_aligned(w)) return fail(Q8MI_REJECTED, "%s: weight pointer not 16-byte aligned", what);
-    const GemvParams p = single(w, y, dst, rows, cols, stride);
-    return launch_mode<MODE>(p, batch, as_stream(stream));
+    const GemvParams p = single(w, y, dst, rows, cols, stride, mode);
+    return launch_any(p, batch, as_stream(stream));
 }
 
 }  // namespace
+
+GemvTuning gemv_tuning() {
+    static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
+    auto read = [] {
+        GemvTuning t{2, 1, 0};   // two workgroups per CU, interleaved units: best of the sweeps
+        if (const char *e = getenv("Q8MI_GEMV_WGS_PER_CU")) t.wgs_per_cu = atoi(e);
+        if (const char *e = getenv("Q8MI_GEMV_INTERLEAVE")) t.interleave = atoi(e);
+        if (const char *e = getenv("Q8MI_GEMV_THREADS")) t.threads = atoi(e);
+        return t;
+    };
+    static const GemvTuning fixed = read();
+    return live ? read() : fixed;
+}
 
 // Any batch through the GEMV kernels, eight activation rows per launch.  Used by
 // the GEMM entry point for shapes its MFMA tile does not cover.
@@ -254,8 +361,8 @@ int gemv_any_batch(const uint8_t *w, const void *y_q8_1, float *dst, uint32_t ro
         const uint32_t m = batch - j0 < Q8MI_MAX_GEMV_BATCH ? batch - j0 : Q8MI_MAX_GEMV_BATCH;
         const GemvParams p = single(w, y + static_cast<uint64_t>(j0) * nb * kQ81Bytes,
                                     dst + static_cast<uint64_t>(j0) * stride_dst_row, rows, cols,
-                                    stride_dst_row);
-        if (int rc = launch_mode<kStoreF32>(p, m, stream)) return rc;
+                                    stride_dst_row, kStoreF32);
+        if (int rc = launch_any(p, m, stream)) return rc;
     }
     return Q8MI_OK;
 }
@@ -266,22 +373,22 @@ using namespace q8mi;
 
 extern "C" int q8mi_gemv(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,
                          uint32_t batch, uint32_t stride, void *stream) {
-    return run_single<kStoreF32>("gemv", w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv", kStoreF32, w, y, dst, rows, cols, batch, stride, stream);
 }
 
 extern "C" int q8mi_gemv_bf16(const uint8_t *w, const void *y, uint16_t *dst, uint32_t rows,
                               uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
-    return run_single<kStoreBF16>("gemv_bf16", w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv_bf16", kStoreBF16, w, y, dst, rows, cols, batch, stride, stream);
 }
 
 extern "C" int q8mi_gemv_add(const uint8_t *w, const void *y, float *dst, uint32_t rows,
                              uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
-    return run_single<kAddF32>("gemv_add", w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv_add", kAddF32, w, y, dst, rows, cols, batch, stride, stream);
 }
 
 extern "C" int q8mi_gemv_add_bf16(const uint8_t *w, const void *y, uint16_t *dst, uint32_t rows,
                                   uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
-    return run_single<kAddBF16>("gemv_add_bf16", w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv_add_bf16", kAddBF16, w, y, dst, rows, cols, batch, stride, stream);
 }
 
 extern "C" int q8mi_gemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const void *y, float *dst,
@@ -291,9 +398,9 @@ extern "C" int q8mi_gemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const vo
     if (rows == 0 || cols == 0) return Q8MI_OK;
     if (!planes_aligned(wg) || !planes_aligned(wu))
         return fail(Q8MI_REJECTED, "gemv_silu_mul: weight pointer not 16-byte aligned");
-    GemvParams p = single(wg, y, dst, rows, cols, stride);
+    GemvParams p = single(wg, y, dst, rows, cols, stride, kSiluMul);
     p.w[1] = wu;
-    return launch_mode<kSiluMul>(p, batch, as_stream(stream));
+    return launch_any(p, batch, as_stream(stream));
 }
 
 extern "C" int q8mi_gemv_fanout4(const uint8_t *w0, const uint8_t *w1, const uint8_t *w2,
@@ -325,12 +432,18 @@ extern "C" int q8mi_gemv_fanout4(const uint8_t *w0, const uint8_t *w1, const uin
         ++n;
     }
     if (n == 0 || cols == 0) return Q8MI_OK;
-    for (uint32_t i = n; i < 4; ++i) p.row_end[i] = total;
+    for (uint32_t i = n; i < 4; ++i) {
+        p.row_end[i] = total;
+        p.w[i] = p.w[n - 1];   // never dereferenced for a row, kept valid for safety
+        p.dst[i] = p.dst[n - 1];
+        p.stride[i] = p.stride[n - 1];
+    }
     p.y = static_cast<const uint8_t *>(y);
     p.total_rows = total;
-    p.cols = cols;
+    p.units = 0;
     p.nb = cols / kQK;
-    return launch_mode<kStoreF32>(p, batch, as_stream(stream));
+    p.mode = kStoreF32;
+    return launch_any(p, batch, as_stream(stream));
 }
 
 extern "C" int q8mi_gemv_two(const uint8_t *w0, const uint8_t *w1, const void *y, float *dst0,

@@ -92,6 +92,29 @@ __global__ __launch_bounds__(256) void block_dots_kernel(const uint8_t *__restri
     out[i] = s;
 }
 
+// ---- measurement helper: plain streaming read ---------------------------------
+// Every lane reads 16 bytes per trip, the grid covers the buffer with a
+// grid-stride loop; the xor of everything read goes to sink[0] only if it is a
+// value that cannot occur, so the loads cannot be optimised away.
+__global__ __launch_bounds__(256) void probe_read_kernel(const v4i *__restrict__ p, uint64_t n16,
+                                                         uint32_t *__restrict__ sink) {
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256;
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    v4i a = {0, 0, 0, 0};
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const v4i v0 = p[i], v1 = p[i + stride], v2 = p[i + 2 * stride], v3 = p[i + 3 * stride];
+        a.x ^= v0.x ^ v1.x ^ v2.x ^ v3.x;
+        a.y ^= v0.y ^ v1.y ^ v2.y ^ v3.y;
+        a.z ^= v0.z ^ v1.z ^ v2.z ^ v3.z;
+        a.w ^= v0.w ^ v1.w ^ v2.w ^ v3.w;
+    }
+    for (; i < n16; i += stride) {
+        const v4i v = p[i];
+        a.x ^= v.x; a.y ^= v.y; a.z ^= v.z; a.w ^= v.w;
+    }
+    if ((a.x ^ a.y ^ a.z ^ a.w) == 0x5a17c0de && (a.x & a.y) == 0x0badf00d) sink[0] = 1;
+}
+
 // ---- synthetic inputs --------------------------------------------------------
 inline uint64_t splitmix64(uint64_t z) {
     z += 0x9E3779B97F4A7C15ull;
@@ -188,6 +211,16 @@ extern "C" int q8mi_block_dots(const uint8_t *weight, const void *y, int y_layou
         weight, static_cast<const uint8_t *>(y), y_layout, cols / kQK, batch, sample_row, sample_j,
         sample_kb, n, out);
     return check_launch("block_dots");
+}
+
+extern "C" int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per_cu, uint32_t *sink,
+                               void *stream) {
+    if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(buf) % 16 != 0)
+        return fail(Q8MI_REJECTED, "probe_read: buffer must be 16-byte aligned and sized");
+    if (wgs_per_cu == 0 || wgs_per_cu > 64) return fail(Q8MI_REJECTED, "probe_read: wgs_per_cu outside 1..64");
+    const uint32_t grid = static_cast<uint32_t>(device_cu_count()) * wgs_per_cu;
+    probe_read_kernel<<<grid, 256, 0, as_stream(stream)>>>(static_cast<const v4i *>(buf), bytes / 16, sink);
+    return check_launch("probe_read");
 }
 
 extern "C" int q8mi_synth_f32(float *out, uint64_t rows, uint64_t cols, uint64_t seed, int kind,

@@ -33,58 +33,86 @@ __device__ __forceinline__ bool beats(float ov, int oi, float v, int i) {
     return ov == v && oi < i;
 }
 
-template <int M, bool XLDS>
-__global__ __launch_bounds__(kGemvThreads) void lm_head_kernel(
+template <int M, int THREADS, int XMODE>
+__global__ __launch_bounds__(THREADS) void lm_head_kernel(
         const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, uint32_t rows, uint32_t nb,
-        q8mi_argmax_pair *__restrict__ partial, float *__restrict__ logits, uint32_t stride_logits) {
+        q8mi_argmax_pair *__restrict__ partial, float *__restrict__ logits, uint32_t stride_logits,
+        int interleave, uint32_t x_bytes) {
     extern __shared__ __align__(16) uint8_t smem[];
-    const uint32_t nsteps = (nb * 2 + 127) / 128;
-    const int *lds_q = reinterpret_cast<const int *>(smem);
-    const float *lds_d = reinterpret_cast<const float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
-    if (XLDS) stage_x_lds<M>(smem, y, nb);
-
+    constexpr int R = RowsPerUnit<M>::value;
+    constexpr uint32_t kPerUnit = M * R;
+    constexpr uint32_t kWaves = THREADS / kWave;
     const uint32_t lane = threadIdx.x % kWave;
-    const uint32_t wave_in_wg = threadIdx.x / kWave;
-    const uint32_t wave = blockIdx.x * kGemvWaves + wave_in_wg;
-    const uint32_t nwaves = gridDim.x * kGemvWaves;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t nsteps = (nb * 2 + 127) / 128;
     const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    const uint32_t units = (rows + R - 1) / R;
+    uint32_t ufirst, ucount, ustride;
+    group_units(units, blockIdx.x, gridDim.x, interleave, ufirst, ucount, ustride);
+    const uint32_t n_items = ucount * nsteps;
+    uint32_t i0, i1;
+    wave_items(n_items, wave, kWaves, i0, i1);
+    float *park_base = reinterpret_cast<float *>(smem + x_bytes);
+    float *my_park = park_base + wave * kParkFloats;
 
-    float best_v[M];
-    int best_i[M];
+    auto rows_of = [&](uint32_t u, RowPtrs<R> &rp) {
 #pragma unroll
-    for (int m = 0; m < M; ++m) { best_v[m] = -INFINITY; best_i[m] = -1; }
-
-    for (uint32_t row = wave; row < rows; row += nwaves) {
-        float acc[M];
-        row_partial<M, XLDS>(w + row * row_bytes, y, lds_q, lds_d, nb, lane, acc);
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-            const float s = wave_sum(acc[m]);  // identical in every lane
-            if (beats(s, static_cast<int>(row), best_v[m], best_i[m])) {
-                best_v[m] = s;
-                best_i[m] = static_cast<int>(row);
-            }
-            if (logits != nullptr && lane == 0) logits[static_cast<uint64_t>(m) * stride_logits + row] = s;
+        for (int r = 0; r < R; ++r) {
+            uint32_t row = R * u + r;
+            row = row < rows - 1 ? row : rows - 1;   // ragged tail: re-read the last row
+            rp.p[r] = w + row * row_bytes;
         }
-    }
-
-    __shared__ float wv[kGemvWaves][Q8MI_MAX_GEMV_BATCH];
-    __shared__ int wi[kGemvWaves][Q8MI_MAX_GEMV_BATCH];
-    if (lane == 0) {
-#pragma unroll
-        for (int m = 0; m < M; ++m) { wv[wave_in_wg][m] = best_v[m]; wi[wave_in_wg][m] = best_i[m]; }
-    }
+    };
+    auto park = [&](uint32_t kk, float total) {
+        if (lane < kPerUnit) my_park[kk * kPerUnit + lane] = total;
+    };
+    gemv_stream<M, R, THREADS, XMODE>(smem, y, nb, ufirst, ustride, i0, i1, rows_of, park);
     __syncthreads();
-    if (threadIdx.x < M) {
-        const int m = threadIdx.x;
-        float v = wv[0][m];
-        int i = wi[0][m];
-        for (int k = 1; k < kGemvWaves; ++k) {
-            if (beats(wv[k][m], wi[k][m], v, i)) { v = wv[k][m]; i = wi[k][m]; }
+
+    auto total_of = [&](uint32_t k, uint32_t mr) {
+        float t = 0.0f;
+        for (uint32_t wv = 0; wv < kWaves; ++wv) {
+            uint32_t a0, a1;
+            wave_items(n_items, wv, kWaves, a0, a1);
+            if (a1 <= a0) continue;
+            const uint32_t kf = a0 / nsteps, kl = (a1 - 1) / nsteps;
+            if (k >= kf && k <= kl) t += park_base[wv * kParkFloats + (k - kf) * kPerUnit + mr];
         }
-        q8mi_argmax_pair *p = partial + static_cast<uint64_t>(m) * gridDim.x + blockIdx.x;
-        p->value = v;
-        p->index = i;
+        return t;
+    };
+
+    // per verify row: every thread scans its share of the workgroup's logits (rows in
+    // ascending order), then an LDS tree picks the workgroup's winner
+    __shared__ float sv[THREADS];
+    __shared__ int si[THREADS];
+    for (uint32_t m = 0; m < M; ++m) {
+        float bv = -INFINITY;
+        int bi = -1;
+        for (uint32_t e = threadIdx.x; e < ucount * R; e += THREADS) {
+            const uint32_t k = e / R, r = e % R;
+            const uint32_t row = R * (ufirst + k * ustride) + r;
+            if (row >= rows) continue;
+            const float s = total_of(k, m * R + r);
+            if (beats(s, static_cast<int>(row), bv, bi)) { bv = s; bi = static_cast<int>(row); }
+            if (logits != nullptr) logits[static_cast<uint64_t>(m) * stride_logits + row] = s;
+        }
+        sv[threadIdx.x] = bv;
+        si[threadIdx.x] = bi;
+        __syncthreads();
+        for (uint32_t stride = THREADS / 2; stride > 0; stride >>= 1) {
+            if (threadIdx.x < stride) {
+                const float ov = sv[threadIdx.x + stride];
+                const int oi = si[threadIdx.x + stride];
+                if (beats(ov, oi, sv[threadIdx.x], si[threadIdx.x])) { sv[threadIdx.x] = ov; si[threadIdx.x] = oi; }
+            }
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            q8mi_argmax_pair *p = partial + static_cast<uint64_t>(m) * gridDim.x + blockIdx.x;
+            p->value = sv[0];
+            p->index = si[0];
+        }
+        __syncthreads();
     }
 }
 
@@ -137,33 +165,60 @@ __global__ __launch_bounds__(kMaxPartials) void lm_head_finalize_kernel(
     }
 }
 
-uint32_t lm_head_grid(uint32_t rows, uint32_t nb, uint32_t batch) {
-    const int cus = device_cu_count();
-    const uint32_t lds = x_lds_bytes(nb, batch);
-    uint32_t per_cu = 4;
-    if (lds <= kMaxXLdsBytes) {
-        per_cu = 160u * 1024u / (lds + 1024u);
-        if (per_cu > 4) per_cu = 4;
-        if (per_cu < 1) per_cu = 1;
+template <int M, int THREADS, int XMODE>
+int launch_inst(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t nb, uint32_t x_bytes,
+                q8mi_argmax_pair *partial, float *logits, uint32_t stride_logits, uint32_t *grid_out,
+                hipStream_t stream) {
+    auto kern = lm_head_kernel<M, THREADS, XMODE>;
+    const uint32_t lds = x_bytes + (THREADS / kWave) * kParkFloats * 4;
+    static thread_local uint32_t cached_lds = 0xffffffffu;
+    static thread_local int cached_occ = 0;
+    if (cached_lds != lds) {
+        if (lds > 64u * 1024u &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(lds)) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "lm_head: cannot reserve %u bytes of LDS", lds);
+        }
+        int occ = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, THREADS, lds) != hipSuccess || occ < 1) {
+            (void)hipGetLastError();
+            occ = 1;
+        }
+        cached_occ = occ;
+        cached_lds = lds;
     }
-    uint32_t grid = static_cast<uint32_t>(cus) * per_cu;
-    const uint32_t max_wgs = (rows + kGemvWaves - 1) / kGemvWaves;
-    if (grid > max_wgs) grid = max_wgs;
-    if (grid > kMaxPartials) grid = kMaxPartials;
-    if (grid == 0) grid = 1;
-    return grid;
+    const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+    const uint32_t units = (rows + RowsPerUnit<M>::value - 1) / RowsPerUnit<M>::value;
+    const GemvTuning tune = gemv_tuning();
+    uint32_t max_per_cu = static_cast<uint32_t>(cached_occ);
+    if (tune.wgs_per_cu > 0 && static_cast<uint32_t>(tune.wgs_per_cu) < max_per_cu) max_per_cu = tune.wgs_per_cu;
+    while (max_per_cu > 1 && cus * max_per_cu > kMaxPartials) --max_per_cu;   // one partial per workgroup
+    const uint32_t grid = pick_grid(units, (nb * 2 + 127) / 128, M, THREADS / kWave, cus, max_per_cu);
+    if (grid > kMaxPartials)
+        return fail(Q8MI_REJECTED, "lm_head: %u rows need %u workgroups, more than the %u partials", rows, grid,
+                    kMaxPartials);
+    *grid_out = grid;
+    kern<<<grid, THREADS, lds, stream>>>(w, y, rows, nb, partial, logits, stride_logits, tune.interleave, x_bytes);
+    return check_launch("lm_head");
 }
 
 template <int M>
-int launch_lm_head(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t nb, uint32_t grid,
-                   q8mi_argmax_pair *partial, float *logits, uint32_t stride_logits, hipStream_t stream) {
-    const uint32_t lds = x_lds_bytes(nb, M);
-    if (lds <= kMaxXLdsBytes) {
-        lm_head_kernel<M, true><<<grid, kGemvThreads, lds, stream>>>(w, y, rows, nb, partial, logits, stride_logits);
-    } else {
-        lm_head_kernel<M, false><<<grid, kGemvThreads, 0, stream>>>(w, y, rows, nb, partial, logits, stride_logits);
-    }
-    return check_launch("lm_head");
+int launch_lm_head(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t nb, q8mi_argmax_pair *partial,
+                   float *logits, uint32_t stride_logits, uint32_t *grid_out, hipStream_t stream) {
+    const uint32_t xb = x_lds_bytes(nb, M);
+    const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
+    const uint32_t tree_256 = 256 * 8, tree_1024 = 1024 * 8;   // static LDS of the argmax tree
+    const int forced = gemv_tuning().threads;
+    if (forced == 256 && xb + park_256 + tree_256 <= kLdsLimit)
+        return launch_inst<M, 256, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
+    if (forced == 1024 && xb + park_1024 + tree_1024 <= kLdsLimit)
+        return launch_inst<M, 1024, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
+    if (xb + park_256 + tree_256 <= 76u * 1024u)
+        return launch_inst<M, 256, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
+    if (xb + park_1024 + tree_1024 <= kLdsLimit)
+        return launch_inst<M, 1024, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
+    return launch_inst<M, 256, kXGlobal>(w, y, rows, nb, 0, partial, logits, stride_logits, grid_out, stream);
 }
 
 }  // namespace
@@ -194,20 +249,20 @@ extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, 
     if (reinterpret_cast<uintptr_t>(weight) % 16 != 0)
         return fail(Q8MI_REJECTED, "lm_head: weight pointer not 16-byte aligned");
     const uint32_t nb = cols / kQK;
-    const uint32_t grid = lm_head_grid(rows, nb, batch);
+    uint32_t grid = 0;
     auto *partial = static_cast<q8mi_argmax_pair *>(scratch);
     const auto *yb = static_cast<const uint8_t *>(y);
     hipStream_t s = as_stream(stream);
     int rc = Q8MI_REJECTED;
     switch (batch) {
-        case 1: rc = launch_lm_head<1>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
-        case 2: rc = launch_lm_head<2>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
-        case 3: rc = launch_lm_head<3>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
-        case 4: rc = launch_lm_head<4>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
-        case 5: rc = launch_lm_head<5>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
-        case 6: rc = launch_lm_head<6>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
-        case 7: rc = launch_lm_head<7>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
-        case 8: rc = launch_lm_head<8>(weight, yb, rows, nb, grid, partial, logits, stride_logits, s); break;
+        case 1: rc = launch_lm_head<1>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
+        case 2: rc = launch_lm_head<2>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
+        case 3: rc = launch_lm_head<3>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
+        case 4: rc = launch_lm_head<4>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
+        case 5: rc = launch_lm_head<5>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
+        case 6: rc = launch_lm_head<6>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
+        case 7: rc = launch_lm_head<7>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
+        case 8: rc = launch_lm_head<8>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
         default: break;
     }
     if (rc != Q8MI_OK) return rc;

@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG_DIR, "libq8mi.so")
+# Q8MI_LIB points at another build of the same library (tuning variants)
+LIB_PATH = os.environ.get("Q8MI_LIB") or os.path.join(PKG_DIR, "libq8mi.so")
 
 OK, REJECTED, LAUNCH_ERROR = 0, 1, 2
 QK = 32
@@ -55,6 +56,7 @@ SIGNATURES = {
                                           _u32, _vp, _vp]),
     "q8mi_repack_q8_0_split_host": (_int, [_vp, _u64, _u64, _vp]),
     "q8mi_repack_q8_0_split": (_int, [_vp, _u64, _u64, _vp, _vp]),
+    "q8mi_probe_read": (_int, [_vp, _u64, _u32, _vp, _vp]),
     "q8mi_synth_f32": (_int, [_vp, _u64, _u64, _u64, _int, C.c_float, _u32, C.c_float, _int]),
     "q8mi_synth_q8_0_weight": (_int, [_vp, _u64, _u64, _u64, C.c_float, _int]),
 }
