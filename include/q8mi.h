@@ -112,6 +112,10 @@ int q8mi_gemm(const uint8_t *weight, const void *y, float *dst, uint32_t rows, u
 int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *dst, uint32_t rows,
                      uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
 
+/* replaces fp32_to_bf16_kernel as used by convert_q8_output_bf16,
+ * src/kernels_cuda.cu:14523-14530: out[i] = bf16(in[i]), round to nearest even. */
+int q8mi_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, void *stream);
+
 /* Checker hook (no counterpart in the reference): writes the int32 block dots
  * S[row][j][kb] = sum_t q_w*q_x for n sampled (row, j, kb) triples, computed on
  * the GPU with the same int8 dot instruction the kernels use.  y_layout:

@@ -92,6 +92,13 @@ __global__ __launch_bounds__(256) void block_dots_kernel(const uint8_t *__restri
     out[i] = s;
 }
 
+// ---- fp32 -> bf16 (round to nearest even), for bf16 activations downstream ----
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float *__restrict__ in,
+                                                          uint16_t *__restrict__ out, uint64_t n) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) out[i] = float_to_bf16_bits(in[i]);
+}
+
 // ---- measurement helper: plain streaming read ---------------------------------
 // Every lane reads 16 bytes per trip, the grid covers the buffer with a
 // grid-stride loop; the xor of everything read goes to sink[0] only if it is a
@@ -211,6 +218,14 @@ extern "C" int q8mi_block_dots(const uint8_t *weight, const void *y, int y_layou
         weight, static_cast<const uint8_t *>(y), y_layout, cols / kQK, batch, sample_row, sample_j,
         sample_kb, n, out);
     return check_launch("block_dots");
+}
+
+extern "C" int q8mi_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, void *stream) {
+    if (n == 0) return Q8MI_OK;
+    const uint64_t grid = (n + 255) / 256;
+    if (grid > 0x7fffffffull) return fail(Q8MI_REJECTED, "f32_to_bf16: too many elements for one launch");
+    f32_to_bf16_kernel<<<static_cast<uint32_t>(grid), 256, 0, as_stream(stream)>>>(in, out, n);
+    return check_launch("f32_to_bf16");
 }
 
 extern "C" int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per_cu, uint32_t *sink,

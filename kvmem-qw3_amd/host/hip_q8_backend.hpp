@@ -1,0 +1,157 @@
+// HipQ8Backend: the Q8_0 linear + argmax slice of qw3's device operator API on
+// one MI355X.
+//
+// The reference executor drives every device op through the virtuals of
+// `qw3::DeviceBackend` (include/qw3/device_backend.hpp:88-).  This class
+// implements, with the same names, arguments and DeviceStatus conventions, the
+// ones that lie on the Q8_0 hot path:
+//   weight_q8_0 (:215), q8_0_matvec (:300), q8_0_matvec_add (:309),
+//   q8_0_matvec_silu_mul (:322), q8_0_matmul_silu_mul (:332),
+//   q8_0_matvec_fanout (:372), q8_0_matmul (:387), q8_0_matmul_fanout (:406),
+//   q8_0_matmul_add (:529), argmax (:2456), argmax_buffer / argmax_to_buffer /
+//   copy_argmax_buffer_to_host (:2458-2473), argmax_batch (:2477),
+//   argmax_launch / argmax_collect (:2503-2509), begin/end_capture, replay_graph
+//   (:120-122), plus the handful of tensor calls a test needs.
+// Routing follows the reference's CUDA backend (src/kernels_cuda.cu:10764-12630,
+// 14559-14658) except where noted in the .cpp; one op is new: lm_head_verify.
+//
+// The small value types below repeat the reference's declarations
+// (device_backend.hpp:24-69) so this header stands alone; inside the reference
+// tree a maintainer deletes them, includes the real header and derives from
+// DeviceBackend.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <memory>
+#include <vector>
+
+namespace qw3 {
+
+struct DeviceStatus {
+    bool ok = true;
+    const char *message = "";
+};
+
+enum class DeviceTensorDType { F32, F16, BF16, I32, Q8_KV, FP8_E4M3 };
+
+struct DeviceTensor {
+    virtual ~DeviceTensor() = default;
+    uint64_t count = 0;
+    uint32_t elem_size = 4;
+    DeviceTensorDType dtype = DeviceTensorDType::F32;
+};
+
+enum class DeviceWeightFormat { F32, BF16, FP8_E4M3, Q8_0, NVFP4_E2M1 };
+
+struct DeviceWeight {
+    virtual ~DeviceWeight() = default;
+    uint64_t rows = 0;
+    uint64_t cols = 0;
+    DeviceWeightFormat format = DeviceWeightFormat::F32;
+};
+
+struct DeviceArgmax {
+    int token = -1;
+    float logit = 0.0f;
+};
+
+struct DeviceArgmaxBuffer {
+    virtual ~DeviceArgmaxBuffer() = default;
+    uint64_t count = 0;
+};
+
+class HipQ8Backend {
+public:
+    HipQ8Backend();
+    ~HipQ8Backend();
+    HipQ8Backend(const HipQ8Backend &) = delete;
+    HipQ8Backend &operator=(const HipQ8Backend &) = delete;
+
+    const char *name() const { return "hip-q8 (gfx950)"; }
+    DeviceStatus begin() { return {}; }
+    DeviceStatus end();           // drains the exec stream (src/kernels_cuda.cu:9807-9823)
+    DeviceStatus synchronize();
+    hipStream_t exec_stream() const { return stream_; }
+
+    // HIP-graph capture of whatever is launched between begin_capture and end_capture
+    bool begin_capture();
+    DeviceStatus end_capture();
+    DeviceStatus replay_graph();
+
+    // tensors / weights
+    std::unique_ptr<DeviceTensor> tensor_f32(uint64_t count, const char *label);
+    std::unique_ptr<DeviceTensor> tensor_bf16(uint64_t count, const char *label);
+    // `data`: interleaved GGUF Q8_0 blocks (34 B); stored split-plane on the device
+    std::unique_ptr<DeviceWeight> weight_q8_0(const void *data, uint64_t rows, uint64_t cols, const char *label);
+    DeviceStatus copy_bytes_from_host(DeviceTensor &x, uint64_t byte_offset, const void *host, uint64_t bytes);
+    DeviceStatus copy_to_host(const DeviceTensor &x, float *host, uint64_t offset, uint64_t count);
+    DeviceStatus copy_bytes_to_host(const DeviceTensor &x, void *host, uint64_t byte_offset, uint64_t bytes);
+    DeviceStatus zero_tensor(DeviceTensor &x);
+
+    // decode-side linear ops (batch 1)
+    DeviceStatus q8_0_matvec(DeviceTensor &out, const DeviceWeight &weight, const DeviceTensor &x);
+    DeviceStatus q8_0_matvec_add(DeviceTensor &accum, const DeviceWeight &weight, const DeviceTensor &x);
+    DeviceStatus q8_0_matvec_silu_mul(DeviceTensor &out, const DeviceWeight &weight_gate,
+                                      const DeviceWeight &weight_up, const DeviceTensor &x);
+    DeviceStatus q8_0_matvec_fanout(DeviceTensor *const *outs, const DeviceWeight *const *weights, uint32_t n,
+                                    const DeviceTensor &x);
+
+    // prefill / verify linear ops
+    DeviceStatus q8_0_matmul(DeviceTensor &out, const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
+                             uint32_t in_stride, uint32_t out_stride);
+    DeviceStatus q8_0_matmul_fanout(DeviceTensor *const *outs, const DeviceWeight *const *weights,
+                                    const uint32_t *out_strides, uint32_t n, const DeviceTensor &x, uint32_t batch,
+                                    uint32_t in_stride);
+    DeviceStatus q8_0_matmul_add(DeviceTensor &out, const DeviceTensor &residual, DeviceTensor &matmul_tmp,
+                                 const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
+                                 uint32_t in_stride, uint32_t out_stride);
+    DeviceStatus q8_0_matmul_silu_mul(DeviceTensor &out, const DeviceWeight &weight_gate,
+                                      const DeviceWeight &weight_up, const DeviceTensor &x, uint32_t batch,
+                                      uint32_t in_stride, uint32_t out_stride);
+
+    // argmax
+    DeviceArgmax argmax(const DeviceTensor &x);
+    DeviceStatus argmax_launch(const DeviceTensor &x);
+    DeviceArgmax argmax_collect();
+    std::unique_ptr<DeviceArgmaxBuffer> argmax_buffer(uint64_t count);
+    DeviceStatus argmax_to_buffer(const DeviceTensor &x, DeviceArgmaxBuffer &out, uint32_t index);
+    DeviceStatus copy_argmax_buffer_to_host(const DeviceArgmaxBuffer &src, DeviceArgmax *host, uint32_t count);
+    DeviceStatus argmax_batch(const DeviceTensor &x, uint32_t batch, uint32_t row_stride,
+                              std::vector<DeviceArgmax> &out);
+
+    // New op (no counterpart in the reference): the whole verify tail in one pass
+    // over the LM-head weights.  Equivalent to q8_0_matmul(logits, w_out, norm, batch,
+    // in_stride, vocab) + argmax_batch + the greedy accept loop
+    // (src/qwen_executor.cpp:6779-6821, src/qwen_native_backend.cpp:15948-15960,
+    // 16048-16052).  rows_out[i] gates drafts[i]; `accepted` is the number of
+    // leading drafts equal to their row's token; `next_token` = token of row
+    // `accepted` (eos if that row has none).
+    DeviceStatus lm_head_verify(const DeviceWeight &w_out, const DeviceTensor &norm, uint32_t batch,
+                                uint32_t in_stride, const int32_t *drafts, uint32_t n_drafts, int32_t eos,
+                                std::vector<DeviceArgmax> &rows_out, uint32_t &accepted, int32_t &next_token);
+
+private:
+    struct Scratch {
+        void *ptr = nullptr;
+        size_t capacity = 0;
+    };
+    DeviceStatus ensure(Scratch &s, size_t need, const char *what);
+    DeviceStatus launch_status(const char *where);
+    DeviceStatus failed(const char *where);
+    DeviceStatus quantize_q8_1(const float *x, uint32_t batch, uint32_t cols, uint32_t stride);
+    DeviceStatus gemv_route(float *out, const DeviceWeight &w, const float *x, uint32_t batch, uint32_t in_stride,
+                            uint32_t out_stride);
+
+    hipStream_t stream_ = nullptr;
+    Scratch q8_1_, d4_, argmax_partial_, argmax_result_, lm_head_, lm_rows_, out_f32_;
+    int32_t *argmax_dev_ = nullptr;    // {token, logit bits}
+    int32_t *argmax_host_ = nullptr;   // pinned mirror
+    int32_t *accept_dev_ = nullptr;    // {accepted, next}
+    hipGraph_t graph_ = nullptr;
+    hipGraphExec_t graph_exec_ = nullptr;
+    bool capturing_ = false;
+};
+
+}  // namespace qw3

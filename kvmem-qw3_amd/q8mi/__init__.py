@@ -46,6 +46,7 @@ SIGNATURES = {
     "q8mi_quantize_q8_1_d4": (_int, [_vp, _vp, _u32, _u32, _u32, _vp]),
     "q8mi_gemm": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_gemm_medium": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_f32_to_bf16": (_int, [_vp, _vp, _u64, _vp]),
     "q8mi_block_dots": (_int, [_u8p, _vp, _int, _u32, _u32, _u32, _vp, _vp, _vp, _u32, _vp, _vp]),
     "q8mi_argmax": (_int, [_vp, _u64, _vp, _vp]),
     "q8mi_argmax_to_pair": (_int, [_vp, _u64, _vp, _u32, _vp]),

@@ -1,0 +1,503 @@
+// Parity driver for HipQ8Backend: every op is called the way the reference's
+// executor and its own backend tests call it (tests/mixed_linear_parity.cu:205-278
+// for the closed-form case) and checked against the CPU oracle on seeded inputs.
+// Prints one line per case; exit code 0 only if all pass.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../kvmem-qw3_amd/host/hip_q8_backend.hpp"
+#include "../../oracle/q8_oracle.h"
+
+namespace {
+
+int g_failed = 0;
+int g_cases = 0;
+
+void report(const char *name, bool ok, const std::string &detail = "") {
+    ++g_cases;
+    if (!ok) ++g_failed;
+    std::printf("%s %s%s%s\n", ok ? "PASS" : "FAIL", name, detail.empty() ? "" : ": ", detail.c_str());
+    std::fflush(stdout);
+}
+
+bool require(const qw3::DeviceStatus &st, const char *what) {
+    if (!st.ok) {
+        std::printf("  status: %s: %s\n", what, st.message);
+        std::fflush(stdout);
+    }
+    return st.ok;
+}
+
+struct Rng {   // splitmix64
+    uint64_t s;
+    explicit Rng(uint64_t seed) : s(seed) {}
+    uint64_t next() {
+        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    float uniform() { return static_cast<float>(next() >> 40) * (1.0f / 16777216.0f); }
+    float normal() {
+        const float u1 = uniform() + 1e-7f, u2 = uniform();
+        return std::sqrt(-2.0f * std::log(u1)) * std::cos(6.2831853f * u2);
+    }
+};
+
+std::vector<float> normal_vec(size_t n, uint64_t seed, float scale = 1.0f) {
+    Rng r(seed);
+    std::vector<float> v(n);
+    for (auto &f : v) f = r.normal() * scale;
+    return v;
+}
+
+struct HostWeight {
+    uint32_t rows, cols;
+    std::vector<uint8_t> gguf;    // interleaved blocks handed to weight_q8_0
+    std::vector<uint8_t> split;   // oracle's split-plane copy
+};
+
+HostWeight make_weight(uint32_t rows, uint32_t cols, uint64_t seed) {
+    HostWeight w{rows, cols, {}, {}};
+    const auto vals = normal_vec(static_cast<size_t>(rows) * cols, seed, 0.05f);
+    w.gguf.resize(static_cast<size_t>(rows) * (cols / 32) * 34);
+    w.split.resize(w.gguf.size());
+    q8o_quantize_q8_0(vals.data(), rows, cols, w.gguf.data());
+    q8o_repack_split_plane(w.gguf.data(), rows, cols, w.split.data());
+    return w;
+}
+
+// oracle result for any batch (slices of 8, like the reference's GEMV dispatch)
+void oracle_linear(const HostWeight &w, const float *x, uint32_t batch, uint32_t in_stride, uint32_t out_stride,
+                   std::vector<float> &ref, std::vector<float> &mag) {
+    ref.assign(static_cast<size_t>(batch) * out_stride, 0.0f);
+    mag.assign(ref.size(), 0.0f);
+    std::vector<uint8_t> y(static_cast<size_t>(8) * (w.cols / 32) * 36);
+    for (uint32_t j0 = 0; j0 < batch; j0 += 8) {
+        const uint32_t m = batch - j0 < 8 ? batch - j0 : 8;
+        q8o_quantize_q8_1(x + static_cast<size_t>(j0) * in_stride, m, w.cols, in_stride, y.data());
+        q8o_gemv(w.split.data(), y.data(), ref.data() + static_cast<size_t>(j0) * out_stride, w.rows, w.cols, m,
+                 out_stride, 4);
+        q8o_gemv_abs(w.split.data(), y.data(), mag.data() + static_cast<size_t>(j0) * out_stride, w.rows, w.cols, m,
+                     out_stride);
+    }
+}
+
+void oracle_gemm_d4(const HostWeight &w, const float *x, uint32_t batch, std::vector<float> &ref) {
+    std::vector<uint8_t> y(static_cast<size_t>(w.cols / 128) * batch * 144);
+    q8o_quantize_q8_1_d4(x, batch, w.cols, w.cols, y.data());
+    ref.assign(static_cast<size_t>(batch) * w.rows, 0.0f);
+    q8o_gemm_d4(w.split.data(), y.data(), ref.data(), w.rows, w.cols, batch, w.rows, 8);
+}
+
+// |got - ref| <= 1e-5 |ref| + 1e-6 * sum|terms|: the allowance for a different
+// fp32 summation order over the same exact per-block products
+bool close_fp32(const std::vector<float> &got, const std::vector<float> &ref, const std::vector<float> &mag,
+                uint32_t batch, uint32_t rows, uint32_t stride, std::string &detail) {
+    for (uint32_t j = 0; j < batch; ++j)
+        for (uint32_t r = 0; r < rows; ++r) {
+            const size_t i = static_cast<size_t>(j) * stride + r;
+            const float tol = 1e-5f * std::fabs(ref[i]) + 1e-6f * mag[i] + 1e-30f;
+            if (!(std::fabs(got[i] - ref[i]) <= tol)) {
+                char buf[160];
+                std::snprintf(buf, sizeof(buf), "[%u,%u] got %.9g want %.9g tol %.3g", j, r, got[i], ref[i], tol);
+                detail = buf;
+                return false;
+            }
+        }
+    return true;
+}
+
+bool close_abs_rel(const std::vector<float> &got, const std::vector<float> &want, float atol, float rtol,
+                   std::string &detail) {
+    if (got.size() != want.size()) { detail = "size mismatch"; return false; }
+    for (size_t i = 0; i < got.size(); ++i) {
+        if (!(std::fabs(got[i] - want[i]) <= atol + rtol * std::fabs(want[i]))) {
+            char buf[128];
+            std::snprintf(buf, sizeof(buf), "[%zu] got %.6g want %.6g", i, got[i], want[i]);
+            detail = buf;
+            return false;
+        }
+    }
+    return true;
+}
+
+std::unique_ptr<qw3::DeviceTensor> upload_f32(qw3::HipQ8Backend &b, const std::vector<float> &v) {
+    auto t = b.tensor_f32(v.size(), "t");
+    if (t) require(b.copy_bytes_from_host(*t, 0, v.data(), v.size() * 4), "upload");
+    return t;
+}
+
+std::vector<float> download_f32(qw3::HipQ8Backend &b, const qw3::DeviceTensor &t) {
+    std::vector<float> v(t.count);
+    require(b.copy_to_host(t, v.data(), 0, t.count), "download");
+    return v;
+}
+
+std::vector<float> download_bf16(qw3::HipQ8Backend &b, const qw3::DeviceTensor &t) {
+    std::vector<uint16_t> raw(t.count);
+    require(b.copy_bytes_to_host(t, raw.data(), 0, t.count * 2), "download bf16");
+    std::vector<float> v(t.count);
+    for (size_t i = 0; i < v.size(); ++i) v[i] = q8o_bf16_to_f32(raw[i]);
+    return v;
+}
+
+// ---- cases ----------------------------------------------------------------------------------------
+
+// Same data and tolerances as the reference's closed-form backend test: every
+// weight block is d = 0.5, q = 1; activations are constant per row.
+void case_closed_form(qw3::HipQ8Backend &b) {
+    constexpr uint32_t rows = 128, cols = 512, batch = 1024;
+    std::vector<uint8_t> packed(static_cast<size_t>(rows) * (cols / 32) * 34);
+    const uint16_t half = q8o_f32_to_f16(0.5f);
+    for (size_t blk = 0; blk < packed.size() / 34; ++blk) {
+        std::memcpy(&packed[blk * 34], &half, 2);
+        std::memset(&packed[blk * 34 + 2], 1, 32);
+    }
+    auto weight = b.weight_q8_0(packed.data(), rows, cols, "w");
+    std::string d;
+    bool ok = weight != nullptr;
+
+    const std::vector<float> single(cols, 0.25f);
+    auto x1 = upload_f32(b, single);
+    const float want1 = cols * 0.5f * 0.25f;
+    auto out1 = b.tensor_bf16(rows, "o");
+    ok = ok && require(b.q8_0_matvec(*out1, *weight, *x1), "matvec bf16");
+    ok = ok && close_abs_rel(download_bf16(b, *out1), std::vector<float>(rows, want1), 0.1f, 0.005f, d);
+    report("closed_form/matvec_bf16", ok, d);
+
+    auto res = b.tensor_bf16(rows, "r");
+    const std::vector<uint16_t> two(rows, q8o_f32_to_bf16(2.0f));
+    ok = require(b.copy_bytes_from_host(*res, 0, two.data(), two.size() * 2), "copy residual");
+    ok = ok && require(b.q8_0_matvec_add(*res, *weight, *x1), "matvec_add bf16");
+    ok = ok && close_abs_rel(download_bf16(b, *res), std::vector<float>(rows, 2.0f + want1), 0.1f, 0.005f, d);
+    report("closed_form/matvec_add_bf16", ok, d);
+
+    std::vector<float> xin(static_cast<size_t>(batch) * cols), want(static_cast<size_t>(batch) * rows);
+    for (uint32_t j = 0; j < batch; ++j) {
+        const float v = static_cast<float>(j + 1) / 64.0f;
+        std::fill(xin.begin() + static_cast<size_t>(j) * cols, xin.begin() + static_cast<size_t>(j + 1) * cols, v);
+        std::fill(want.begin() + static_cast<size_t>(j) * rows, want.begin() + static_cast<size_t>(j + 1) * rows,
+                  cols * 0.5f * v);
+    }
+    auto xb = upload_f32(b, xin);
+    auto ob = b.tensor_bf16(want.size(), "ob");
+    ok = require(b.q8_0_matmul(*ob, *weight, *xb, batch, cols, rows), "matmul bf16");
+    ok = ok && close_abs_rel(download_bf16(b, *ob), want, 0.25f, 0.01f, d);
+    report("closed_form/matmul_bf16_batch1024", ok, d);
+
+    // the same in fp32: amax/127 scales make x/d exactly 127, so the result is exact
+    auto of = b.tensor_f32(want.size(), "of");
+    ok = require(b.q8_0_matmul(*of, *weight, *xb, batch, cols, rows), "matmul f32");
+    ok = ok && close_abs_rel(download_f32(b, *of), want, 0.0f, 2e-6f, d);
+    report("closed_form/matmul_f32_batch1024", ok, d);
+}
+
+void case_matvec_family(qw3::HipQ8Backend &b) {
+    const uint32_t rows = 1000, cols = 2048;
+    const HostWeight w = make_weight(rows, cols, 11), w2 = make_weight(rows, cols, 12);
+    auto dw = b.weight_q8_0(w.gguf.data(), rows, cols, "w");
+    auto dw2 = b.weight_q8_0(w2.gguf.data(), rows, cols, "w2");
+    const auto x = normal_vec(cols, 13);
+    auto dx = upload_f32(b, x);
+    std::vector<float> ref, mag, ref2, mag2;
+    oracle_linear(w, x.data(), 1, cols, rows, ref, mag);
+    oracle_linear(w2, x.data(), 1, cols, rows, ref2, mag2);
+    std::string d;
+
+    auto out = b.tensor_f32(rows, "o");
+    bool ok = require(b.q8_0_matvec(*out, *dw, *dx), "matvec");
+    ok = ok && close_fp32(download_f32(b, *out), ref, mag, 1, rows, rows, d);
+    report("matvec_f32", ok, d);
+
+    const auto base = normal_vec(rows, 14);
+    auto acc = upload_f32(b, base);
+    ok = require(b.q8_0_matvec_add(*acc, *dw, *dx), "matvec_add");
+    std::vector<float> want(rows), magadd(rows);
+    for (uint32_t r = 0; r < rows; ++r) { want[r] = base[r] + ref[r]; magadd[r] = mag[r] + std::fabs(base[r]); }
+    ok = ok && close_fp32(download_f32(b, *acc), want, magadd, 1, rows, rows, d);
+    report("matvec_add_f32", ok, d);
+
+    // silu(g) * u: compared against the oracle's own fused form; tolerance widened
+    // by the derivative bound |silu'| <= 1.1 and one ulp of expf
+    std::vector<uint8_t> y(static_cast<size_t>(cols / 32) * 36);
+    q8o_quantize_q8_1(x.data(), 1, cols, cols, y.data());
+    std::vector<float> silu(rows);
+    q8o_gemv_silu_mul(w.split.data(), w2.split.data(), y.data(), silu.data(), rows, cols, 1, rows);
+    ok = require(b.q8_0_matvec_silu_mul(*out, *dw, *dw2, *dx), "silu_mul");
+    {
+        const auto got = download_f32(b, *out);
+        for (uint32_t r = 0; r < rows && ok; ++r) {
+            const float tg = 1e-5f * std::fabs(ref[r]) + 1e-6f * mag[r];
+            const float tu = 1e-5f * std::fabs(ref2[r]) + 1e-6f * mag2[r];
+            const float tol = 1.1f * tg * std::fabs(ref2[r]) + tu * std::fabs(ref[r]) + 4e-7f * std::fabs(silu[r]) +
+                              1e-30f;
+            if (!(std::fabs(got[r] - silu[r]) <= tol)) {
+                char buf[128];
+                std::snprintf(buf, sizeof(buf), "[%u] got %.9g want %.9g tol %.3g", r, got[r], silu[r], tol);
+                d = buf;
+                ok = false;
+            }
+        }
+    }
+    report("matvec_silu_mul", ok, d);
+
+    // fan-out: three weights of different heights sharing one activation
+    const HostWeight wa = make_weight(768, cols, 21), wb = make_weight(130, cols, 22), wc = make_weight(31, cols, 23);
+    auto da = b.weight_q8_0(wa.gguf.data(), wa.rows, cols, "a");
+    auto db = b.weight_q8_0(wb.gguf.data(), wb.rows, cols, "b");
+    auto dc = b.weight_q8_0(wc.gguf.data(), wc.rows, cols, "c");
+    auto oa = b.tensor_f32(wa.rows, "oa"), ob = b.tensor_f32(wb.rows, "ob"), oc = b.tensor_f32(wc.rows, "oc");
+    qw3::DeviceTensor *outs[3] = {oa.get(), ob.get(), oc.get()};
+    const qw3::DeviceWeight *ws[3] = {da.get(), db.get(), dc.get()};
+    ok = require(b.q8_0_matvec_fanout(outs, ws, 3, *dx), "fanout");
+    const HostWeight *hw[3] = {&wa, &wb, &wc};
+    for (int i = 0; i < 3 && ok; ++i) {
+        oracle_linear(*hw[i], x.data(), 1, cols, hw[i]->rows, ref, mag);
+        ok = close_fp32(download_f32(b, *outs[i]), ref, mag, 1, hw[i]->rows, hw[i]->rows, d);
+    }
+    report("matvec_fanout3", ok, d);
+}
+
+void case_matmul(qw3::HipQ8Backend &b) {
+    std::string d;
+    // batch <= 8 and strided batches: GEMV route, bit-for-bit the Q8_1 quantizer
+    {
+        const uint32_t rows = 515, cols = 1024;
+        const HostWeight w = make_weight(rows, cols, 31);
+        auto dw = b.weight_q8_0(w.gguf.data(), rows, cols, "w");
+        for (uint32_t batch : {2u, 5u, 8u, 19u}) {
+            const uint32_t in_stride = cols + 64, out_stride = rows + 9;
+            const auto x = normal_vec(static_cast<size_t>(batch) * in_stride, 32 + batch);
+            auto dx = upload_f32(b, x);
+            auto out = b.tensor_f32(static_cast<size_t>(batch) * out_stride, "o");
+            require(b.zero_tensor(*out), "zero");
+            bool ok = require(b.q8_0_matmul(*out, *dw, *dx, batch, in_stride, out_stride), "matmul strided");
+            std::vector<float> ref, mag;
+            oracle_linear(w, x.data(), batch, in_stride, out_stride, ref, mag);
+            const auto got = download_f32(b, *out);
+            ok = ok && close_fp32(got, ref, mag, batch, rows, out_stride, d);
+            for (uint32_t j = 0; j < batch && ok; ++j)     // the gap between rows stays untouched
+                for (uint32_t r = rows; r < out_stride; ++r)
+                    if (got[static_cast<size_t>(j) * out_stride + r] != 0.0f) { ok = false; d = "wrote into the stride gap"; }
+            report(("matmul_strided_batch" + std::to_string(batch)).c_str(), ok, d);
+        }
+    }
+    // contiguous batch > 8, D4 layout: MFMA tile (and its medium-batch variant)
+    {
+        const uint32_t rows = 384, cols = 1024;
+        const HostWeight w = make_weight(rows, cols, 41);
+        auto dw = b.weight_q8_0(w.gguf.data(), rows, cols, "w");
+        for (uint32_t batch : {9u, 16u, 64u, 65u, 300u}) {
+            const auto x = normal_vec(static_cast<size_t>(batch) * cols, 42 + batch);
+            auto dx = upload_f32(b, x);
+            auto out = b.tensor_f32(static_cast<size_t>(batch) * rows, "o");
+            bool ok = require(b.q8_0_matmul(*out, *dw, *dx, batch, cols, rows), "matmul d4");
+            std::vector<float> ref, lin, mag;
+            oracle_gemm_d4(w, x.data(), batch, ref);
+            oracle_linear(w, x.data(), batch, cols, rows, lin, mag);   // magnitudes only
+            ok = ok && close_fp32(download_f32(b, *out), ref, mag, batch, rows, rows, d);
+            report(("matmul_d4_batch" + std::to_string(batch)).c_str(), ok, d);
+        }
+    }
+    // contiguous batch > 8 where the layout rule keeps Q8_1 (rows < 128, cols % 128 != 0)
+    {
+        const uint32_t rows = 100, cols = 480, batch = 40;
+        const HostWeight w = make_weight(rows, cols, 51);
+        auto dw = b.weight_q8_0(w.gguf.data(), rows, cols, "w");
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 52);
+        auto dx = upload_f32(b, x);
+        auto out = b.tensor_f32(static_cast<size_t>(batch) * rows, "o");
+        bool ok = require(b.q8_0_matmul(*out, *dw, *dx, batch, cols, rows), "matmul q8_1 layout");
+        std::vector<float> ref, mag;
+        oracle_linear(w, x.data(), batch, cols, rows, ref, mag);
+        ok = ok && close_fp32(download_f32(b, *out), ref, mag, batch, rows, rows, d);
+        report("matmul_q8_1_layout_batch40", ok, d);
+    }
+    // fan-out at batch 4 and in-place residual add at batch 3
+    {
+        const uint32_t cols = 768, batch = 4;
+        const HostWeight wa = make_weight(256, cols, 61), wb = make_weight(64, cols, 62);
+        auto da = b.weight_q8_0(wa.gguf.data(), wa.rows, cols, "a");
+        auto db = b.weight_q8_0(wb.gguf.data(), wb.rows, cols, "b");
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 63);
+        auto dx = upload_f32(b, x);
+        const uint32_t strides[2] = {300, 64};
+        auto oa = b.tensor_f32(batch * strides[0], "oa"), ob = b.tensor_f32(batch * strides[1], "ob");
+        qw3::DeviceTensor *outs[2] = {oa.get(), ob.get()};
+        const qw3::DeviceWeight *ws[2] = {da.get(), db.get()};
+        bool ok = require(b.q8_0_matmul_fanout(outs, ws, strides, 2, *dx, batch, cols), "matmul_fanout");
+        std::vector<float> ref, mag;
+        oracle_linear(wa, x.data(), batch, cols, strides[0], ref, mag);
+        ok = ok && close_fp32(download_f32(b, *oa), ref, mag, batch, wa.rows, strides[0], d);
+        oracle_linear(wb, x.data(), batch, cols, strides[1], ref, mag);
+        ok = ok && close_fp32(download_f32(b, *ob), ref, mag, batch, wb.rows, strides[1], d);
+        report("matmul_fanout_batch4", ok, d);
+
+        const uint32_t nb = 3;
+        const auto base = normal_vec(static_cast<size_t>(nb) * wa.rows, 64);
+        auto acc = upload_f32(b, base);
+        auto tmp = b.tensor_f32(1, "tmp");
+        ok = require(b.q8_0_matmul_add(*acc, *acc, *tmp, *da, *dx, nb, cols, wa.rows), "matmul_add");
+        oracle_linear(wa, x.data(), nb, cols, wa.rows, ref, mag);
+        for (size_t i = 0; i < ref.size(); ++i) { ref[i] += base[i]; mag[i] += std::fabs(base[i]); }
+        ok = ok && close_fp32(download_f32(b, *acc), ref, mag, nb, wa.rows, wa.rows, d);
+        report("matmul_add_inplace_batch3", ok, d);
+
+        // forms the backend declines, as the reference does, so that the caller's fallback runs
+        auto other = b.tensor_f32(static_cast<size_t>(nb) * wa.rows, "other");
+        ok = !b.q8_0_matmul_add(*other, *acc, *tmp, *da, *dx, nb, cols, wa.rows).ok;
+        ok = ok && !b.q8_0_matmul_silu_mul(*other, *da, *da, *dx, nb, cols, wa.rows).ok;
+        ok = ok && b.weight_q8_0(wa.gguf.data(), 4, 40, "bad") == nullptr;
+        report("declined_forms", ok);
+    }
+}
+
+void case_argmax(qw3::HipQ8Backend &b) {
+    std::string d;
+    const uint32_t n = 248320;
+    auto logits = normal_vec(n, 71);
+    logits[777] = logits[200000] = 9.5f;   // a tie: the lower index wins
+    auto dl = upload_f32(b, logits);
+    const q8o_argmax_pair want = q8o_argmax_row(logits.data(), n);
+    const qw3::DeviceArgmax got = b.argmax(*dl);
+    report("argmax_vocab", got.token == want.index && got.logit == want.value && got.token == 777);
+
+    bool ok = require(b.argmax_launch(*dl), "argmax_launch");
+    const qw3::DeviceArgmax late = b.argmax_collect();
+    report("argmax_launch_collect", ok && late.token == want.index && late.logit == want.value);
+
+    auto buf = b.argmax_buffer(4);
+    ok = buf != nullptr && require(b.argmax_to_buffer(*dl, *buf, 2), "argmax_to_buffer");
+    qw3::DeviceArgmax host[4] = {};
+    ok = ok && require(b.copy_argmax_buffer_to_host(*buf, host, 3), "copy_argmax_buffer_to_host");
+    ok = ok && host[2].token == want.index && host[2].logit == want.value;
+    ok = ok && !b.argmax_to_buffer(*dl, *buf, 4).ok && b.argmax_buffer(0) == nullptr;
+    report("argmax_to_buffer", ok);
+
+    for (uint32_t stride : {1000u, 50000u, 262144u, 262145u}) {   // the last takes the host scan
+        const uint32_t batch = 5;
+        auto x = normal_vec(static_cast<size_t>(batch) * stride, 72 + stride);
+        x[static_cast<size_t>(3) * stride + 10] = x[static_cast<size_t>(3) * stride + 900] = 8.0f;
+        for (uint32_t c = 0; c < stride; ++c) x[static_cast<size_t>(4) * stride + c] = -INFINITY;
+        auto dx = upload_f32(b, x);
+        std::vector<qw3::DeviceArgmax> rows;
+        ok = require(b.argmax_batch(*dx, batch, stride, rows), "argmax_batch");
+        std::vector<q8o_argmax_pair> ref(batch);
+        if (q8o_argmax_rows(x.data(), batch, stride, ref.data()) != 0) q8o_argmax_rows_scan(x.data(), batch, stride, ref.data());
+        for (uint32_t j = 0; j < batch && ok; ++j)
+            if (rows[j].token != ref[j].index || std::memcmp(&rows[j].logit, &ref[j].value, 4) != 0) {
+                ok = false;
+                d = "row " + std::to_string(j) + " got " + std::to_string(rows[j].token) + " want " + std::to_string(ref[j].index);
+            }
+        report(("argmax_batch_stride" + std::to_string(stride)).c_str(), ok, d);
+    }
+}
+
+void case_lm_head_verify(qw3::HipQ8Backend &b) {
+    const uint32_t vocab = 30000, cols = 1024, eos = 5;
+    const HostWeight w = make_weight(vocab, cols, 81);
+    auto dw = b.weight_q8_0(w.gguf.data(), vocab, cols, "lm");
+    for (uint32_t batch : {1u, 4u, 8u}) {
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 82 + batch);
+        auto dx = upload_f32(b, x);
+        std::vector<float> ref, mag;
+        oracle_linear(w, x.data(), batch, cols, vocab, ref, mag);
+        std::vector<q8o_argmax_pair> rows(batch);
+        q8o_argmax_rows_scan(ref.data(), batch, vocab, rows.data());
+        std::vector<int32_t> toks(batch);
+        for (uint32_t j = 0; j < batch; ++j) toks[j] = rows[j].index;
+        bool ok = true;
+        std::string d;
+        for (uint32_t prefix = 0; prefix < batch && ok; ++prefix) {
+            std::vector<int32_t> drafts(batch - 1);
+            for (uint32_t i = 0; i + 1 < batch; ++i) drafts[i] = i < prefix ? toks[i] : (toks[i] + 1) % static_cast<int32_t>(vocab);
+            int32_t want_next = -1;
+            const uint32_t want_acc = q8o_accept(toks.data(), drafts.data(), batch - 1, eos, &want_next);
+            std::vector<qw3::DeviceArgmax> got;
+            uint32_t acc = 99;
+            int32_t next = -1;
+            ok = require(b.lm_head_verify(*dw, *dx, batch, cols, drafts.data(), batch - 1, eos, got, acc, next), "lm_head_verify");
+            ok = ok && acc == want_acc && next == want_next && want_acc == prefix;
+            for (uint32_t j = 0; j < batch && ok; ++j) {
+                const float tol = 1e-5f * std::fabs(rows[j].value) + 1e-6f * mag[static_cast<size_t>(j) * vocab + rows[j].index];
+                ok = got[j].token == rows[j].index && std::fabs(got[j].logit - rows[j].value) <= tol;
+            }
+            if (!ok) d = "prefix " + std::to_string(prefix);
+        }
+        // the unfused route through the same API gives the same tokens
+        auto logits = b.tensor_f32(static_cast<size_t>(batch) * vocab, "logits");
+        std::vector<qw3::DeviceArgmax> unfused;
+        ok = ok && require(b.q8_0_matmul(*logits, *dw, *dx, batch, cols, vocab), "lm matmul");
+        ok = ok && require(b.argmax_batch(*logits, batch, vocab, unfused), "lm argmax_batch");
+        for (uint32_t j = 0; j < batch && ok; ++j) ok = unfused[j].token == rows[j].index;
+        report(("lm_head_verify_batch" + std::to_string(batch)).c_str(), ok, d);
+    }
+}
+
+// A captured decode-style sequence replayed several times with eager work and
+// synchronizations in between; every replay must equal the eager result bit for bit.
+void case_graph_replay(qw3::HipQ8Backend &b) {
+    const uint32_t hidden = 1024, ffn = 3072;
+    const HostWeight wg = make_weight(ffn, hidden, 91), wu = make_weight(ffn, hidden, 92), wd = make_weight(hidden, ffn, 93);
+    auto dg = b.weight_q8_0(wg.gguf.data(), ffn, hidden, "g");
+    auto du = b.weight_q8_0(wu.gguf.data(), ffn, hidden, "u");
+    auto dd = b.weight_q8_0(wd.gguf.data(), hidden, ffn, "d");
+    const auto x0 = normal_vec(hidden, 94);
+    auto x = upload_f32(b, x0);
+    auto act = b.tensor_f32(ffn, "act");
+    auto resid = b.tensor_f32(hidden, "resid");
+    auto step = [&]() {
+        return b.q8_0_matvec_silu_mul(*act, *dg, *du, *x).ok && b.q8_0_matvec_add(*resid, *dd, *act).ok;
+    };
+    bool ok = require(b.zero_tensor(*resid), "zero") && step() && require(b.synchronize(), "sync");   // eager: sizes the scratch
+    const auto eager = download_f32(b, *resid);
+    ok = ok && b.begin_capture() && step();
+    ok = require(b.end_capture(), "end_capture") && ok;
+    std::string d;
+    for (int rep = 0; rep < 4 && ok; ++rep) {
+        ok = require(b.zero_tensor(*resid), "zero") && require(b.replay_graph(), "replay") && require(b.synchronize(), "sync");
+        const auto got = download_f32(b, *resid);
+        if (std::memcmp(got.data(), eager.data(), got.size() * 4) != 0) { ok = false; d = "replay " + std::to_string(rep) + " differs"; }
+        // unrelated eager work between replays, using the same scratch
+        auto tmp = b.tensor_f32(ffn, "tmp");
+        ok = ok && b.q8_0_matvec(*tmp, *dg, *x).ok && require(b.synchronize(), "sync");
+    }
+    report("graph_replay_x4", ok, d);
+
+    // growth of a scratch buffer is refused while capturing
+    const HostWeight wbig = make_weight(64, 8192, 95);
+    auto dbig = b.weight_q8_0(wbig.gguf.data(), 64, 8192, "big");
+    auto xbig = upload_f32(b, normal_vec(static_cast<size_t>(8) * 8192, 96));
+    auto obig = b.tensor_f32(8 * 64, "obig");
+    ok = b.begin_capture();
+    const bool refused = !b.q8_0_matmul(*obig, *dbig, *xbig, 8, 8192, 64).ok;
+    (void)b.end_capture();
+    report("capture_refuses_scratch_growth", ok && refused);
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+    const std::string only = argc > 1 ? argv[1] : "";
+    qw3::HipQ8Backend backend;
+    std::printf("backend: %s\n", backend.name());
+    struct Case { const char *name; void (*fn)(qw3::HipQ8Backend &); };
+    const Case cases[] = {
+        {"closed_form", case_closed_form}, {"matvec", case_matvec_family}, {"matmul", case_matmul},
+        {"argmax", case_argmax}, {"lm_head", case_lm_head_verify}, {"graph", case_graph_replay},
+    };
+    for (const auto &c : cases) {
+        if (!only.empty() && only != c.name) continue;
+        std::printf("== %s\n", c.name);
+        std::fflush(stdout);
+        c.fn(backend);
+    }
+    require(backend.end(), "end");
+    std::printf("%d cases, %d failed\n", g_cases, g_failed);
+    return g_failed == 0 && g_cases > 0 ? 0 : 1;
+}
