@@ -181,6 +181,10 @@ int q8mi_repack_q8_0_split(const void *gguf_blocks, uint64_t rows, uint64_t cols
  * reference.  sink: one device uint32 (never written in practice). */
 int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per_cu, uint32_t *sink,
                     void *stream);
+/* Plain device-to-device copy of `bytes` bytes by a kernel (reads `bytes`,
+ * writes `bytes`): the known-size launch that hardware memory-traffic counters
+ * are calibrated against.  No counterpart in the reference. */
+int q8mi_probe_copy(const void *src, void *dst, uint64_t bytes, void *stream);
 
 /* ---- synthetic inputs (host side, for benches and tests) ----------------- */
 /* Counter-based generator: element i of stream `seed` depends only on

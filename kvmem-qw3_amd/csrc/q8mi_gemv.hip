@@ -6,8 +6,10 @@
 // kernel is a stream over the int8 plane of each row (see q8mi_gemv_core.hpp
 // for the streaming core).  This file adds what differs between the entry
 // points: which rows form a unit, and what happens to a finished unit (store,
-// residual add, bf16 rounding, SwiGLU).  All of that is wave-uniform and runs
-// once per unit, so it is a runtime switch rather than a template parameter.
+// residual add, bf16 rounding, SwiGLU).  Store/add/bf16 are wave-uniform and run
+// once per unit, so they are a runtime switch; SwiGLU changes which rows a unit
+// streams and is a template parameter (its launches also show up under their own
+// kernel name in a profile).
 #include <stdlib.h>
 
 #include "q8mi_gemv_core.hpp"
@@ -72,7 +74,7 @@ __device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, flo
 // Unit u covers rows R*u .. R*u+R-1 of the concatenated row space; for SwiGLU it
 // covers rows (R/2)*u .. of BOTH weights: slots 0..R/2-1 are gate rows, slots
 // R/2..R-1 the matching up rows.
-template <int M, int THREADS, int XMODE>
+template <int M, int THREADS, int XMODE, bool SILU>
 __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int R = RowsPerUnit<M>::value;
@@ -96,7 +98,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
     const uint32_t last_row = p.total_rows - 1;
 
     auto rows_of = [&](uint32_t u, RowPtrs<R> &rp) {
-        if (p.mode == kSiluMul) {
+        if constexpr (SILU) {
 #pragma unroll
             for (int r = 0; r < R / 2; ++r) {
                 uint32_t row = (R / 2) * u + r;
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
         }
         return t;
     };
-    if (p.mode == kSiluMul) {
+    if constexpr (SILU) {
         constexpr uint32_t kHalf = R / 2;
         for (uint32_t e = threadIdx.x; e < ucount * M * kHalf; e += THREADS) {
             const uint32_t k = e / (M * kHalf), m = (e / kHalf) % M, r = e % kHalf;
@@ -231,12 +233,12 @@ __global__ __launch_bounds__(256) void gemv_unaligned_kernel(const GemvParams p,
 }
 
 // One launch of a given instantiation: geometry is cached per (instantiation, LDS size).
-template <int M, int THREADS, int XMODE>
+template <int M, int THREADS, int XMODE, bool SILU>
 int launch_inst(GemvParams p, uint32_t x_bytes, hipStream_t stream) {
-    auto kern = gemv_kernel<M, THREADS, XMODE>;
+    auto kern = gemv_kernel<M, THREADS, XMODE, SILU>;
     constexpr uint32_t R = RowsPerUnit<M>::value;
     p.x_bytes = x_bytes;
-    p.units = p.mode == kSiluMul ? (p.total_rows + R / 2 - 1) / (R / 2) : (p.total_rows + R - 1) / R;
+    p.units = SILU ? (p.total_rows + R / 2 - 1) / (R / 2) : (p.total_rows + R - 1) / R;
     const uint32_t lds = x_bytes + (THREADS / kWave) * kParkFloats * 4;
     static thread_local uint32_t cached_lds = 0xffffffffu;
     static thread_local int cached_occ = 0;
@@ -269,16 +271,21 @@ int launch_inst(GemvParams p, uint32_t x_bytes, hipStream_t stream) {
     return check_launch("gemv");
 }
 
-template <int M>
-int launch_m(const GemvParams &p, hipStream_t stream) {
+template <int M, bool SILU>
+int launch_ms(const GemvParams &p, hipStream_t stream) {
     const uint32_t xb = x_lds_bytes(p.nb, M);
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
     const int forced = gemv_tuning().threads;
-    if (forced == 256 && xb + park_256 <= kLdsLimit) return launch_inst<M, 256, kXLds>(p, xb, stream);
-    if (forced == 1024 && xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds>(p, xb, stream);
-    if (xb + park_256 <= 76u * 1024u) return launch_inst<M, 256, kXLds>(p, xb, stream);   // two per CU fit
-    if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds>(p, xb, stream);
-    return launch_inst<M, 256, kXGlobal>(p, 0, stream);
+    if (forced == 256 && xb + park_256 <= kLdsLimit) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);
+    if (forced == 1024 && xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds, SILU>(p, xb, stream);
+    if (xb + park_256 <= 76u * 1024u) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);   // two per CU fit
+    if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds, SILU>(p, xb, stream);
+    return launch_inst<M, 256, kXGlobal, SILU>(p, 0, stream);
+}
+
+template <int M>
+int launch_m(const GemvParams &p, hipStream_t stream) {
+    return p.mode == kSiluMul ? launch_ms<M, true>(p, stream) : launch_ms<M, false>(p, stream);
 }
 
 int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {

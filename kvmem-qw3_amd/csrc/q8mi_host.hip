@@ -122,6 +122,14 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const v4i *__restrict__
     if ((a.x ^ a.y ^ a.z ^ a.w) == 0x5a17c0de && (a.x & a.y) == 0x0badf00d) sink[0] = 1;
 }
 
+// Plain copy, 16 bytes per lane per trip: a kernel whose HBM reads and writes are
+// both exactly `bytes`, used to calibrate memory-traffic counters.
+__global__ __launch_bounds__(256) void probe_copy_kernel(const v4i *__restrict__ src, v4i *__restrict__ dst,
+                                                         uint64_t n16) {
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 // ---- synthetic inputs --------------------------------------------------------
 inline uint64_t splitmix64(uint64_t z) {
     z += 0x9E3779B97F4A7C15ull;
@@ -236,6 +244,15 @@ extern "C" int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per
     const uint32_t grid = static_cast<uint32_t>(device_cu_count()) * wgs_per_cu;
     probe_read_kernel<<<grid, 256, 0, as_stream(stream)>>>(static_cast<const v4i *>(buf), bytes / 16, sink);
     return check_launch("probe_read");
+}
+
+extern "C" int q8mi_probe_copy(const void *src, void *dst, uint64_t bytes, void *stream) {
+    if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0)
+        return fail(Q8MI_REJECTED, "probe_copy: buffers must be 16-byte aligned and sized");
+    const uint32_t grid = static_cast<uint32_t>(device_cu_count()) * 8;
+    probe_copy_kernel<<<grid, 256, 0, as_stream(stream)>>>(static_cast<const v4i *>(src), static_cast<v4i *>(dst),
+                                                           bytes / 16);
+    return check_launch("probe_copy");
 }
 
 extern "C" int q8mi_synth_f32(float *out, uint64_t rows, uint64_t cols, uint64_t seed, int kind,

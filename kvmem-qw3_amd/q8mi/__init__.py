@@ -58,6 +58,7 @@ SIGNATURES = {
     "q8mi_repack_q8_0_split_host": (_int, [_vp, _u64, _u64, _vp]),
     "q8mi_repack_q8_0_split": (_int, [_vp, _u64, _u64, _vp, _vp]),
     "q8mi_probe_read": (_int, [_vp, _u64, _u32, _vp, _vp]),
+    "q8mi_probe_copy": (_int, [_vp, _vp, _u64, _vp]),
     "q8mi_synth_f32": (_int, [_vp, _u64, _u64, _u64, _int, C.c_float, _u32, C.c_float, _int]),
     "q8mi_synth_q8_0_weight": (_int, [_vp, _u64, _u64, _u64, C.c_float, _int]),
 }
