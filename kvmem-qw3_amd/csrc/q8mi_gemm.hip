@@ -13,6 +13,11 @@
 // makes the fp16 weight scale a per-lane constant and the output stores
 // contiguous along the weight-row axis (dst is [batch][rows]).
 //
+// Two staging variants share the tiling and the arithmetic.  Rows whose int8 plane is
+// 16-byte aligned (cols/32 a multiple of 8: every model shape) use direct global->LDS
+// loads, described where that kernel is defined; other rows use the register-staged
+// kernel below, whose LDS layout is:
+//
 // LDS record (144 B, both operands): [4 x fp32 scales][128 x int8].  The 144-B
 // pitch is what the D4 activation blocks already have in memory, and it spreads
 // the 16-byte fragment reads of 8 consecutive rows over all banks.  Activation
@@ -24,6 +29,8 @@
 // F = 12582912 + S exactly (|S| <= 516128 < 2^22).  g = fma(F, d_w, -12582912*d_w)
 // is then the correctly rounded d_w*S (12582912*d_w is exact: d_w has 11
 // significant bits), and acc = fma(g, d_y, acc): two FMAs per (output, block).
+#include <cstdio>
+
 #include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
 
@@ -228,6 +235,209 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_kernel(
     }
 }
 
+
+// ---- direct-to-LDS variant (rows whose int8 plane is 16-byte aligned) ----------------------
+// Stage layout (38912 B, two stages):
+//   [0, 16384)      weight quants, 128 rows x 128 B; 16-byte piece p of row r sits in slot p ^ swz(r),
+//                   so equal pieces of 8 or 16 consecutive rows fall on distinct banks
+//   [16384, 34816)  activation records exactly as in memory (128 x 144 B: 16 B scales + 128 B quants)
+//   [34816, 36864)  weight scales as fp32, [sub-block][row]
+//   [36864, 38912)  activation scales as fp32, [sub-block][row]
+// Quants travel global -> LDS without passing through registers (global_load_lds_dwordx4: lane l of
+// a wave writes 16 bytes at M0 + 16 l); only the scales go through registers.  All per-lane
+// offsets are constant over the K loop, the per-step bases are scalar, so staging costs ten
+// instructions per wave and step.
+constexpr int kWqBytes = kTileRows * 128;
+constexpr int kYrBytes = kTileCols * kRec;
+constexpr int kScBytes = 4 * 128 * 4;
+constexpr int kOffYr = kWqBytes, kOffWsc = kOffYr + kYrBytes, kOffYsc = kOffWsc + kScBytes;
+static_assert(kOffYsc + kScBytes == kStageBytes, "both variants use the same LDS budget");
+
+using gptr = const __attribute__((address_space(1))) void *;
+using lptr = __attribute__((address_space(3))) void *;
+
+// 16 bytes per lane from global memory straight into LDS at lds_wave_base + lane * 16.
+// Issued as inline assembly so that the compiler's wait-count pass does not make every later
+// LDS read wait for it; completion is awaited explicitly (vmcnt(0)) before the stage's barrier.
+__device__ __forceinline__ void dma16(const uint8_t *uniform_base, uint32_t lane_off, uint32_t lds_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_off), "v"(lane_off), "s"(uniform_base) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_offset_of(const void *p) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lptr)p));
+}
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    return reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// slot swizzle of the weight stage: 8 (and 16) consecutive rows put equal pieces on distinct banks
+__device__ __forceinline__ uint32_t swz(uint32_t row) { return (row & 7u) ^ ((row >> 3) & 1u); }
+
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+struct Scales { v2u wd; v4i yd; };
+
+// Per-lane byte offsets that do not change over the K loop.
+struct LaneOffsets {
+    uint32_t wq[4];   // weight quant chunk i of this wave, relative to the tile's first row + quant plane
+    uint32_t yr;      // lane * 16
+    uint32_t sc;      // weight row (tid % 128) of the scale load
+    uint32_t ysc;     // record (tid % 128) of the activation scale load
+};
+
+template <bool CHECK>
+__device__ __forceinline__ void stage_issue(uint32_t stage_off, Scales &sc, const LaneOffsets &lo,
+                                            const uint8_t *wq_base, const uint8_t *wd_base, const uint8_t *y_base,
+                                            uint32_t y_limit, uint32_t wave, uint32_t tid) {
+    // wq_base: tile's first row, quant plane, this super-block (uniform); y_base: first record of the stage
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(wq_base, lo.wq[i], stage_off + (wave * 4 + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+        const uint32_t c = wave + 4 * i;
+        if (c < 18) {
+            uint32_t off = c * 1024 + lo.yr;
+            if (CHECK) off = off <= y_limit ? off : y_limit;
+            dma16(y_base, off, stage_off + kOffYr + c * 1024);
+        }
+    }
+    // scales through registers; every thread loads both kinds (branch-free), half of each is used
+    sc.wd = *(const __attribute__((address_space(1))) v2u *)(wd_base + lo.sc);
+    uint32_t off = lo.ysc;
+    if (CHECK) off = off <= y_limit ? off : y_limit;
+    sc.yd = *(const __attribute__((address_space(1))) v4i *)(y_base + off);
+    (void)tid;
+}
+
+__device__ __forceinline__ void stage_scales(uint8_t *stage, const Scales &sc, uint32_t tid) {
+    if (tid < 128) {
+        float *wsc = reinterpret_cast<float *>(stage + kOffWsc);
+        wsc[0 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.x & 0xffffu));
+        wsc[1 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.x >> 16));
+        wsc[2 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.y & 0xffffu));
+        wsc[3 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.y >> 16));
+    } else {
+        int *ysc = reinterpret_cast<int *>(stage + kOffYsc);
+        const uint32_t j = tid - 128;
+        ysc[0 * 128 + j] = sc.yd.x; ysc[1 * 128 + j] = sc.yd.y; ysc[2 * 128 + j] = sc.yd.z; ysc[3 * 128 + j] = sc.yd.w;
+    }
+}
+
+template <bool CHECK>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const uint32_t tid = threadIdx.x, lane = tid % kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
+    const uint32_t id = blockIdx.x, xcd = id % 8u, seq = id / 8u;
+    const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
+    if (rt >= row_tiles) return;
+    const uint32_t row0 = rt * kTileRows, col0 = ct * kTileCols;
+    const uint32_t nsb = nb / 4;
+
+    v16i seed;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) seed[i] = static_cast<int>(kMagicBits);
+    float acc[4][16];
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
+
+    const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    LaneOffsets lo;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t r = (wave * 4 + i) * 8 + lane / 8;
+        uint32_t gr = r;
+        if (CHECK) gr = row0 + r < rows ? r : rows - 1 - row0;
+        lo.wq[i] = gr * static_cast<uint32_t>(row_bytes) + ((lane & 7u) ^ swz(r)) * 16;
+    }
+    lo.yr = lane * 16;
+    {
+        uint32_t gr = tid & 127u;
+        if (CHECK) gr = row0 + gr < rows ? gr : rows - 1 - row0;
+        lo.sc = gr * static_cast<uint32_t>(row_bytes);
+        lo.ysc = (tid & 127u) * kRec;
+    }
+    const uint8_t *wd_base = uniform_ptr(w + row0 * row_bytes);          // scale plane of the tile's first row
+    const uint8_t *wq_base = wd_base + 2 * nb;                            // quant plane
+    const uint8_t *y_base = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec);
+    const uint64_t y_step = static_cast<uint64_t>(batch) * kRec;
+    // last valid 16-byte offset from y_base within the whole activation buffer (CHECK only)
+    uint64_t y_room = static_cast<uint64_t>(nsb) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
+    const uint32_t smem_off = lds_offset_of(smem);
+
+    Scales sc;
+    stage_issue<CHECK>(smem_off, sc, lo, wq_base, wd_base, y_base,
+                       static_cast<uint32_t>(y_room < 0xffffffffull ? y_room : 0xffffffffull), wave, tid);
+    stage_scales(smem, sc, tid);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    const uint32_t fl = swz(l32);
+    const uint32_t a_off = kOffYr + (wave * 32 + l32) * kRec + 16 + lhalf * 16;
+    const uint32_t b_row = l32 * 128;
+    asm volatile("" : "+v"(seed));   // keep the seed in registers instead of rebuilding it per MFMA group
+
+    for (uint32_t sb = 0; sb < nsb; ++sb) {
+        const uint32_t cur_sel = (sb & 1u) * kStageBytes, nxt_sel = kStageBytes - cur_sel;
+        uint8_t *cur = smem + cur_sel;
+        const bool more = sb + 1 < nsb;
+        if (more) {
+            wq_base += 128; wd_base += 8; y_base += y_step; y_room -= y_step;
+            stage_issue<CHECK>(smem_off + nxt_sel, sc, lo, wq_base, wd_base, y_base,
+                               static_cast<uint32_t>(y_room < 0xffffffffull ? y_room : 0xffffffffull), wave, tid);
+        }
+        const float *wsc = reinterpret_cast<const float *>(cur + kOffWsc);
+        const float *ysc = reinterpret_cast<const float *>(cur + kOffYsc);
+#pragma unroll 1
+        for (uint32_t sub = 0; sub < 4; ++sub) {
+            const v4i a = *reinterpret_cast<const v4i *>(cur + a_off + sub * 32);
+            const uint32_t b_off = b_row + (((2 * sub + lhalf) ^ fl) * 16);
+            float dy[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 t = *reinterpret_cast<const float4 *>(ysc + sub * 128 + wave * 32 + 8 * g + 4 * lhalf);
+                dy[4 * g + 0] = t.x; dy[4 * g + 1] = t.y; dy[4 * g + 2] = t.z; dy[4 * g + 3] = t.w;
+            }
+            v16i r[4];
+            float dw[4];
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const v4i b = *reinterpret_cast<const v4i *>(cur + rb * 32 * 128 + b_off);
+                dw[rb] = wsc[sub * 128 + rb * 32 + l32];
+                r[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, seed, 0, 0, 0);
+            }
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const float cw = -kMagic * dw[rb];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float g = fmaf(as_f32(r[rb][v]), dw[rb], cw);
+                    acc[rb][v] = fmaf(g, dy[v], acc[rb][v]);
+                }
+            }
+        }
+        if (more) stage_scales(smem + nxt_sel, sc, tid);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+        const uint32_t r = row0 + rb * 32 + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t j = col0 + wave * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
+            if (!CHECK || (r < rows && j < batch)) dst[static_cast<uint64_t>(j) * stride_dst + r] = acc[rb][v];
+        }
+    }
+}
+
 template <bool CHECK, bool A16>
 int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb,
                    uint32_t batch, uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid,
@@ -241,9 +451,31 @@ int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows
             return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", kLdsBytes);
         }
         granted = true;
+#ifdef Q8MI_TRACE
+        int occ = -1;
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, gemm_d4_kernel<CHECK, A16>, kGemmThreads, kLdsBytes);
+        fprintf(stderr, "gemm_d4_kernel<%d,%d>: %d workgroups per CU\n", int(CHECK), int(A16), occ);
+#endif
     }
     gemm_d4_kernel<CHECK, A16><<<grid, kGemmThreads, kLdsBytes, stream>>>(
         w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
+    return check_launch("gemm");
+}
+
+template <bool CHECK>
+int launch_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
+               uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid, hipStream_t stream) {
+    static bool granted = false;
+    if (!granted) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_dma_kernel<CHECK>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", kLdsBytes);
+        }
+        granted = true;
+    }
+    gemm_d4_dma_kernel<CHECK><<<grid, kGemmThreads, kLdsBytes, stream>>>(w, y, dst, rows, nb, batch, stride,
+                                                                        row_tiles, col_tiles);
     return check_launch("gemm");
 }
 
@@ -259,12 +491,12 @@ int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, u
     const uint32_t nb = cols / kQK;
     const bool a16 = nb % 8 == 0;
     const auto *yb = static_cast<const uint8_t *>(y);
-    if (check) {
-        return a16 ? launch_variant<true, true>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
-                   : launch_variant<true, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
+    if (a16) {
+        return check ? launch_dma<true>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
+                     : launch_dma<false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
     }
-    return a16 ? launch_variant<false, true>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
-               : launch_variant<false, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
+    return check ? launch_variant<true, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
+                 : launch_variant<false, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
 }
 
 }  // namespace
