@@ -30,6 +30,7 @@
 // is then the correctly rounded d_w*S (12582912*d_w is exact: d_w has 11
 // significant bits), and acc = fma(g, d_y, acc): two FMAs per (output, block).
 #include <cstdio>
+#include <cstdlib>
 
 #include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
@@ -237,28 +238,37 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_kernel(
 
 
 // ---- direct-to-LDS variant (rows whose int8 plane is 16-byte aligned) ----------------------
-// Stage layout (38912 B, two stages):
-//   [0, 16384)      weight quants, 128 rows x 128 B; 16-byte piece p of row r sits in slot p ^ swz(r),
-//                   so equal pieces of 8 or 16 consecutive rows fall on distinct banks
-//   [16384, 34816)  activation records exactly as in memory (128 x 144 B: 16 B scales + 128 B quants)
-//   [34816, 36864)  weight scales as fp32, [sub-block][row]
-//   [36864, 38912)  activation scales as fp32, [sub-block][row]
+// Workgroup tile: 32*RB weight rows x 128 activation rows; RB = 4 is the main tile, RB = 1 a
+// quarter tile used for the rows left over after the last full round of main tiles (and for
+// problems too small to fill the chip with main tiles).
+// Stage layout (two stages; TR = 32*RB):
+//   weight quants      TR rows x 128 B; 16-byte piece p of row r sits in slot p ^ swz(r), so equal
+//                      pieces of 8 or 16 consecutive rows fall on distinct banks
+//   activation records exactly as in memory (128 x 144 B: 16 B scales + 128 B quants)
+//   weight scales      fp32, [sub-block][row]
+//   activation scales  fp32, [sub-block][row]
 // Quants travel global -> LDS without passing through registers (global_load_lds_dwordx4: lane l of
 // a wave writes 16 bytes at M0 + 16 l); only the scales go through registers.  All per-lane
-// offsets are constant over the K loop, the per-step bases are scalar, so staging costs ten
-// instructions per wave and step.
-constexpr int kWqBytes = kTileRows * 128;
-constexpr int kYrBytes = kTileCols * kRec;
-constexpr int kScBytes = 4 * 128 * 4;
-constexpr int kOffYr = kWqBytes, kOffWsc = kOffYr + kYrBytes, kOffYsc = kOffWsc + kScBytes;
-static_assert(kOffYsc + kScBytes == kStageBytes, "both variants use the same LDS budget");
+// offsets are constant over the K loop and the per-step bases are scalar, so staging costs about
+// ten instructions per wave and step.
+template <int RB>
+struct DmaTile {
+    static constexpr int kRows = 32 * RB;
+    static constexpr int kWq = kRows * 128;
+    static constexpr int kOffYr = kWq;
+    static constexpr int kOffWsc = kOffYr + kTileCols * kRec;
+    static constexpr int kOffYsc = kOffWsc + 4 * kRows * 4;
+    static constexpr int kStage = kOffYsc + 4 * kTileCols * 4;
+    static constexpr int kLds = 2 * kStage;
+};
+static_assert(DmaTile<4>::kStage == kStageBytes, "main tile: same LDS budget as the register-staged kernel");
 
-using gptr = const __attribute__((address_space(1))) void *;
 using lptr = __attribute__((address_space(3))) void *;
 
-// 16 bytes per lane from global memory straight into LDS at lds_wave_base + lane * 16.
-// Issued as inline assembly so that the compiler's wait-count pass does not make every later
-// LDS read wait for it; completion is awaited explicitly (vmcnt(0)) before the stage's barrier.
+// 16 bytes per lane from global memory (scalar base + 32-bit lane offset) straight into LDS at
+// lds_off + lane * 16.  Issued as inline assembly so that the compiler's wait-count pass does not
+// make every later LDS read wait for it; completion is awaited explicitly (vmcnt(0)) before the
+// barrier that publishes the stage.
 __device__ __forceinline__ void dma16(const uint8_t *uniform_base, uint32_t lane_off, uint32_t lds_off) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_off), "v"(lane_off), "s"(uniform_base) : "memory", "m0");
@@ -273,128 +283,135 @@ __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     return reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
-// slot swizzle of the weight stage: 8 (and 16) consecutive rows put equal pieces on distinct banks
 __device__ __forceinline__ uint32_t swz(uint32_t row) { return (row & 7u) ^ ((row >> 3) & 1u); }
 
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 struct Scales { v2u wd; v4i yd; };
 
 // Per-lane byte offsets that do not change over the K loop.
+template <int RB>
 struct LaneOffsets {
-    uint32_t wq[4];   // weight quant chunk i of this wave, relative to the tile's first row + quant plane
+    uint32_t wq[RB];  // weight quant chunk i of this wave, relative to the tile's first row, quant plane
     uint32_t yr;      // lane * 16
-    uint32_t sc;      // weight row (tid % 128) of the scale load
+    uint32_t sc;      // weight row of this thread's scale load, relative to the tile's first row
     uint32_t ysc;     // record (tid % 128) of the activation scale load
 };
 
-template <bool CHECK>
-__device__ __forceinline__ void stage_issue(uint32_t stage_off, Scales &sc, const LaneOffsets &lo,
+template <bool CHECK, int RB>
+__device__ __forceinline__ void stage_issue(uint32_t stage_off, Scales &sc, const LaneOffsets<RB> &lo,
                                             const uint8_t *wq_base, const uint8_t *wd_base, const uint8_t *y_base,
-                                            uint32_t y_limit, uint32_t wave, uint32_t tid) {
-    // wq_base: tile's first row, quant plane, this super-block (uniform); y_base: first record of the stage
+                                            uint32_t y_limit, uint32_t wave) {
+    using T = DmaTile<RB>;
+    // weight quants: RB chunks of 8 rows x 128 B per wave
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma16(wq_base, lo.wq[i], stage_off + (wave * 4 + i) * 1024);
+    for (int i = 0; i < RB; ++i) dma16(wq_base, lo.wq[i], stage_off + (wave * RB + i) * 1024);
+    // activation records: 18 chunks of 1 KB, contiguous in memory
 #pragma unroll
     for (int i = 0; i < 5; ++i) {
         const uint32_t c = wave + 4 * i;
         if (c < 18) {
             uint32_t off = c * 1024 + lo.yr;
             if (CHECK) off = off <= y_limit ? off : y_limit;
-            dma16(y_base, off, stage_off + kOffYr + c * 1024);
+            dma16(y_base, off, stage_off + T::kOffYr + c * 1024);
         }
     }
-    // scales through registers; every thread loads both kinds (branch-free), half of each is used
+    // scales through registers; every thread loads both kinds (branch-free), a part of each is used
     sc.wd = *(const __attribute__((address_space(1))) v2u *)(wd_base + lo.sc);
     uint32_t off = lo.ysc;
     if (CHECK) off = off <= y_limit ? off : y_limit;
     sc.yd = *(const __attribute__((address_space(1))) v4i *)(y_base + off);
-    (void)tid;
 }
 
+template <int RB>
 __device__ __forceinline__ void stage_scales(uint8_t *stage, const Scales &sc, uint32_t tid) {
-    if (tid < 128) {
-        float *wsc = reinterpret_cast<float *>(stage + kOffWsc);
-        wsc[0 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.x & 0xffffu));
-        wsc[1 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.x >> 16));
-        wsc[2 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.y & 0xffffu));
-        wsc[3 * 128 + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.y >> 16));
-    } else {
-        int *ysc = reinterpret_cast<int *>(stage + kOffYsc);
+    using T = DmaTile<RB>;
+    if (tid < T::kRows) {
+        float *wsc = reinterpret_cast<float *>(stage + T::kOffWsc);
+        wsc[0 * T::kRows + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.x & 0xffffu));
+        wsc[1 * T::kRows + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.x >> 16));
+        wsc[2 * T::kRows + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.y & 0xffffu));
+        wsc[3 * T::kRows + tid] = half_bits_to_float(static_cast<uint16_t>(sc.wd.y >> 16));
+    } else if (tid >= 128) {
+        int *ysc = reinterpret_cast<int *>(stage + T::kOffYsc);
         const uint32_t j = tid - 128;
         ysc[0 * 128 + j] = sc.yd.x; ysc[1 * 128 + j] = sc.yd.y; ysc[2 * 128 + j] = sc.yd.z; ysc[3 * 128 + j] = sc.yd.w;
     }
 }
 
-template <bool CHECK>
+template <bool CHECK, int RB>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
         const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
         uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles) {
+    using T = DmaTile<RB>;
     extern __shared__ __align__(16) uint8_t smem[];
     const uint32_t tid = threadIdx.x, lane = tid % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
+    // consecutive workgroup ids land on different XCDs: give every XCD whole row tiles and walk
+    // the column tiles of a row tile back to back, so its weights stay in that XCD's L2
     const uint32_t id = blockIdx.x, xcd = id % 8u, seq = id / 8u;
     const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
-    if (rt >= row_tiles) return;
-    const uint32_t row0 = rt * kTileRows, col0 = ct * kTileCols;
+    if (rt >= row_tiles) return;   // uniform for the workgroup
+    const uint32_t row0 = rt * T::kRows, col0 = ct * kTileCols;
     const uint32_t nsb = nb / 4;
 
     v16i seed;
 #pragma unroll
     for (int i = 0; i < 16; ++i) seed[i] = static_cast<int>(kMagicBits);
-    float acc[4][16];
+    float acc[RB][16];
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
 
     const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
-    LaneOffsets lo;
+    LaneOffsets<RB> lo;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t r = (wave * 4 + i) * 8 + lane / 8;
+    for (int i = 0; i < RB; ++i) {
+        const uint32_t r = (wave * RB + i) * 8 + lane / 8;
         uint32_t gr = r;
-        if (CHECK) gr = row0 + r < rows ? r : rows - 1 - row0;
+        if (CHECK) gr = row0 + r < rows ? r : rows - 1 - row0;   // rows past the end re-read the last row
         lo.wq[i] = gr * static_cast<uint32_t>(row_bytes) + ((lane & 7u) ^ swz(r)) * 16;
     }
     lo.yr = lane * 16;
     {
-        uint32_t gr = tid & 127u;
+        uint32_t gr = tid & (T::kRows - 1);
         if (CHECK) gr = row0 + gr < rows ? gr : rows - 1 - row0;
         lo.sc = gr * static_cast<uint32_t>(row_bytes);
         lo.ysc = (tid & 127u) * kRec;
     }
-    const uint8_t *wd_base = uniform_ptr(w + row0 * row_bytes);          // scale plane of the tile's first row
-    const uint8_t *wq_base = wd_base + 2 * nb;                            // quant plane
+    const uint8_t *wd_base = uniform_ptr(w + row0 * row_bytes);   // scale plane of the tile's first row
+    const uint8_t *wq_base = wd_base + 2 * nb;                     // its quant plane
     const uint8_t *y_base = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec);
     const uint64_t y_step = static_cast<uint64_t>(batch) * kRec;
-    // last valid 16-byte offset from y_base within the whole activation buffer (CHECK only)
+    // last 16-byte offset from y_base that is still inside the activation buffer (used when CHECK)
     uint64_t y_room = static_cast<uint64_t>(nsb) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
+    auto limit32 = [](uint64_t v) { return static_cast<uint32_t>(v < 0xffffffffull ? v : 0xffffffffull); };
     const uint32_t smem_off = lds_offset_of(smem);
 
     Scales sc;
-    stage_issue<CHECK>(smem_off, sc, lo, wq_base, wd_base, y_base,
-                       static_cast<uint32_t>(y_room < 0xffffffffull ? y_room : 0xffffffffull), wave, tid);
-    stage_scales(smem, sc, tid);
+    stage_issue<CHECK, RB>(smem_off, sc, lo, wq_base, wd_base, y_base, limit32(y_room), wave);
+    stage_scales<RB>(smem, sc, tid);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     const uint32_t fl = swz(l32);
-    const uint32_t a_off = kOffYr + (wave * 32 + l32) * kRec + 16 + lhalf * 16;
+    const uint32_t a_off = T::kOffYr + (wave * 32 + l32) * kRec + 16 + lhalf * 16;
     const uint32_t b_row = l32 * 128;
-    asm volatile("" : "+v"(seed));   // keep the seed in registers instead of rebuilding it per MFMA group
+    asm volatile("" : "+v"(seed));   // keep the seed in registers instead of rebuilding it per block
 
     for (uint32_t sb = 0; sb < nsb; ++sb) {
-        const uint32_t cur_sel = (sb & 1u) * kStageBytes, nxt_sel = kStageBytes - cur_sel;
-        uint8_t *cur = smem + cur_sel;
+        const uint32_t cur_sel = (sb & 1u) * T::kStage, nxt_sel = T::kStage - cur_sel;
+        const uint8_t *cur = smem + cur_sel;
         const bool more = sb + 1 < nsb;
         if (more) {
             wq_base += 128; wd_base += 8; y_base += y_step; y_room -= y_step;
-            stage_issue<CHECK>(smem_off + nxt_sel, sc, lo, wq_base, wd_base, y_base,
-                               static_cast<uint32_t>(y_room < 0xffffffffull ? y_room : 0xffffffffull), wave, tid);
+            stage_issue<CHECK, RB>(smem_off + nxt_sel, sc, lo, wq_base, wd_base, y_base, limit32(y_room), wave);
         }
-        const float *wsc = reinterpret_cast<const float *>(cur + kOffWsc);
-        const float *ysc = reinterpret_cast<const float *>(cur + kOffYsc);
+        const float *wsc = reinterpret_cast<const float *>(cur + T::kOffWsc);
+        const float *ysc = reinterpret_cast<const float *>(cur + T::kOffYsc);
+        // one Q8 block (K = 32) per trip; kept rolled so that only the result patches of one block
+        // are live at a time
 #pragma unroll 1
         for (uint32_t sub = 0; sub < 4; ++sub) {
             const v4i a = *reinterpret_cast<const v4i *>(cur + a_off + sub * 32);
@@ -405,16 +422,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
                 const float4 t = *reinterpret_cast<const float4 *>(ysc + sub * 128 + wave * 32 + 8 * g + 4 * lhalf);
                 dy[4 * g + 0] = t.x; dy[4 * g + 1] = t.y; dy[4 * g + 2] = t.z; dy[4 * g + 3] = t.w;
             }
-            v16i r[4];
-            float dw[4];
+            v16i r[RB];
+            float dw[RB];
 #pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
+            for (int rb = 0; rb < RB; ++rb) {
                 const v4i b = *reinterpret_cast<const v4i *>(cur + rb * 32 * 128 + b_off);
-                dw[rb] = wsc[sub * 128 + rb * 32 + l32];
+                dw[rb] = wsc[sub * T::kRows + rb * 32 + l32];
                 r[rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, seed, 0, 0, 0);
             }
 #pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
+            for (int rb = 0; rb < RB; ++rb) {
                 const float cw = -kMagic * dw[rb];
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
@@ -423,12 +440,13 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
                 }
             }
         }
-        if (more) stage_scales(smem + nxt_sel, sc, tid);
+        if (more) stage_scales<RB>(smem + nxt_sel, sc, tid);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
+    // D[i][n]: n = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (activation row)
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb) {
+    for (int rb = 0; rb < RB; ++rb) {
         const uint32_t r = row0 + rb * 32 + l32;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -462,21 +480,57 @@ int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows
     return check_launch("gemm");
 }
 
-template <bool CHECK>
+// Workgroups of each tile shape that one CU holds at a time (queried once per instantiation).
+template <bool CHECK, int RB>
 int launch_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
-               uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid, hipStream_t stream) {
+               uint32_t stride, hipStream_t stream) {
+    using T = DmaTile<RB>;
     static bool granted = false;
     if (!granted) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_dma_kernel<CHECK>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess) {
+        if (T::kLds > 64 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_dma_kernel<CHECK, RB>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, T::kLds) != hipSuccess) {
             (void)hipGetLastError();
-            return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", kLdsBytes);
+            return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", T::kLds);
         }
         granted = true;
     }
-    gemm_d4_dma_kernel<CHECK><<<grid, kGemmThreads, kLdsBytes, stream>>>(w, y, dst, rows, nb, batch, stride,
-                                                                        row_tiles, col_tiles);
+    const uint32_t row_tiles = (rows + T::kRows - 1) / T::kRows;
+    const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
+    const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
+    if (grid64 > 0x7fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    gemm_d4_dma_kernel<CHECK, RB><<<static_cast<uint32_t>(grid64), kGemmThreads, T::kLds, stream>>>(
+        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
     return check_launch("gemm");
+}
+
+template <int RB>
+int launch_dma_rows(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
+                    uint32_t stride, hipStream_t stream) {
+    const bool check = (rows % (32 * RB) != 0) || (batch % kTileCols != 0);
+    return check ? launch_dma<true, RB>(w, y, dst, rows, nb, batch, stride, stream)
+                 : launch_dma<false, RB>(w, y, dst, rows, nb, batch, stride, stream);
+}
+
+// Tile choice.  Workgroups are scheduled dynamically and a lone workgroup on a CU runs nearly
+// twice as fast as two sharing its VALUs, so a partly filled last round of main tiles costs
+// little: problems with at least 0.4 main tiles per resident slot (two per CU) use main tiles
+// throughout; smaller ones use quarter tiles, which put four times as many workgroups on the chip
+// (measured crossover on MI355X: between 160 and 256 main tiles).
+// Q8MI_GEMM_TILE (1 or 4, read only when the process runs with Q8MI_TUNE=1) overrides the choice.
+int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
+                    uint32_t stride, hipStream_t stream) {
+    const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
+    const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
+    const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
+    const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
+    int tile = tiles * 5 >= slots * 2 ? 4 : 1;
+    static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
+    if (live) {
+        if (const char *e = getenv("Q8MI_GEMM_TILE")) tile = atoi(e) == 1 ? 1 : 4;
+    }
+    return tile == 4 ? launch_dma_rows<4>(w, y, dst, rows, nb, batch, stride, stream)
+                     : launch_dma_rows<1>(w, y, dst, rows, nb, batch, stride, stream);
 }
 
 int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,
@@ -491,10 +545,7 @@ int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, u
     const uint32_t nb = cols / kQK;
     const bool a16 = nb % 8 == 0;
     const auto *yb = static_cast<const uint8_t *>(y);
-    if (a16) {
-        return check ? launch_dma<true>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
-                     : launch_dma<false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
-    }
+    if (a16) return launch_gemm_dma(w, yb, dst, rows, nb, batch, stride, stream);
     return check ? launch_variant<true, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
                  : launch_variant<false, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
 }

@@ -345,17 +345,17 @@ int run_single(const char *what, int mode, const uint8_t *w, const void *y, void
 
 }  // namespace
 
+// Shipped configuration: two workgroups per CU, interleaved units (best of the sweeps).
 GemvTuning gemv_tuning() {
     static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
     auto read = [] {
-        GemvTuning t{2, 1, 0};   // two workgroups per CU, interleaved units: best of the sweeps
+        GemvTuning t{2, 1, 0};
         if (const char *e = getenv("Q8MI_GEMV_WGS_PER_CU")) t.wgs_per_cu = atoi(e);
         if (const char *e = getenv("Q8MI_GEMV_INTERLEAVE")) t.interleave = atoi(e);
         if (const char *e = getenv("Q8MI_GEMV_THREADS")) t.threads = atoi(e);
         return t;
     };
-    static const GemvTuning fixed = read();
-    return live ? read() : fixed;
+    return live ? read() : GemvTuning{2, 1, 0};
 }
 
 // Any batch through the GEMV kernels, eight activation rows per launch.  Used by

@@ -74,6 +74,36 @@ def test_gemm_reference_shapes(gpu, oracle, rows, batch, cols):
     d4_block_dots(oracle, dw, w, dy, y, rows, cols, batch, seed=cols, n=512)
 
 
+@pytest.mark.parametrize("rows,batch,cols", [(4096, 2048, 256), (4480, 2050, 512), (9000, 1024, 256),
+                                             (17408, 2048, 128)])
+def test_gemm_large_tilings(gpu, oracle, rows, batch, cols):
+    """Shapes with at least one full round of main tiles on the chip: main tiles only, and main
+    tiles + quarter tiles for the leftover rows (ragged in rows and batch), with a padded
+    output stride."""
+    w = synth.q8_0_weight(rows, cols, seed=rows + 3 * cols)
+    x = synth.normal(batch, cols, seed=batch + 5 * cols)
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    stride = rows + 8
+    got = run_gemm(dw, dy, rows, cols, batch, stride=stride)
+    assert np.all(got[:, rows:].view(np.uint32) == 0xffffffff), "stores must stay inside the rows"
+    assert np.isfinite(got[:, :rows]).all(), "every output must be written"
+    rng = np.random.default_rng(rows + batch)
+    n = 40000
+    sr = rng.integers(0, rows, n, dtype=np.uint32)
+    sj = rng.integers(0, batch, n, dtype=np.uint32)
+    edge_rows = [0, rows - 1, rows - 33, max(rows - 129, 0), (rows // 128) * 128 - 1, (rows // 128) * 128 % rows]
+    sr[:len(edge_rows)] = edge_rows
+    sj[:len(edge_rows)] = [0, batch - 1, batch - 1, 0, batch - 1, batch // 2]
+    rc, ref_s, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, sr, sj)
+    assert_close_fp32(got[sj, sr], ref_s, absum, f"gemm {rows}x{batch}x{cols} (sampled)")
+    # all rows of two activation rows, to catch a misplaced tile anywhere along the weight rows
+    for j in (0, batch - 1):
+        rr = np.arange(rows, dtype=np.uint32)
+        rc, ref_c, absum_c = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr, np.full(rows, j, np.uint32))
+        assert_close_fp32(got[j, :rows], ref_c, absum_c, f"gemm column {j}")
+
+
 def test_gemm_reference_tolerance_restated(gpu):
     """tests/mmq_parity.cu:246-254 restated: output vs fp32 dot of the dequantised
     operands within 5e-3 abs or 1e-3 rel, U(-0.5,0.5) weights and U(-1,1) activations."""
