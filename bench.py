@@ -4,10 +4,13 @@
 One "step" = one pass over the decode GEMV set of one 27B-style layer at M=1
 (BASELINE config 1), through the C ABI exactly as the executor would drive it:
 
-    quantize_q8_1(x[5120])   -> gemv_fanout4  Q 5120x6144, K 5120x1024, V 5120x1024
-    quantize_q8_1(a[6144])   -> gemv_add      O 6144x5120   (residual add)
-    quantize_q8_1(x[5120])   -> gemv_silu_mul gate, up 5120x17408 each
-    quantize_q8_1(f[17408])  -> gemv_add      down 17408x5120
+    qgemv_fanout4(x[5120])   Q 5120x6144, K 5120x1024, V 5120x1024   (quantizer fused into the GEMV)
+    qgemv_add(a[6144])       O 6144x5120, residual add               (fused)
+    qgemv_silu_mul(x[5120])  gate, up 5120x17408 each                (fused)
+    quantize_q8_1(f[17408])  -> gemv_add   down 17408x5120           (two launches: rows above 8192 columns)
+
+which is the routing of the host layer (HipQ8Backend) at batch 1; for batch 2..8 every op is
+quantize_q8_1 + GEMV (two launches), as in the reference.
 
 `value` is algorithmic bytes per step / time per step with all inputs resident
 in HBM, cycling through several distinct copies of the layer's weights so that
@@ -79,9 +82,27 @@ class DecodeStep:
         outs = 4 * m * (QDIM + 2 * KVDIM + HIDDEN + FFN + HIDDEN)
         return layer_bytes + act + outs
 
+    @property
+    def fused(self):
+        return self.m == 1
+
+    @property
+    def launches(self):
+        return 5 if self.fused else 8
+
     def run(self, layer, stream=None):
         L, m, w = self.L, self.m, layer.w
         ok = self.ok
+        if self.fused:
+            ok(L.q8mi_qgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.x.ptr, HIDDEN,
+                                    self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
+                                    HIDDEN, m, QDIM, KVDIM, KVDIM, 0, stream), "qfanout4")
+            ok(L.q8mi_qgemv_add(w["o"].ptr, self.attn.ptr, ATTN_OUT, self.h.ptr, 0, HIDDEN, ATTN_OUT, m, HIDDEN,
+                                stream), "qo")
+            self.run_silu(layer, stream)
+            ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, m, FFN, FFN, stream), "quantize")
+            ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, m, HIDDEN, stream), "down")
+            return
         ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize")
         ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.y5120.ptr,
                                self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
@@ -94,6 +115,10 @@ class DecodeStep:
         ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, m, HIDDEN, stream), "down")
 
     def run_silu(self, layer, stream=None):
+        if self.fused:
+            self.ok(self.L.q8mi_qgemv_silu_mul(layer.w["gate"].ptr, layer.w["up"].ptr, self.x.ptr, HIDDEN,
+                                               self.ffn.ptr, FFN, HIDDEN, self.m, FFN, stream), "qsilu_mul")
+            return
         self.ok(self.L.q8mi_gemv_silu_mul(layer.w["gate"].ptr, layer.w["up"].ptr, self.y5120.ptr, self.ffn.ptr,
                                           FFN, HIDDEN, self.m, FFN, stream), "silu_mul")
 
@@ -284,12 +309,12 @@ def main():
                                "(QKV 5120x8192 fan-out, O 6144x5120 +residual, gate/up 5120x17408 SwiGLU, "
                                "down 17408x5120 +residual), Q8_0 N(0,0.02) weights, Q8_1 N(0,1) activations",
                    "weight_copies_cycled": args.copies, "bytes_per_step": step_bytes,
-                   "launches_per_step": 8},
+                   "launches_per_step": step.launches},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "resident_gbps": round(step_bytes / (ms_resident * 1e-3) / 1e9, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(),
-                     "kernel": "gemv_kernel<1, 256, 0, true> (SwiGLU: gate+up 2 x 5120x17408)",
+                     "kernel": "gemv_kernel<1, 256, 2, true> (SwiGLU with fused quantizer: gate+up 2 x 5120x17408)",
                      "bytes_per_launch": silu_bytes, "launch_ms": round(back_ms, 5),
                      "launch_ms_mean": round(mean_ms, 5),
                      "launch_ms_median": round(med_ms, 5), "launch_ms_min": round(min_ms, 5),

@@ -30,7 +30,9 @@ struct GemvParams {
     void *dst[4];
     uint32_t row_end[4];  // cumulative row counts of the concatenated row space
     uint32_t stride[4];
-    const uint8_t *y;     // Q8_1 blocks, [batch][nb]
+    const uint8_t *y;     // Q8_1 blocks, [batch][nb] (null when xf is set)
+    const float *xf;      // fp32 activations to be quantized while staging (fused entry points)
+    uint32_t x_stride;    // floats between rows of xf
     uint32_t total_rows;  // rows of the concatenated space (SwiGLU: rows of one weight)
     uint32_t units;
     uint32_t nb;
@@ -88,8 +90,8 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
 #ifdef Q8MI_TRACE
     const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
 #endif
-    uint32_t ufirst, ucount, ustride;
-    group_units(p.units, blockIdx.x, gridDim.x, p.interleave, ufirst, ucount, ustride);
+    const UnitSeq useq = group_units(p.units, blockIdx.x, gridDim.x, p.interleave);
+    const uint32_t ucount = useq.count;
     const uint32_t n_items = ucount * nsteps;
     uint32_t i0, i1;
     wave_items(n_items, wave, kWaves, i0, i1);
@@ -119,7 +121,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
     auto park = [&](uint32_t kk, float total) {
         if (lane < kPerUnit) my_park[kk * kPerUnit + lane] = total;
     };
-    gemv_stream<M, R, THREADS, XMODE>(smem, p.y, p.nb, ufirst, ustride, i0, i1, rows_of, park);
+    gemv_stream<M, R, THREADS, XMODE>(smem, p.y, p.xf, p.x_stride, p.nb, useq, i0, i1, rows_of, park);
 #ifdef Q8MI_TRACE
     const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
 #endif
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
         constexpr uint32_t kHalf = R / 2;
         for (uint32_t e = threadIdx.x; e < ucount * M * kHalf; e += THREADS) {
             const uint32_t k = e / (M * kHalf), m = (e / kHalf) % M, r = e % kHalf;
-            const uint32_t row = kHalf * (ufirst + k * ustride) + r;
+            const uint32_t row = kHalf * useq.unit(k) + r;
             if (row >= p.total_rows) continue;
             const float g = total_of(k, m * R + r);
             const float up = total_of(k, m * R + kHalf + r);
@@ -159,7 +161,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
         for (uint32_t e = threadIdx.x; e < ucount * kPerUnit; e += THREADS) {
             const uint32_t k = e / kPerUnit, mr = e % kPerUnit;
             const uint32_t m = mr / R, r = mr % R;
-            const uint32_t row = R * (ufirst + k * ustride) + r;
+            const uint32_t row = R * useq.unit(k) + r;
             if (row >= p.total_rows) continue;
             const RowRef ref = resolve_row(p, row);
             store_out(p.mode, ref.dst, static_cast<uint64_t>(m) * ref.stride + ref.local, total_of(k, mr));
@@ -276,6 +278,11 @@ int launch_ms(const GemvParams &p, hipStream_t stream) {
     const uint32_t xb = x_lds_bytes(p.nb, M);
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
     const int forced = gemv_tuning().threads;
+    if (p.xf != nullptr) {   // fused quantizer: the activations must fit LDS
+        if (xb + park_256 <= 76u * 1024u && forced != 1024) return launch_inst<M, 256, kXF32, SILU>(p, xb, stream);
+        if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXF32, SILU>(p, xb, stream);
+        return fail(Q8MI_REJECTED, "qgemv: %u activation rows of %u columns do not fit LDS", M, p.nb * 32);
+    }
     if (forced == 256 && xb + park_256 <= kLdsLimit) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);
     if (forced == 1024 && xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds, SILU>(p, xb, stream);
     if (xb + park_256 <= 76u * 1024u) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);   // two per CU fit
@@ -290,6 +297,7 @@ int launch_m(const GemvParams &p, hipStream_t stream) {
 
 int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
     if (p.nb % 8 != 0) {
+        if (p.xf != nullptr) return fail(Q8MI_REJECTED, "qgemv: cols %u not a multiple of 256", p.nb * 32);
         const uint32_t cus = static_cast<uint32_t>(device_cu_count());
         uint32_t grid = cus * 8;
         const uint32_t max_wgs = (p.total_rows + 3) / 4;
@@ -319,14 +327,23 @@ int shape_gate(const char *what, uint32_t cols, uint32_t batch) {
 
 bool planes_aligned(const void *w) { return reinterpret_cast<uintptr_t>(w) % 16 == 0; }
 
-GemvParams single(const uint8_t *w, const void *y, void *dst, uint32_t rows, uint32_t cols,
+// Activations of a call: Q8_1 blocks, or fp32 rows for the entry points that quantize in the kernel.
+struct XSource {
+    const void *y_q8_1;
+    const float *xf;
+    uint32_t stride_x;
+};
+
+GemvParams single(const uint8_t *w, const XSource &x, void *dst, uint32_t rows, uint32_t cols,
                   uint32_t stride, int mode) {
     GemvParams p{};
     p.w[0] = w;
     p.dst[0] = dst;
     p.stride[0] = stride;
     for (int i = 0; i < 4; ++i) p.row_end[i] = rows;
-    p.y = static_cast<const uint8_t *>(y);
+    p.y = static_cast<const uint8_t *>(x.y_q8_1);
+    p.xf = x.xf;
+    p.x_stride = x.stride_x;
     p.total_rows = rows;
     p.units = 0;   // set per batch size at launch
     p.nb = cols / kQK;
@@ -334,7 +351,7 @@ GemvParams single(const uint8_t *w, const void *y, void *dst, uint32_t rows, uin
     return p;
 }
 
-int run_single(const char *what, int mode, const uint8_t *w, const void *y, void *dst, uint32_t rows,
+int run_single(const char *what, int mode, const uint8_t *w, const XSource &y, void *dst, uint32_t rows,
                uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
     if (int rc = shape_gate(what, cols, batch)) return rc;
     if (rows == 0 || cols == 0) return Q8MI_OK;
@@ -366,7 +383,7 @@ int gemv_any_batch(const uint8_t *w, const void *y_q8_1, float *dst, uint32_t ro
     const auto *y = static_cast<const uint8_t *>(y_q8_1);
     for (uint32_t j0 = 0; j0 < batch; j0 += Q8MI_MAX_GEMV_BATCH) {
         const uint32_t m = batch - j0 < Q8MI_MAX_GEMV_BATCH ? batch - j0 : Q8MI_MAX_GEMV_BATCH;
-        const GemvParams p = single(w, y + static_cast<uint64_t>(j0) * nb * kQ81Bytes,
+        const GemvParams p = single(w, XSource{y + static_cast<uint64_t>(j0) * nb * kQ81Bytes, nullptr, 0},
                                     dst + static_cast<uint64_t>(j0) * stride_dst_row, rows, cols,
                                     stride_dst_row, kStoreF32);
         if (int rc = launch_any(p, m, stream)) return rc;
@@ -380,27 +397,26 @@ using namespace q8mi;
 
 extern "C" int q8mi_gemv(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,
                          uint32_t batch, uint32_t stride, void *stream) {
-    return run_single("gemv", kStoreF32, w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv", kStoreF32, w, XSource{y, nullptr, 0}, dst, rows, cols, batch, stride, stream);
 }
 
 extern "C" int q8mi_gemv_bf16(const uint8_t *w, const void *y, uint16_t *dst, uint32_t rows,
                               uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
-    return run_single("gemv_bf16", kStoreBF16, w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv_bf16", kStoreBF16, w, XSource{y, nullptr, 0}, dst, rows, cols, batch, stride, stream);
 }
 
 extern "C" int q8mi_gemv_add(const uint8_t *w, const void *y, float *dst, uint32_t rows,
                              uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
-    return run_single("gemv_add", kAddF32, w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv_add", kAddF32, w, XSource{y, nullptr, 0}, dst, rows, cols, batch, stride, stream);
 }
 
 extern "C" int q8mi_gemv_add_bf16(const uint8_t *w, const void *y, uint16_t *dst, uint32_t rows,
                                   uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
-    return run_single("gemv_add_bf16", kAddBF16, w, y, dst, rows, cols, batch, stride, stream);
+    return run_single("gemv_add_bf16", kAddBF16, w, XSource{y, nullptr, 0}, dst, rows, cols, batch, stride, stream);
 }
 
-extern "C" int q8mi_gemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const void *y, float *dst,
-                                  uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride,
-                                  void *stream) {
+static int run_silu_mul(const uint8_t *wg, const uint8_t *wu, const XSource &y, float *dst, uint32_t rows,
+                        uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
     if (int rc = shape_gate("gemv_silu_mul", cols, batch)) return rc;
     if (rows == 0 || cols == 0) return Q8MI_OK;
     if (!planes_aligned(wg) || !planes_aligned(wu))
@@ -410,11 +426,16 @@ extern "C" int q8mi_gemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const vo
     return launch_any(p, batch, as_stream(stream));
 }
 
-extern "C" int q8mi_gemv_fanout4(const uint8_t *w0, const uint8_t *w1, const uint8_t *w2,
-                                 const uint8_t *w3, const void *y, float *d0, float *d1, float *d2,
-                                 float *d3, uint32_t rows0, uint32_t rows1, uint32_t rows2,
-                                 uint32_t rows3, uint32_t cols, uint32_t batch, uint32_t s0,
-                                 uint32_t s1, uint32_t s2, uint32_t s3, void *stream) {
+extern "C" int q8mi_gemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const void *y, float *dst,
+                                  uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride,
+                                  void *stream) {
+    return run_silu_mul(wg, wu, XSource{y, nullptr, 0}, dst, rows, cols, batch, stride, stream);
+}
+
+static int run_fanout4(const uint8_t *w0, const uint8_t *w1, const uint8_t *w2, const uint8_t *w3,
+                       const XSource &y, float *d0, float *d1, float *d2, float *d3, uint32_t rows0,
+                       uint32_t rows1, uint32_t rows2, uint32_t rows3, uint32_t cols, uint32_t batch, uint32_t s0,
+                       uint32_t s1, uint32_t s2, uint32_t s3, void *stream) {
     if (int rc = shape_gate("gemv_fanout4", cols, batch)) return rc;
     const uint64_t declared = static_cast<uint64_t>(rows0) + rows1 + rows2 + rows3;
     if (declared == 0 || declared > 0xffffffffull)
@@ -445,12 +466,50 @@ extern "C" int q8mi_gemv_fanout4(const uint8_t *w0, const uint8_t *w1, const uin
         p.dst[i] = p.dst[n - 1];
         p.stride[i] = p.stride[n - 1];
     }
-    p.y = static_cast<const uint8_t *>(y);
+    p.y = static_cast<const uint8_t *>(y.y_q8_1);
+    p.xf = y.xf;
+    p.x_stride = y.stride_x;
     p.total_rows = total;
     p.units = 0;
     p.nb = cols / kQK;
     p.mode = kStoreF32;
     return launch_any(p, batch, as_stream(stream));
+}
+
+extern "C" int q8mi_gemv_fanout4(const uint8_t *w0, const uint8_t *w1, const uint8_t *w2,
+                                 const uint8_t *w3, const void *y, float *d0, float *d1, float *d2,
+                                 float *d3, uint32_t rows0, uint32_t rows1, uint32_t rows2,
+                                 uint32_t rows3, uint32_t cols, uint32_t batch, uint32_t s0,
+                                 uint32_t s1, uint32_t s2, uint32_t s3, void *stream) {
+    return run_fanout4(w0, w1, w2, w3, XSource{y, nullptr, 0}, d0, d1, d2, d3, rows0, rows1, rows2, rows3, cols,
+                       batch, s0, s1, s2, s3, stream);
+}
+
+// ---- entry points that quantize the activations inside the GEMV ------------------------------
+extern "C" int q8mi_qgemv(const uint8_t *w, const float *x, uint32_t stride_x_row, void *dst, int dst_is_bf16,
+                          uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
+    return run_single("qgemv", dst_is_bf16 ? kStoreBF16 : kStoreF32, w, XSource{nullptr, x, stride_x_row}, dst, rows,
+                      cols, batch, stride, stream);
+}
+
+extern "C" int q8mi_qgemv_add(const uint8_t *w, const float *x, uint32_t stride_x_row, void *dst, int dst_is_bf16,
+                              uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride, void *stream) {
+    return run_single("qgemv_add", dst_is_bf16 ? kAddBF16 : kAddF32, w, XSource{nullptr, x, stride_x_row}, dst, rows,
+                      cols, batch, stride, stream);
+}
+
+extern "C" int q8mi_qgemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const float *x, uint32_t stride_x_row,
+                                   float *dst, uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride,
+                                   void *stream) {
+    return run_silu_mul(wg, wu, XSource{nullptr, x, stride_x_row}, dst, rows, cols, batch, stride, stream);
+}
+
+extern "C" int q8mi_qgemv_fanout4(const uint8_t *w0, const uint8_t *w1, const uint8_t *w2, const uint8_t *w3,
+                                  const float *x, uint32_t stride_x_row, float *d0, float *d1, float *d2, float *d3,
+                                  uint32_t rows0, uint32_t rows1, uint32_t rows2, uint32_t rows3, uint32_t cols,
+                                  uint32_t batch, uint32_t s0, uint32_t s1, uint32_t s2, uint32_t s3, void *stream) {
+    return run_fanout4(w0, w1, w2, w3, XSource{nullptr, x, stride_x_row}, d0, d1, d2, d3, rows0, rows1, rows2, rows3,
+                       cols, batch, s0, s1, s2, s3, stream);
 }
 
 extern "C" int q8mi_gemv_two(const uint8_t *w0, const uint8_t *w1, const void *y, float *dst0,

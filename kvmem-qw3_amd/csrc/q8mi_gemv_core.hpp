@@ -27,6 +27,7 @@
 
 #include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
+#include "q8mi_quantize_core.hpp"
 
 namespace q8mi {
 
@@ -44,7 +45,9 @@ constexpr int kDepth = Q8MI_GEMV_DEPTH;        // items in flight per wave
 constexpr uint32_t kLdsLimit = 160u * 1024u;    // LDS per CU on gfx950
 constexpr uint32_t kParkFloats = 1024;           // per-wave LDS area (floats) for the sums of the units it touched
 
-enum XMode : int { kXLds = 0, kXGlobal = 1 };
+// Where a lane finds the activations: Q8_1 blocks staged in LDS, Q8_1 blocks read from
+// global memory, or fp32 activations quantized to Q8_1 while they are staged in LDS.
+enum XMode : int { kXLds = 0, kXGlobal = 1, kXF32 = 2 };
 
 // LDS footprint of `batch` activation rows: per 64-block step 128 16-byte
 // pieces of int8 and 64 fp32 scales, zero-padded to whole steps.
@@ -126,6 +129,61 @@ __device__ __forceinline__ void stage_x_lds(uint8_t *smem, const uint8_t *__rest
     __syncthreads();
 }
 
+// Same LDS image as stage_x_lds, produced from fp32 activations: every workgroup quantizes
+// the M rows itself (M * cols / 4 float4 loads spread over the workgroup), with the code the
+// stand-alone quantizer uses, so the int8 values and the fp16-rounded scales are the same bits.
+// The block sum `s` of Q8_1 is not needed by Q8_0 dots and is not formed.  x rows are
+// stride_x floats apart; cols = 32 * nb.  Ends with a workgroup barrier.
+template <int M, int THREADS>
+__device__ __forceinline__ void stage_x_f32(uint8_t *smem, const float *__restrict__ x, uint32_t stride_x,
+                                            uint32_t nb) {
+    constexpr int kBatch = 6;   // float4 loads in flight per thread: one trip for a 6144-column row at 256 threads
+    const uint32_t nsteps = (nb * 2 + 127) / 128;
+    uint32_t *wq = reinterpret_cast<uint32_t *>(smem);
+    float *wd = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
+    const uint32_t blocks_padded = nsteps * 64;
+    const uint32_t per_row = nb * 8;                        // float4 chunks per activation row
+    const uint32_t total = static_cast<uint32_t>(M) * per_row;   // multiple of 8: lanes of a block stay together
+    const bool vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride_x % 4 == 0);
+    for (uint32_t base = 0; base < total; base += THREADS * kBatch) {
+        Float4 v[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t c = base + u * THREADS + threadIdx.x;
+            const uint32_t cc = c < total ? c : 0;
+            const float *src = x + static_cast<uint64_t>(cc / per_row) * stride_x + (cc % per_row) * 4;
+            v[u] = vec ? load4<true>(src) : load4<false>(src);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t c = base + u * THREADS + threadIdx.x;
+            float d;
+            const uint32_t packed = quantize4_q8_1(v[u], d);   // all lanes take part in the exchanges
+            if (c < total) {
+                const uint32_t m = c / per_row, within = c % per_row;
+                const uint32_t blk = m * blocks_padded + within / 8;
+                wq[blk * 8 + within % 8] = packed;
+                if (within % 8 == 0) wd[blk] = half_bits_to_float(float_to_half_bits(d));
+            }
+        }
+    }
+    const uint32_t pad = blocks_padded - nb;
+    for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(M) * pad * 9; i += THREADS) {
+        const uint32_t b = i / 9, part = i % 9;
+        const uint32_t blk = (b / pad) * blocks_padded + nb + b % pad;
+        if (part == 0) wd[blk] = 0.0f; else wq[blk * 8 + (part - 1)] = 0u;
+    }
+    __syncthreads();
+}
+
+// Activations of the workgroup into LDS, by mode (no-op when lanes read them from global memory).
+template <int M, int THREADS, int XMODE>
+__device__ __forceinline__ void stage_x(uint8_t *smem, const uint8_t *__restrict__ y, const float *__restrict__ xf,
+                                        uint32_t stride_x, uint32_t nb) {
+    if (XMODE == kXLds) stage_x_lds<M, THREADS>(smem, y, nb);
+    if (XMODE == kXF32) stage_x_f32<M, THREADS>(smem, xf, stride_x, nb);
+}
+
 // Weight bytes of one item held by a lane.
 template <int R>
 struct Item {
@@ -172,7 +230,7 @@ __device__ __forceinline__ XOperand load_x(uint32_t m, uint32_t p1, uint32_t p2,
     o.x1 = v4i{0, 0, 0, 0};
     o.x2 = v4i{0, 0, 0, 0};
     o.dx = 0.0f;
-    if (XMODE == kXLds) {
+    if (XMODE != kXGlobal) {
         // LDS is zero-padded to whole steps, so no guards: pieces past the row's end
         // multiply the re-read weight bytes by zero
         o.x1 = *reinterpret_cast<const v4i *>(lds_q + (m * nsteps * 128 + p1) * 4);
@@ -229,8 +287,31 @@ __device__ __forceinline__ void compute_item(const Item<R> &it, uint32_t step, u
     }
 }
 
-// Streams the items [i0, i1) of a workgroup's unit sequence unit(k) = ufirst +
-// k * ustride; item i is step i % nsteps of unit(i / nsteps).  A wave's range may
+// A workgroup's share of the units, in the order it streams them: either a contiguous,
+// balanced slice (interleave == 0) or every ngroups-th unit starting at the workgroup's
+// index (interleave != 0; neighbouring workgroups then read neighbouring rows).
+struct UnitSeq {
+    uint32_t first, stride, count;
+    __device__ __forceinline__ uint32_t unit(uint32_t k) const { return first + k * stride; }
+};
+
+__device__ __forceinline__ UnitSeq group_units(uint32_t units, uint32_t group, uint32_t ngroups, int interleave) {
+    UnitSeq s;
+    if (interleave) {
+        s.first = group;
+        s.stride = ngroups;
+        s.count = group < units ? (units - group + ngroups - 1) / ngroups : 0;
+    } else {
+        s.first = static_cast<uint32_t>(static_cast<uint64_t>(units) * group / ngroups);
+        const uint32_t end = static_cast<uint32_t>(static_cast<uint64_t>(units) * (group + 1) / ngroups);
+        s.count = end - s.first;
+        s.stride = 1;
+    }
+    return s;
+}
+
+// Streams the items [i0, i1) of a workgroup's unit sequence useq.unit(k); item i is
+// step i % nsteps of unit(i / nsteps).  A wave's range may
 // begin or end in the middle of a unit, so what it hands to `park` is a PARTIAL
 // sum over the steps it covered; the caller combines the partials of all waves
 // after a barrier.
@@ -248,15 +329,16 @@ __device__ __forceinline__ void compute_item(const Item<R> &it, uint32_t step, u
 // the last item and whose sums are never parked.
 // Must be called by every wave of the workgroup (it contains the staging barrier).
 template <int M, int R, int THREADS, int XMODE, class RowsOf, class Park>
-__device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb,
-                                            uint32_t ufirst, uint32_t ustride, uint32_t i0, uint32_t i1,
+__device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__restrict__ y,
+                                            const float *__restrict__ xf, uint32_t stride_x, uint32_t nb,
+                                            const UnitSeq &useq, uint32_t i0, uint32_t i1,
                                             RowsOf rows_of, Park park) {
     const uint32_t nsteps = (nb * 2 + 127) / 128;
     const uint32_t lane = threadIdx.x % kWave;
     const int *lds_q = reinterpret_cast<const int *>(smem);
     const float *lds_d = reinterpret_cast<const float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
     if (i1 <= i0) {   // wave-uniform; idle waves still take part in the staging barrier
-        if (XMODE == kXLds) stage_x_lds<M, THREADS>(smem, y, nb);
+        stage_x<M, THREADS, XMODE>(smem, y, xf, stride_x, nb);
         return;
     }
     const uint32_t n_items = i1 - i0;
@@ -267,14 +349,14 @@ __device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__rest
     // issue cursor: unit ordinal, step, items left to issue for real
     uint32_t ik = k0, istep = s0, ileft = n_items;
     RowPtrs<R> irows;
-    rows_of(ufirst + ik * ustride, irows);
+    rows_of(useq.unit(ik), irows);
     auto advance_issue = [&]() {
         if (ileft > 1) {       // otherwise: keep re-reading the last real item
             --ileft;
             if (++istep == nsteps) {
                 istep = 0;
                 ++ik;
-                rows_of(ufirst + ik * ustride, irows);
+                rows_of(useq.unit(ik), irows);
             }
         }
     };
@@ -283,7 +365,7 @@ __device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__rest
         issue_item(items[d], irows, istep, lane, nb);
         advance_issue();
     }
-    if (XMODE == kXLds) stage_x_lds<M, THREADS>(smem, y, nb);
+    stage_x<M, THREADS, XMODE>(smem, y, xf, stride_x, nb);
 
     float acc[M][R];
 #pragma unroll
@@ -318,23 +400,6 @@ __device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__rest
             issue_item(items[d], irows, istep, lane, nb);
             advance_issue();
         }
-    }
-}
-
-// A workgroup's share of the units: either a contiguous, balanced slice
-// (interleave == 0) or every ngroups-th unit starting at the workgroup's index
-// (interleave != 0; neighbouring workgroups then read neighbouring rows).
-__device__ __forceinline__ void group_units(uint32_t units, uint32_t group, uint32_t ngroups, int interleave,
-                                            uint32_t &first, uint32_t &count, uint32_t &stride) {
-    if (interleave) {
-        first = group;
-        stride = ngroups;
-        count = group < units ? (units - group + ngroups - 1) / ngroups : 0;
-    } else {
-        first = static_cast<uint32_t>(static_cast<uint64_t>(units) * group / ngroups);
-        const uint32_t end = static_cast<uint32_t>(static_cast<uint64_t>(units) * (group + 1) / ngroups);
-        count = end - first;
-        stride = 1;
     }
 }
 

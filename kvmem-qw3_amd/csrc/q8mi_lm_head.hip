@@ -47,8 +47,8 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
     const uint32_t nsteps = (nb * 2 + 127) / 128;
     const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
     const uint32_t units = (rows + R - 1) / R;
-    uint32_t ufirst, ucount, ustride;
-    group_units(units, blockIdx.x, gridDim.x, interleave, ufirst, ucount, ustride);
+    const UnitSeq useq = group_units(units, blockIdx.x, gridDim.x, interleave);
+    const uint32_t ucount = useq.count;
     const uint32_t n_items = ucount * nsteps;
     uint32_t i0, i1;
     wave_items(n_items, wave, kWaves, i0, i1);
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
     auto park = [&](uint32_t kk, float total) {
         if (lane < kPerUnit) my_park[kk * kPerUnit + lane] = total;
     };
-    gemv_stream<M, R, THREADS, XMODE>(smem, y, nb, ufirst, ustride, i0, i1, rows_of, park);
+    gemv_stream<M, R, THREADS, XMODE>(smem, y, nullptr, 0, nb, useq, i0, i1, rows_of, park);
     __syncthreads();
 
     auto total_of = [&](uint32_t k, uint32_t mr) {
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
         int bi = -1;
         for (uint32_t e = threadIdx.x; e < ucount * R; e += THREADS) {
             const uint32_t k = e / R, r = e % R;
-            const uint32_t row = R * (ufirst + k * ustride) + r;
+            const uint32_t row = R * useq.unit(k) + r;
             if (row >= rows) continue;
             const float s = total_of(k, m * R + r);
             if (beats(s, static_cast<int>(row), bv, bi)) { bv = s; bi = static_cast<int>(row); }

@@ -9,47 +9,14 @@
 // so the fp16 `s` field is bit-identical to the one its 32-lane xor butterfly
 // produces: lane exchanges xor 4, 2, 1 cover the first three levels, the last
 // two are the in-lane adds (c0+c2, c1+c3) and (e0+e1).
-#include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
+#include "q8mi_quantize_core.hpp"
 
 namespace q8mi {
 namespace {
 
 constexpr int kQuantThreads = 256;
 constexpr int kElemsPerLane = 4;
-
-struct Float4 {
-    float x, y, z, w;
-};
-
-template <bool VEC>
-__device__ __forceinline__ Float4 load4(const float *p) {
-    Float4 v;
-    if (VEC) {
-        const float4 t = *reinterpret_cast<const float4 *>(p);
-        v.x = t.x; v.y = t.y; v.z = t.z; v.w = t.w;
-    } else {
-        v.x = p[0]; v.y = p[1]; v.z = p[2]; v.w = p[3];
-    }
-    return v;
-}
-
-__device__ __forceinline__ float group8_amax(const Float4 &v) {
-    float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    m = fmaxf(m, swizzle_xor4(m));
-    m = fmaxf(m, dpp_f32<kDppXor2>(m));
-    m = fmaxf(m, dpp_f32<kDppXor1>(m));
-    return m;
-}
-
-// __float2int_rn semantics: nearest-even, NaN -> 0 (v_cvt_i32_f32 saturates and
-// maps NaN to 0; rintf first so the conversion itself is exact).
-__device__ __forceinline__ int rn_int(float v) { return static_cast<int>(rintf(v)); }
-
-__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
-    return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
-           ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
-}
 
 template <bool VEC>
 __global__ __launch_bounds__(kQuantThreads) void quantize_q8_1_kernel(
@@ -60,7 +27,8 @@ __global__ __launch_bounds__(kQuantThreads) void quantize_q8_1_kernel(
     const uint32_t j = blockIdx.y;
     const Float4 v = load4<VEC>(x + static_cast<uint64_t>(j) * stride_x_row + i0);
 
-    const float amax = group8_amax(v);
+    float d;
+    const uint32_t packed = quantize4_q8_1(v, d);
 
     // level 1..3 of the reference tree across lanes, component-wise
     float s0 = v.x, s1 = v.y, s2 = v.z, s3 = v.w;
@@ -72,16 +40,11 @@ __global__ __launch_bounds__(kQuantThreads) void quantize_q8_1_kernel(
     // level 4 and 5 inside the lane
     const float sum = (s0 + s2) + (s1 + s3);
 
-    const float d = amax / 127.0f;
-    int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
-    if (amax != 0.0f) {
-        q0 = rn_int(v.x / d); q1 = rn_int(v.y / d); q2 = rn_int(v.z / d); q3 = rn_int(v.w / d);
-    }
     const uint32_t kb = i0 / kQK;
     const uint32_t sub = (i0 % kQK) / kElemsPerLane;  // 0..7
     uint32_t *blk = reinterpret_cast<uint32_t *>(
         y + (static_cast<uint64_t>(j) * nb + kb) * kQ81Bytes);
-    blk[1 + sub] = pack4(q0, q1, q2, q3);
+    blk[1 + sub] = packed;
     if (sub == 0) {
         blk[0] = static_cast<uint32_t>(float_to_half_bits(d)) |
                  (static_cast<uint32_t>(float_to_half_bits(sum)) << 16);

@@ -10,6 +10,8 @@
 //     uses the GEMV.  Here all batch <= 8 routes agree.
 //   * q8_0_matvec_fanout fuses up to four weights into one launch at batch 1
 //     (the reference pairs only same-shape neighbours, :11261-11290).
+//   * batch-1 ops on rows of at most 8192 columns run as one launch that quantizes the
+//     activations inside the GEMV; the outputs are the same bits as the two-step form.
 //   * strided batch > 8 (in_stride != cols or out_stride != rows), which the
 //     reference serves with a legacy kernel outside this path, runs as GEMV
 //     slices of eight rows.
@@ -213,6 +215,10 @@ DeviceStatus HipQ8Backend::quantize_q8_1(const float *x, uint32_t batch, uint32_
     return {};
 }
 
+// Batch-1 ops on rows of at most 8192 columns quantize inside the GEMV (one launch instead of
+// two, same bits); longer rows and batches above 1 are faster with the stand-alone quantizer.
+static bool fuse_quantizer(uint32_t batch, uint32_t cols) { return batch == 1 && cols % 256 == 0 && cols <= 8192; }
+
 // dispatch_q8_matvec, src/kernels_cuda.cu:14617-14658: any batch as GEMV slices of <= 8 rows
 DeviceStatus HipQ8Backend::gemv_route(float *out, const DeviceWeight &weight, const float *x, uint32_t batch,
                                       uint32_t in_stride, uint32_t out_stride) {
@@ -220,6 +226,9 @@ DeviceStatus HipQ8Backend::gemv_route(float *out, const DeviceWeight &weight, co
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
     const uint32_t xs = (batch == 1 && in_stride == 0) ? cols : in_stride;
     const uint32_t os = (batch == 1 && out_stride == 0) ? rows : out_stride;
+    if (fuse_quantizer(batch, cols) &&
+        q8mi_qgemv(w.ptr, x, xs, out, 0, rows, cols, 1, os, stream_) == Q8MI_OK)
+        return launch_status("hip q8_0_matvec fused");
     for (uint32_t j0 = 0; j0 < batch; j0 += 8) {
         const uint32_t m = batch - j0 < 8 ? batch - j0 : 8;
         if (auto st = quantize_q8_1(x + static_cast<uint64_t>(j0) * xs, m, cols, xs); !st.ok) return st;
@@ -238,6 +247,9 @@ DeviceStatus HipQ8Backend::q8_0_matvec(DeviceTensor &out, const DeviceWeight &we
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "q8_0_matvec: weight is not Q8_0"};
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
     if (o.is_bf16()) {
+        if (fuse_quantizer(1, cols) &&
+            q8mi_qgemv(w.ptr, T(x).f32(), cols, o.bf16(), 1, rows, cols, 1, rows, stream_) == Q8MI_OK)
+            return launch_status("hip q8_0_matvec bf16 fused");
         if (auto st = quantize_q8_1(T(x).f32(), 1, cols, cols); !st.ok) return st;
         if (!ported::launch_mmvq_q8_0_bf16(w.ptr, q8_1_.ptr, o.bf16(), rows, cols, 1, rows, stream_))
             return failed("mmvq_q8_0_bf16");
@@ -252,6 +264,9 @@ DeviceStatus HipQ8Backend::q8_0_matvec_add(DeviceTensor &accum, const DeviceWeig
     auto &o = T(accum);
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "q8_0_matvec_add: weight is not Q8_0"};
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
+    if (fuse_quantizer(1, cols) &&
+        q8mi_qgemv_add(w.ptr, T(x).f32(), cols, o.ptr, o.is_bf16() ? 1 : 0, rows, cols, 1, rows, stream_) == Q8MI_OK)
+        return launch_status("hip q8_0_matvec_add fused");
     if (auto st = quantize_q8_1(T(x).f32(), 1, cols, cols); !st.ok) return st;
     const bool ok = o.is_bf16()
         ? ported::launch_mmvq_q8_0_add_bf16(w.ptr, q8_1_.ptr, o.bf16(), rows, cols, 1, rows, stream_)
@@ -269,6 +284,9 @@ DeviceStatus HipQ8Backend::q8_0_matvec_silu_mul(DeviceTensor &out, const DeviceW
     if (g.rows != u.rows || g.cols != u.cols) return {false, "q8_0_matvec_silu_mul: gate/up shapes differ"};
     if (T(out).is_bf16()) return {false, "q8_0_matvec_silu_mul: bf16 output not supported"};
     const uint32_t cols = static_cast<uint32_t>(g.cols), rows = static_cast<uint32_t>(g.rows);
+    if (fuse_quantizer(1, cols) &&
+        q8mi_qgemv_silu_mul(g.ptr, u.ptr, T(x).f32(), cols, T(out).f32(), rows, cols, 1, rows, stream_) == Q8MI_OK)
+        return launch_status("hip q8_0_matvec_silu_mul fused");
     if (auto st = quantize_q8_1(T(x).f32(), 1, cols, cols); !st.ok) return st;
     if (!ported::launch_mmvq_q8_0_silu_mul(g.ptr, u.ptr, q8_1_.ptr, T(out).f32(), rows, cols, 1, rows, stream_))
         return failed("mmvq_q8_0_silu_mul");
@@ -344,7 +362,10 @@ DeviceStatus HipQ8Backend::q8_0_matmul_fanout(DeviceTensor *const *outs, const D
         }
         return {};
     }
-    if (auto st = quantize_q8_1(T(x).f32(), batch, cols, in_stride); !st.ok) return st;
+    const bool fused = fuse_quantizer(batch, cols);
+    if (!fused) {
+        if (auto st = quantize_q8_1(T(x).f32(), batch, cols, in_stride); !st.ok) return st;
+    }
     for (uint32_t i0 = 0; i0 < n; i0 += 4) {
         const uint8_t *wp[4] = {nullptr, nullptr, nullptr, nullptr};
         float *op[4] = {nullptr, nullptr, nullptr, nullptr};
@@ -354,6 +375,12 @@ DeviceStatus HipQ8Backend::q8_0_matmul_fanout(DeviceTensor *const *outs, const D
             op[i - i0] = T(*outs[i]).f32();
             r[i - i0] = static_cast<uint32_t>(W(*weights[i]).rows);
             s[i - i0] = out_strides[i];
+        }
+        if (fused) {
+            if (q8mi_qgemv_fanout4(wp[0], wp[1], wp[2], wp[3], T(x).f32(), in_stride, op[0], op[1], op[2], op[3], r[0],
+                                   r[1], r[2], r[3], cols, batch, s[0], s[1], s[2], s[3], stream_) != Q8MI_OK)
+                return failed("qgemv_fanout4");
+            continue;
         }
         if (!ported::launch_mmvq_q8_0_fanout4_batch(wp[0], wp[1], wp[2], wp[3], q8_1_.ptr, op[0], op[1], op[2], op[3],
                                                     r[0], r[1], r[2], r[3], cols, batch, s[0], s[1], s[2], s[3],

@@ -58,6 +58,11 @@ SIGNATURES = {
     "q8mi_repack_q8_0_split_host": (_int, [_vp, _u64, _u64, _vp]),
     "q8mi_repack_q8_0_split": (_int, [_vp, _u64, _u64, _vp, _vp]),
     "q8mi_probe_read": (_int, [_vp, _u64, _u32, _vp, _vp]),
+    "q8mi_qgemv": (_int, [_vp, _vp, _u32, _vp, _int, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_qgemv_add": (_int, [_vp, _vp, _u32, _vp, _int, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_qgemv_silu_mul": (_int, [_vp, _vp, _vp, _u32, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_qgemv_fanout4": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32,
+                                  _u32, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_probe_copy": (_int, [_vp, _vp, _u64, _vp]),
     "q8mi_synth_f32": (_int, [_vp, _u64, _u64, _u64, _int, C.c_float, _u32, C.c_float, _int]),
     "q8mi_synth_q8_0_weight": (_int, [_vp, _u64, _u64, _u64, C.c_float, _int]),
