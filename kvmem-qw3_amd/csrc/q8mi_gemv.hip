@@ -13,6 +13,7 @@
 #include <stdlib.h>
 
 #include "q8mi_gemv_core.hpp"
+#include "q8mi_gemv_mfma_core.hpp"
 
 namespace q8mi {
 namespace {
@@ -186,6 +187,114 @@ __device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, flo
     }
 }
 
+// ---- matrix-core variant for batch 3..32 (see q8mi_gemv_mfma_core.hpp) --------------------------
+// Unit u covers rows 4u .. 4u+3 of the concatenated row space; for SwiGLU gate rows 2u, 2u+1
+// (fragment rows 0, 1) and the matching up rows (fragment rows 2, 3).
+template <int MG, int THREADS, bool SILU>
+__global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, uint32_t batch,
+                                                            uint32_t park_floats) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr uint32_t MP = 4 * MG;
+    constexpr uint32_t kWaves = THREADS / kWave;
+    constexpr uint32_t kPerUnit = 4 * kMfmaUnitRows * MP;   // [chunk][row][activation row]
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, r = lane & 3u;
+    const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
+    const uint64_t row_bytes = static_cast<uint64_t>(p.nb) * 34;
+    const UnitSeq useq = group_units(p.units, blockIdx.x, gridDim.x, p.interleave);
+    const uint32_t ucount = useq.count;
+    const uint32_t n_items = ucount * nitems;
+    uint32_t i0, i1;
+    wave_items(n_items, wave, kWaves, i0, i1);
+    float *park_base = reinterpret_cast<float *>(smem + p.x_bytes);   // [wave][park_floats]
+    float *my_park = park_base + wave * park_floats;
+    const uint32_t last_row = p.total_rows - 1;
+
+    auto row_ptr = [&](uint32_t u) -> const uint8_t * {   // fragment row q is the one this lane loads
+        if constexpr (SILU) {
+            uint32_t row = 2 * u + (q & 1u);
+            row = row < last_row ? row : last_row;
+            return (q < 2 ? p.w[0] : p.w[1]) + row * row_bytes;
+        } else {
+            uint32_t row = 4 * u + q;
+            row = row < last_row ? row : last_row;
+            const RowRef a = resolve_row(p, row);
+            return a.w + a.local * row_bytes;
+        }
+    };
+    auto park = [&](uint32_t kk, auto &acc) {
+        if (q == c) {
+            float *dst = my_park + kk * kPerUnit + (c * kMfmaUnitRows + r) * MP;
+#pragma unroll
+            for (int g = 0; g < MG; ++g) {
+                float4 v;
+                v.x = acc[g][0]; v.y = acc[g][1]; v.z = acc[g][2]; v.w = acc[g][3];
+                *reinterpret_cast<float4 *>(dst + 4 * g) = v;
+            }
+        }
+    };
+#ifdef Q8MI_TRACE
+    const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
+#endif
+    mfma_stream<MG, THREADS>(smem, p.y, p.nb, batch, useq, i0, i1, row_ptr, park);
+#ifdef Q8MI_TRACE
+    const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
+#endif
+    __syncthreads();
+#ifdef Q8MI_TRACE
+    if (p.trace && threadIdx.x == 0) {
+        p.trace[blockIdx.x * 4 + 0] = t_begin;
+        p.trace[blockIdx.x * 4 + 1] = t_stream;
+        p.trace[blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
+    }
+#endif
+
+    // unit ranges of the waves, worked out once (wave w touched unit ordinals kf[w] .. kl[w])
+    __shared__ uint32_t s_kf[kWaves], s_kl[kWaves];
+    if (threadIdx.x < kWaves) {
+        uint32_t a0, a1;
+        wave_items(n_items, threadIdx.x, kWaves, a0, a1);
+        s_kf[threadIdx.x] = a1 > a0 ? a0 / nitems : 1u;
+        s_kl[threadIdx.x] = a1 > a0 ? (a1 - 1) / nitems : 0u;   // empty range: kf > kl
+    }
+    __syncthreads();
+    // total for unit ordinal k, fragment row rr, activation row m: partials in wave order, chunks in order
+    auto total_of = [&](uint32_t k, uint32_t rr, uint32_t m) {
+        float t = 0.0f;
+#pragma unroll
+        for (uint32_t w = 0; w < kWaves; ++w) {
+            const uint32_t kf = s_kf[w], kl = s_kl[w];
+            if (k < kf || k > kl) continue;
+            const float *e = park_base + w * park_floats + (k - kf) * kPerUnit + rr * MP + m;
+            t += ((e[0] + e[kMfmaUnitRows * MP]) + e[2 * kMfmaUnitRows * MP]) + e[3 * kMfmaUnitRows * MP];
+        }
+        return t;
+    };
+    if constexpr (SILU) {
+        for (uint32_t e = threadIdx.x; e < ucount * batch * 2; e += THREADS) {
+            const uint32_t k = e / (batch * 2), m = (e / 2) % batch, rr = e % 2;
+            const uint32_t row = 2 * useq.unit(k) + rr;
+            if (row >= p.total_rows) continue;
+            const float g = total_of(k, rr, m);
+            const float up = total_of(k, 2 + rr, m);
+            const float silu = g / (1.0f + __expf(-g));
+            static_cast<float *>(p.dst[0])[static_cast<uint64_t>(m) * p.stride[0] + row] = silu * up;
+        }
+    } else {
+        for (uint32_t e = threadIdx.x; e < ucount * batch * 4; e += THREADS) {
+            const uint32_t k = e / (batch * 4), m = (e / 4) % batch, rr = e % 4;
+            const uint32_t row = 4 * useq.unit(k) + rr;
+            if (row >= p.total_rows) continue;
+            const RowRef ref = resolve_row(p, row);
+            store_out(p.mode, ref.dst, static_cast<uint64_t>(m) * ref.stride + ref.local, total_of(k, rr, m));
+        }
+    }
+#ifdef Q8MI_TRACE
+    if (p.trace && threadIdx.x == 0) p.trace[blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
+#endif
+}
+
 // Fallback for rows whose planes are not 16-byte aligned (cols/32 not a
 // multiple of 8): one lane per 32-element block, 2-byte weight loads.
 __global__ __launch_bounds__(256) void gemv_unaligned_kernel(const GemvParams p, uint32_t batch) {
@@ -279,6 +388,7 @@ int launch_ms(const GemvParams &p, hipStream_t stream) {
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
     const int forced = gemv_tuning().threads;
     if (p.xf != nullptr) {   // fused quantizer: the activations must fit LDS
+        if (M > 2) return fail(Q8MI_REJECTED, "qgemv: batch %d above 2 (quantize once and use the GEMV instead)", M);
         if (xb + park_256 <= 76u * 1024u && forced != 1024) return launch_inst<M, 256, kXF32, SILU>(p, xb, stream);
         if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXF32, SILU>(p, xb, stream);
         return fail(Q8MI_REJECTED, "qgemv: %u activation rows of %u columns do not fit LDS", M, p.nb * 32);
@@ -295,6 +405,51 @@ int launch_m(const GemvParams &p, hipStream_t stream) {
     return p.mode == kSiluMul ? launch_ms<M, true>(p, stream) : launch_ms<M, false>(p, stream);
 }
 
+// One workgroup of 512 threads per CU: its eight waves split the items of its units evenly, so a
+// matrix only needs as many 4-row units as there are CUs to keep the chip busy.
+template <int MG, bool SILU>
+int launch_mfma(GemvParams p, uint32_t batch, hipStream_t stream) {
+    constexpr int THREADS = 512;
+    auto kern = gemv_mfma_kernel<MG, THREADS, SILU>;
+    const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+    p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
+    p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG);
+    p.interleave = gemv_tuning().interleave;
+    const uint32_t grid = p.units < cus ? p.units : cus;
+    const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
+    const uint32_t per_group = (p.units + grid - 1) / grid;
+    const uint32_t park_floats = max_units_touched(per_group, nitems, THREADS / kWave) * mfma_park_floats_per_unit(MG);
+    const uint32_t lds = p.x_bytes + (THREADS / kWave) * park_floats * 4;
+    constexpr uint32_t kDynLimit = kLdsLimit - 256;   // the kernel also has a few static LDS words
+    if (lds > kDynLimit) return fail(Q8MI_REJECTED, "gemv (matrix-core variant): %u bytes of LDS needed", lds);
+    static thread_local uint32_t granted = 0;
+    if (lds > 64u * 1024u && lds > granted) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(kDynLimit)) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
+        }
+        granted = kDynLimit;
+    }
+#ifdef Q8MI_TRACE
+    p.trace = nullptr;
+    if (const char *e = getenv("Q8MI_TRACE_PTR")) p.trace = reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 0));
+#endif
+    kern<<<grid, THREADS, lds, stream>>>(p, batch, park_floats);
+    return check_launch("gemv_mfma");
+}
+
+// Activations that fit LDS in the matrix-core layout (with room for the parked sums).
+bool mfma_fits(uint32_t nb, uint32_t batch) {
+    return mfma_x_lds_bytes(nb, batch, (batch + 3) / 4) + 16u * 1024u <= kLdsLimit - 256;
+}
+
+int launch_mfma_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
+    const bool silu = p.mode == kSiluMul;
+    if (batch <= 4) return silu ? launch_mfma<1, true>(p, batch, stream) : launch_mfma<1, false>(p, batch, stream);
+    return silu ? launch_mfma<2, true>(p, batch, stream) : launch_mfma<2, false>(p, batch, stream);
+}
+
 int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
     if (p.nb % 8 != 0) {
         if (p.xf != nullptr) return fail(Q8MI_REJECTED, "qgemv: cols %u not a multiple of 256", p.nb * 32);
@@ -305,6 +460,8 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         gemv_unaligned_kernel<<<grid, 256, 0, stream>>>(p, batch);
         return check_launch("gemv_unaligned");
     }
+    if (p.xf == nullptr && batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) && mfma_fits(p.nb, batch))
+        return launch_mfma_any(p, batch, stream);
     switch (batch) {
         case 1: return launch_m<1>(p, stream);
         case 2: return launch_m<2>(p, stream);
@@ -362,17 +519,20 @@ int run_single(const char *what, int mode, const uint8_t *w, const XSource &y, v
 
 }  // namespace
 
-// Shipped configuration: two workgroups per CU, interleaved units (best of the sweeps).
+// Shipped configuration: two workgroups per CU, interleaved units (best of the sweeps);
+// the matrix-core variant from batch kMfmaFromBatch on.
+constexpr int kMfmaFromBatch = 3;
 GemvTuning gemv_tuning() {
     static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
     auto read = [] {
-        GemvTuning t{2, 1, 0};
+        GemvTuning t{2, 1, 0, kMfmaFromBatch};
         if (const char *e = getenv("Q8MI_GEMV_WGS_PER_CU")) t.wgs_per_cu = atoi(e);
         if (const char *e = getenv("Q8MI_GEMV_INTERLEAVE")) t.interleave = atoi(e);
         if (const char *e = getenv("Q8MI_GEMV_THREADS")) t.threads = atoi(e);
+        if (const char *e = getenv("Q8MI_GEMV_MFMA_FROM")) t.mfma_from = atoi(e);
         return t;
     };
-    return live ? read() : GemvTuning{2, 1, 0};
+    return live ? read() : GemvTuning{2, 1, 0, kMfmaFromBatch};
 }
 
 // Any batch through the GEMV kernels, eight activation rows per launch.  Used by

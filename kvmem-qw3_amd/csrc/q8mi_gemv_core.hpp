@@ -424,6 +424,7 @@ struct GemvTuning {
     int wgs_per_cu;    // 0 = as many as fit (occupancy)
     int interleave;    // unit assignment, see group_units
     int threads;       // 0 = by LDS footprint, else 256 or 1024
+    int mfma_from;     // smallest batch served by the matrix-core variant
 };
 GemvTuning gemv_tuning();
 

@@ -1,0 +1,272 @@
+// Matrix-core variant of the Q8_0 x Q8_1 GEMV for small batches (3 .. 32
+// activation rows), shared by the GEMV family and the fused LM-head kernel.
+//
+// From batch 3 on the dot-product GEMV is bound by its VALU work (eight dot4 per
+// weight block and activation row).  Here the int8 dots go to
+// v_mfma_i32_16x16x32_i8 instead, and the VALU only rescales: the weights are
+// still read exactly once and the kernel stays HBM-bound up to batch 16.
+//
+// One MFMA multiplies A (16 x 32) by B (32 x 16).  Its K extent is 32 = one Q8
+// block, so one instruction may only ever see one block per (row, column) pair,
+// but nothing says the 16 columns must be 16 weight rows.  They are 4 weight
+// rows x 4 K-chunks, and the 16 A rows are 4 activation rows x the same 4
+// K-chunks:
+//     column n = 4 c + r   weight row r of the unit, block  kb(c, s)
+//     row    i = 4 c' + m  activation row m,           block  kb(c', s)
+//     kb(c, s) = 32 item + 4 s + c       (s = 0..7: eight MFMAs per item)
+// so one step consumes 128 contiguous bytes of each of the four rows.  The global loads are issued
+// in memory order (lane L reads bytes 8 (L % 16) .. of row L / 16: consecutive lanes, consecutive
+// addresses, which is what the vector memory path coalesces) and the 8-byte pieces are then moved to
+// the lanes the MFMA wants them in (lane 16 q + 4 c + r takes from lane 16 r + 4 c + q) with
+// ds_bpermute, which uses the LDS crossbar but no LDS memory.
+// D[i][n] pairs chunk c' of an activation row with chunk c of a weight row; the
+// products with c' == c are the wanted int32 block dots, the other three
+// quarters of D are discarded.  A lane holds D[4 q + v][n] (q = lane / 16,
+// v = 0..3), so the wanted values sit in the lanes with q == c, all four
+// registers of them (m = v): no per-lane register selection is needed.
+// Matrix-core time is free here (an HBM-bound stream needs under 2 % of the
+// int8 MFMA rate); what the layout buys is a unit of only FOUR weight rows, so
+// that a 5120-row matrix still splits into 1280 units.
+//
+// Work decomposition (as in the dot-product GEMV): unit = 4 rows, item = 32
+// blocks of a unit (1 KiB per row: eight 8-byte loads per lane, plus the row's 32 fp16
+// scales), a workgroup owns a list of units, its waves split the item list
+// evenly and park partial sums per touched unit in LDS.  A parked entry is
+// [chunk][row][activation row]: the four chunk partials of a row are added in
+// the combine phase, in chunk order.
+// Batches above 4 reuse the weight fragment for MG = ceil(batch / 4) MFMAs with
+// different activation fragments.
+#pragma once
+
+#include "q8mi_gemv_core.hpp"
+
+namespace q8mi {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+constexpr uint32_t kMfmaItemBlocks = 32;   // blocks of a row per item: 4 chunks x 8 steps
+constexpr uint32_t kMfmaUnitRows = 4;
+
+// LDS image of the activations:
+//   quants   [batch rows][nb][32 B], rows row_pitch = 32 nb + 128 bytes apart.  A fragment read
+//            (lane = activation row m, chunk c, k-quarter q) touches m * row_pitch + 32 c + 8 q
+//            (+ the step's offset): 128 contiguous bytes per activation row, and the odd
+//            multiple of 128 in the pitch puts rows m and m + 1 on the two halves of the banks
+//   scales   [nb][MP] fp32 (MP = 4 MG activation rows, padded): the four chunks of a step read
+//            four neighbouring MP-float groups
+__host__ __device__ inline uint32_t mfma_xq_row_pitch(uint32_t nb) { return nb * 32 + 128; }
+__host__ __device__ inline uint32_t mfma_xq_bytes(uint32_t nb, uint32_t batch) { return batch * mfma_xq_row_pitch(nb); }
+inline uint32_t mfma_x_lds_bytes(uint32_t nb, uint32_t batch, uint32_t mg) {
+    return mfma_xq_bytes(nb, batch) + nb * 4 * mg * 4;
+}
+// Floats one wave parks per touched unit.
+inline uint32_t mfma_park_floats_per_unit(uint32_t mg) { return 4 * kMfmaUnitRows * 4 * mg; }
+
+struct MfmaItem {
+    v2i q[8];   // per step: bytes 8 (L % 16) .. +8 of the step's 128 bytes of row L / 16 (memory order)
+    int d;      // fp16 scales 2 (L % 16), 2 (L % 16) + 1 of the item's 32, row L / 16
+};
+
+// Copies `batch` rows of Q8_1 activations into the LDS image above.  Ends with a barrier.
+template <int MG, int THREADS>
+__device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb,
+                                             uint32_t batch) {
+    constexpr uint32_t MP = 4 * MG;
+    constexpr int kBatch = 4;
+    const uint32_t row_pitch = mfma_xq_row_pitch(nb);
+    uint8_t *xq = smem;
+    uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
+    // row by row (a row is nb * 36 bytes, a multiple of 16: nb % 8 == 0), so that locating a dword
+    // needs no division by nb; all loads of a trip are issued before the first is used
+    const uint32_t row_dw = nb * 9, row_ch = row_dw / 4;
+    auto put = [&](uint32_t m, uint32_t g, uint32_t word) {   // g: dword index inside row m
+        const uint32_t kb = g / 9, part = g % 9;
+        if (part == 0) {
+            *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
+        } else {
+            *reinterpret_cast<uint32_t *>(xq + m * row_pitch + kb * 32 + (part - 1) * 4) = word;
+        }
+    };
+    if (reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+        const v4i *src = reinterpret_cast<const v4i *>(y);
+        const uint32_t total_ch = batch * row_ch;
+        for (uint32_t base = 0; base < total_ch; base += THREADS * kBatch) {
+            v4i v[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint32_t c = base + u * THREADS + threadIdx.x;
+                v[u] = src[c < total_ch ? c : 0];
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint32_t c = base + u * THREADS + threadIdx.x;
+                if (c < total_ch) {
+                    uint32_t m = 0, cc = c;                 // batch <= 32: a short subtract loop beats a division
+                    while (cc >= row_ch) { cc -= row_ch; ++m; }
+                    put(m, 4 * cc + 0, static_cast<uint32_t>(v[u].x));
+                    put(m, 4 * cc + 1, static_cast<uint32_t>(v[u].y));
+                    put(m, 4 * cc + 2, static_cast<uint32_t>(v[u].z));
+                    put(m, 4 * cc + 3, static_cast<uint32_t>(v[u].w));
+                }
+            }
+        }
+    } else {
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(y);
+        for (uint32_t m = 0; m < batch; ++m)
+            for (uint32_t g = threadIdx.x; g < row_dw; g += THREADS) put(m, g, src[m * row_dw + g]);
+    }
+    // scales of the padding rows batch .. 4 MG - 1 (their products are never stored; keep them finite)
+    if (batch < MP) {
+        const uint32_t pad = MP - batch;
+        for (uint32_t i = threadIdx.x; i < nb * pad; i += THREADS) {
+            const uint32_t kb = i / pad, m = batch + i % pad;
+            *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = 0.0f;
+        }
+    }
+    __syncthreads();
+}
+
+// Streams the items [i0, i1) of the workgroup's unit sequence (item i = part i % nitems of unit
+// i / nitems, nitems = ceil(nb / 32)).
+//   row_ptr(u)             the weight row (scale plane) this lane LOADS for unit u: fragment row lane / 16,
+//                          clamped to a readable row
+//   park(kk, acc)          once per unit touched (kk = 0, 1, ...), wave-uniform control flow; acc[g][v] is
+//                          this lane's partial sum for activation row 4 g + v and fragment row lane % 4,
+//                          meaningful in the lanes with lane / 16 == (lane % 16) / 4; must not touch
+//                          global memory
+// Must be called by every wave of the workgroup (contains the staging barrier).
+template <int MG, int THREADS, class RowPtr, class Park>
+__device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb, uint32_t batch,
+                                            const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
+                                            Park park) {
+    constexpr uint32_t MP = 4 * MG;
+    constexpr float kMagic = 12582912.0f;
+    const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, m4 = lane & 3u;
+    if (i1 <= i0) {
+        mfma_stage_x<MG, THREADS>(smem, y, nb, batch);
+        return;
+    }
+    const uint32_t n_items = i1 - i0;
+    const uint32_t n_padded = (n_items + 1) / 2 * 2;
+
+    MfmaItem items[2];
+    uint32_t ik = i0 / nitems, istep = i0 % nitems, ileft = n_items;
+    const uint8_t *irow = row_ptr(useq.unit(ik));
+    const uint32_t l16 = lane & 15u;
+    auto issue = [&](MfmaItem &it) {
+        const uint32_t left = nb - istep * kMfmaItemBlocks;          // blocks of the row from this item on
+        const uint32_t vsteps = left >= kMfmaItemBlocks ? 8u : left / 4;   // steps with real blocks (nb % 8 == 0)
+        it.d = *reinterpret_cast<const int *>(irow + istep * 64 + l16 * 4);   // stays inside the row
+        const uint8_t *qp = irow + 2 * nb + istep * 1024 + l16 * 8;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            // steps past the row's end re-read step 0; compute gives them a zero scale
+            it.q[s] = *reinterpret_cast<const v2i *>(qp + (static_cast<uint32_t>(s) < vsteps ? s * 128 : 0));
+        }
+        if (ileft > 1) {          // otherwise keep re-reading the last real item
+            --ileft;
+            if (++istep == nitems) {
+                istep = 0;
+                ++ik;
+                irow = row_ptr(useq.unit(ik));
+            }
+        }
+    };
+    issue(items[0]);
+    issue(items[1]);
+    mfma_stage_x<MG, THREADS>(smem, y, nb, batch);
+
+    const uint32_t row_pitch = mfma_xq_row_pitch(nb);
+    const uint8_t *xq = smem;
+    const uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
+    // activation fragment rows of this lane, one per MFMA group (clamped: rows past the batch are never stored)
+    uint32_t a_row[MG];
+#pragma unroll
+    for (int g = 0; g < MG; ++g) {
+        const uint32_t m = 4 * g + m4;
+        a_row[g] = (m < batch ? m : batch - 1) * row_pitch + 32 * c + 8 * q;
+    }
+    // source lanes of the operand shuffle (byte addresses for ds_bpermute)
+    const int src_q = static_cast<int>((16 * m4 + 4 * c + q) * 4);
+    const int src_d = static_cast<int>((16 * m4 + (c >> 1)) * 4);
+    v4i seed;
+    seed.x = seed.y = seed.z = seed.w = 0x4B400000;   // 1.5 * 2^23: the int32 result read as fp32 is 12582912 + S
+    asm volatile("" : "+v"(seed));
+
+    float acc[MG][4];
+#pragma unroll
+    for (int g = 0; g < MG; ++g)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[g][v] = 0.0f;
+
+    uint32_t cstep = i0 % nitems, kk = 0;
+    for (uint32_t t = 0; t < n_padded; t += 2) {
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            const MfmaItem &it = items[d];
+            const uint32_t left = nb - cstep * kMfmaItemBlocks;
+            const uint32_t vsteps = left >= kMfmaItemBlocks ? 8u : left / 4;
+            const uint8_t *xq_chunk = xq + cstep * 1024;
+            const uint8_t *xd_chunk = xd + (cstep * kMfmaItemBlocks + c) * MP * 4;
+            // activation fragments and scales are fetched one step ahead of the MFMAs that use them
+            long a_nxt[MG];
+            float4 dx_nxt[MG];
+#pragma unroll
+            for (int g = 0; g < MG; ++g) {
+                a_nxt[g] = *reinterpret_cast<const long *>(xq_chunk + a_row[g]);
+                dx_nxt[g] = *reinterpret_cast<const float4 *>(xd_chunk + 16 * g);
+            }
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                long a_cur[MG];
+                float4 dx_cur[MG];
+#pragma unroll
+                for (int g = 0; g < MG; ++g) { a_cur[g] = a_nxt[g]; dx_cur[g] = dx_nxt[g]; }
+                if (s < 7) {
+                    // steps past the row's end read step 0 again (finite values; their weight scale is zero)
+                    const uint32_t sn = static_cast<uint32_t>(s + 1) < vsteps ? s + 1 : 0;
+#pragma unroll
+                    for (int g = 0; g < MG; ++g) {
+                        a_nxt[g] = *reinterpret_cast<const long *>(xq_chunk + a_row[g] + sn * 128);
+                        dx_nxt[g] = *reinterpret_cast<const float4 *>(xd_chunk + sn * 4 * MP * 4 + 16 * g);
+                    }
+                }
+                // halfword 4 s + c of the row's scales: dword 2 s + c / 2 (held by lane 16 r + 2 s + c / 2), half c % 2
+                const uint32_t dword = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(src_d + 8 * s, it.d));
+                const uint16_t hbits = static_cast<uint16_t>((c & 1u) ? (dword >> 16) : (dword & 0xffffu));
+                const float dw = static_cast<uint32_t>(s) < vsteps ? half_bits_to_float(hbits) : 0.0f;
+                const float cw = -kMagic * dw;
+                v2i bq;
+                bq.x = __builtin_amdgcn_ds_bpermute(src_q, it.q[s].x);
+                bq.y = __builtin_amdgcn_ds_bpermute(src_q, it.q[s].y);
+                const long b = __builtin_bit_cast(long, bq);
+                v4i r[MG];
+#pragma unroll
+                for (int g = 0; g < MG; ++g) r[g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_cur[g], b, seed, 0, 0, 0);
+#pragma unroll
+                for (int g = 0; g < MG; ++g) {
+                    acc[g][0] = fmaf(fmaf(as_f32(r[g].x), dw, cw), dx_cur[g].x, acc[g][0]);
+                    acc[g][1] = fmaf(fmaf(as_f32(r[g].y), dw, cw), dx_cur[g].y, acc[g][1]);
+                    acc[g][2] = fmaf(fmaf(as_f32(r[g].z), dw, cw), dx_cur[g].z, acc[g][2]);
+                    acc[g][3] = fmaf(fmaf(as_f32(r[g].w), dw, cw), dx_cur[g].w, acc[g][3]);
+                }
+            }
+            ++cstep;
+            const uint32_t done = t + d + 1;
+            if (done <= n_items && (cstep == nitems || done == n_items)) {
+                park(kk, acc);
+                ++kk;
+#pragma unroll
+                for (int g = 0; g < MG; ++g)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[g][v] = 0.0f;
+            }
+            if (cstep == nitems) cstep = 0;
+            issue(items[d]);
+        }
+    }
+}
+
+}  // namespace q8mi

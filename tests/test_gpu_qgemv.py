@@ -32,6 +32,9 @@ def test_qgemv_equals_two_step(gpu, rows, cols, batch):
     one = hip.DeviceBuffer(4 * n).fill(0xee)
     ok(L.q8mi_gemv(dw.ptr, dy.ptr, two.ptr, rows, cols, batch, rows, NULL), "gemv")
     rc = L.q8mi_qgemv(dw.ptr, dx.ptr, stride_x, one.ptr, 0, rows, cols, batch, rows, NULL)
+    if batch > 2:
+        assert rc == q8mi.REJECTED, "the fused form serves batch 1 and 2 only"
+        return
     if rc == q8mi.REJECTED:
         # declined only when the staged activations (plus the per-wave result area) exceed LDS
         steps = (cols // 32 * 2 + 127) // 128
@@ -52,7 +55,7 @@ def test_qgemv_equals_two_step(gpu, rows, cols, batch):
     assert np.array_equal(bits(a1, n), bits(a2, n))
 
 
-@pytest.mark.parametrize("batch", [1, 4, 8])
+@pytest.mark.parametrize("batch", [1, 2])
 def test_qgemv_silu_and_fanout_equal_two_step(gpu, batch):
     L = gpu.lib()
     rows, cols = 1000, 1024
@@ -80,4 +83,5 @@ def test_qgemv_rejections(gpu):
     b = hip.DeviceBuffer(1 << 16)
     assert L.q8mi_qgemv(b.ptr, b.ptr, 96, b.ptr, 0, 4, 96, 1, 4, NULL) == q8mi.REJECTED      # cols % 256
     assert L.q8mi_qgemv(b.ptr, b.ptr, 256, b.ptr, 0, 4, 256, 9, 4, NULL) == q8mi.REJECTED    # batch > 8
+    assert L.q8mi_qgemv(b.ptr, b.ptr, 256, b.ptr, 0, 4, 256, 3, 4, NULL) == q8mi.REJECTED    # batch > 2
     assert L.q8mi_qgemv(b.ptr, b.ptr, 250, b.ptr, 0, 4, 250, 1, 4, NULL) == q8mi.REJECTED    # cols % 32
