@@ -15,6 +15,7 @@
 // wins, equal logits go to the lower token id, src/kernels_cuda.cu:1765-1771),
 // which is independent of the order partials are merged in for NaN-free logits.
 #include "q8mi_gemv_core.hpp"
+#include "q8mi_gemv_mfma_core.hpp"
 
 namespace q8mi {
 namespace {
@@ -93,6 +94,104 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
             const uint32_t row = R * useq.unit(k) + r;
             if (row >= rows) continue;
             const float s = total_of(k, m * R + r);
+            if (beats(s, static_cast<int>(row), bv, bi)) { bv = s; bi = static_cast<int>(row); }
+            if (logits != nullptr) logits[static_cast<uint64_t>(m) * stride_logits + row] = s;
+        }
+        sv[threadIdx.x] = bv;
+        si[threadIdx.x] = bi;
+        __syncthreads();
+        for (uint32_t stride = THREADS / 2; stride > 0; stride >>= 1) {
+            if (threadIdx.x < stride) {
+                const float ov = sv[threadIdx.x + stride];
+                const int oi = si[threadIdx.x + stride];
+                if (beats(ov, oi, sv[threadIdx.x], si[threadIdx.x])) { sv[threadIdx.x] = ov; si[threadIdx.x] = oi; }
+            }
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            q8mi_argmax_pair *p = partial + static_cast<uint64_t>(m) * gridDim.x + blockIdx.x;
+            p->value = sv[0];
+            p->index = si[0];
+        }
+        __syncthreads();
+    }
+}
+
+// Matrix-core variant for 3 or more verify rows (see q8mi_gemv_mfma_core.hpp): same unit and
+// item decomposition as the GEMV's matrix-core kernel at the same grid, so the logits are the
+// same bits as that GEMV's.
+template <int MG, int THREADS>
+__global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, uint32_t rows, uint32_t nb, uint32_t batch,
+        q8mi_argmax_pair *__restrict__ partial, float *__restrict__ logits, uint32_t stride_logits,
+        int interleave, uint32_t x_bytes, uint32_t park_floats) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr uint32_t MP = 4 * MG;
+    constexpr uint32_t kWaves = THREADS / kWave;
+    constexpr uint32_t kPerUnit = 4 * kMfmaUnitRows * MP;
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, r = lane & 3u;
+    const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
+    const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    const uint32_t units = (rows + kMfmaUnitRows - 1) / kMfmaUnitRows;
+    const UnitSeq useq = group_units(units, blockIdx.x, gridDim.x, interleave);
+    const uint32_t ucount = useq.count;
+    const uint32_t n_items = ucount * nitems;
+    uint32_t i0, i1;
+    wave_items(n_items, wave, kWaves, i0, i1);
+    float *park_base = reinterpret_cast<float *>(smem + x_bytes);
+    float *my_park = park_base + wave * park_floats;
+
+    auto row_ptr = [&](uint32_t u) -> const uint8_t * {
+        uint32_t row = kMfmaUnitRows * u + q;
+        row = row < rows - 1 ? row : rows - 1;
+        return w + row * row_bytes;
+    };
+    auto park = [&](uint32_t kk, auto &acc) {
+        if (q == c) {
+            float *dst = my_park + kk * kPerUnit + (c * kMfmaUnitRows + r) * MP;
+#pragma unroll
+            for (int g = 0; g < MG; ++g) {
+                float4 v;
+                v.x = acc[g][0]; v.y = acc[g][1]; v.z = acc[g][2]; v.w = acc[g][3];
+                *reinterpret_cast<float4 *>(dst + 4 * g) = v;
+            }
+        }
+    };
+    mfma_stream<MG, THREADS>(smem, y, nb, batch, useq, i0, i1, row_ptr, park);
+    __syncthreads();
+
+    __shared__ uint32_t s_kf[kWaves], s_kl[kWaves];
+    if (threadIdx.x < kWaves) {
+        uint32_t a0, a1;
+        wave_items(n_items, threadIdx.x, kWaves, a0, a1);
+        s_kf[threadIdx.x] = a1 > a0 ? a0 / nitems : 1u;
+        s_kl[threadIdx.x] = a1 > a0 ? (a1 - 1) / nitems : 0u;
+    }
+    __syncthreads();
+    auto total_of = [&](uint32_t k, uint32_t rr, uint32_t m) {
+        float t = 0.0f;
+#pragma unroll
+        for (uint32_t wv = 0; wv < kWaves; ++wv) {
+            const uint32_t kf = s_kf[wv], kl = s_kl[wv];
+            if (k < kf || k > kl) continue;
+            const float *e = park_base + wv * park_floats + (k - kf) * kPerUnit + rr * MP + m;
+            t += ((e[0] + e[kMfmaUnitRows * MP]) + e[2 * kMfmaUnitRows * MP]) + e[3 * kMfmaUnitRows * MP];
+        }
+        return t;
+    };
+
+    __shared__ float sv[THREADS];
+    __shared__ int si[THREADS];
+    for (uint32_t m = 0; m < batch; ++m) {
+        float bv = -INFINITY;
+        int bi = -1;
+        for (uint32_t e = threadIdx.x; e < ucount * kMfmaUnitRows; e += THREADS) {   // rows in ascending order
+            const uint32_t k = e / kMfmaUnitRows, rr = e % kMfmaUnitRows;
+            const uint32_t row = kMfmaUnitRows * useq.unit(k) + rr;
+            if (row >= rows) continue;
+            const float s = total_of(k, rr, m);
             if (beats(s, static_cast<int>(row), bv, bi)) { bv = s; bi = static_cast<int>(row); }
             if (logits != nullptr) logits[static_cast<uint64_t>(m) * stride_logits + row] = s;
         }
@@ -203,6 +302,46 @@ int launch_inst(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t nb, 
     return check_launch("lm_head");
 }
 
+template <int MG>
+int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t nb, uint32_t batch,
+                        q8mi_argmax_pair *partial, float *logits, uint32_t stride_logits, uint32_t *grid_out,
+                        hipStream_t stream) {
+    constexpr int THREADS = 512;
+    auto kern = lm_head_mfma_kernel<MG, THREADS>;
+    const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+    const uint32_t units = (rows + kMfmaUnitRows - 1) / kMfmaUnitRows;
+    uint32_t grid = units < cus ? units : cus;     // the geometry of the GEMV's matrix-core launch
+    if (grid > kMaxPartials) grid = kMaxPartials;
+    const uint32_t x_bytes = mfma_x_lds_bytes(nb, batch, MG);
+    const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
+    const uint32_t per_group = (units + grid - 1) / grid;
+    const uint32_t park_floats = max_units_touched(per_group, nitems, THREADS / kWave) * mfma_park_floats_per_unit(MG);
+    const uint32_t lds = x_bytes + (THREADS / kWave) * park_floats * 4;
+    constexpr uint32_t kDynLimit = kLdsLimit - THREADS * 8 - 256;   // static LDS: the argmax tree and a few words
+    if (lds > kDynLimit) return fail(Q8MI_REJECTED, "lm_head (matrix-core variant): %u bytes of LDS needed", lds);
+    static thread_local bool granted = false;
+    if (lds > 64u * 1024u && !granted) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(kDynLimit)) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "lm_head: cannot reserve %u bytes of LDS", lds);
+        }
+        granted = true;
+    }
+    *grid_out = grid;
+    kern<<<grid, THREADS, lds, stream>>>(w, y, rows, nb, batch, partial, logits, stride_logits,
+                                         gemv_tuning().interleave, x_bytes, park_floats);
+    return check_launch("lm_head");
+}
+
+// Same routing rule as the GEMV: matrix-core variant from gemv_tuning().mfma_from rows on, when
+// the activations fit LDS in its layout.
+bool lm_head_uses_mfma(uint32_t nb, uint32_t batch) {
+    const uint32_t mg = (batch + 3) / 4;
+    return batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) &&
+           mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u <= kLdsLimit - 256;
+}
+
 template <int M>
 int launch_lm_head(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t nb, q8mi_argmax_pair *partial,
                    float *logits, uint32_t stride_logits, uint32_t *grid_out, hipStream_t stream) {
@@ -254,7 +393,12 @@ extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, 
     const auto *yb = static_cast<const uint8_t *>(y);
     hipStream_t s = as_stream(stream);
     int rc = Q8MI_REJECTED;
-    switch (batch) {
+    if (lm_head_uses_mfma(nb, batch)) {
+        rc = batch <= 4 ? launch_lm_head_mfma<1>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s)
+                        : launch_lm_head_mfma<2>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s);
+    }
+    // very tall weights park more partial sums per workgroup than LDS holds: dot-product variant
+    if (rc == Q8MI_REJECTED) switch (batch) {
         case 1: rc = launch_lm_head<1>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
         case 2: rc = launch_lm_head<2>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
         case 3: rc = launch_lm_head<3>(weight, yb, rows, nb, partial, logits, stride_logits, &grid, s); break;
