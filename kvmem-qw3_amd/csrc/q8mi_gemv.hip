@@ -190,7 +190,7 @@ __device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, flo
 // ---- matrix-core variant for batch 3..32 (see q8mi_gemv_mfma_core.hpp) --------------------------
 // Unit u covers rows 4u .. 4u+3 of the concatenated row space; for SwiGLU gate rows 2u, 2u+1
 // (fragment rows 0, 1) and the matching up rows (fragment rows 2, 3).
-template <int MG, int THREADS, bool SILU>
+template <int MG, int THREADS, bool SILU, bool HS>
 __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, uint32_t batch,
                                                             uint32_t park_floats) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
 #ifdef Q8MI_TRACE
     const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
 #endif
-    mfma_stream<MG, THREADS>(smem, p.y, p.nb, batch, useq, i0, i1, row_ptr, park);
+    mfma_stream<MG, THREADS, HS>(smem, p.y, p.nb, batch, useq, i0, i1, row_ptr, park);
 #ifdef Q8MI_TRACE
     const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
 #endif
@@ -407,13 +407,13 @@ int launch_m(const GemvParams &p, hipStream_t stream) {
 
 // One workgroup of 512 threads per CU: its eight waves split the items of its units evenly, so a
 // matrix only needs as many 4-row units as there are CUs to keep the chip busy.
-template <int MG, bool SILU>
+template <int MG, bool SILU, bool HS>
 int launch_mfma(GemvParams p, uint32_t batch, hipStream_t stream) {
     constexpr int THREADS = 512;
-    auto kern = gemv_mfma_kernel<MG, THREADS, SILU>;
+    auto kern = gemv_mfma_kernel<MG, THREADS, SILU, HS>;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
-    p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG);
+    p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG, HS);
     p.interleave = gemv_tuning().interleave;
     const uint32_t grid = p.units < cus ? p.units : cus;
     const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
@@ -440,14 +440,23 @@ int launch_mfma(GemvParams p, uint32_t batch, hipStream_t stream) {
 }
 
 // Activations that fit LDS in the matrix-core layout (with room for the parked sums).
-bool mfma_fits(uint32_t nb, uint32_t batch) {
-    return mfma_x_lds_bytes(nb, batch, (batch + 3) / 4) + 16u * 1024u <= kLdsLimit - 256;
+// (8 KB: what the eight waves park for the short unit lists of such long rows.)
+bool mfma_fits(uint32_t nb, uint32_t batch, bool half_scales) {
+    return mfma_x_lds_bytes(nb, batch, (batch + 3) / 4, half_scales) + (half_scales ? 8u : 16u) * 1024u <=
+           kLdsLimit - 256;
+}
+
+template <bool HS>
+int launch_mfma_hs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
+    const bool silu = p.mode == kSiluMul;
+    if (batch <= 4)
+        return silu ? launch_mfma<1, true, HS>(p, batch, stream) : launch_mfma<1, false, HS>(p, batch, stream);
+    return silu ? launch_mfma<2, true, HS>(p, batch, stream) : launch_mfma<2, false, HS>(p, batch, stream);
 }
 
 int launch_mfma_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
-    const bool silu = p.mode == kSiluMul;
-    if (batch <= 4) return silu ? launch_mfma<1, true>(p, batch, stream) : launch_mfma<1, false>(p, batch, stream);
-    return silu ? launch_mfma<2, true>(p, batch, stream) : launch_mfma<2, false>(p, batch, stream);
+    if (mfma_fits(p.nb, batch, false)) return launch_mfma_hs<false>(p, batch, stream);
+    return launch_mfma_hs<true>(p, batch, stream);
 }
 
 int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
@@ -460,8 +469,11 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         gemv_unaligned_kernel<<<grid, 256, 0, stream>>>(p, batch);
         return check_launch("gemv_unaligned");
     }
-    if (p.xf == nullptr && batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) && mfma_fits(p.nb, batch))
-        return launch_mfma_any(p, batch, stream);
+    if (p.xf == nullptr && batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) &&
+        (mfma_fits(p.nb, batch, false) || mfma_fits(p.nb, batch, true))) {
+        const int rc = launch_mfma_any(p, batch, stream);
+        if (rc != Q8MI_REJECTED) return rc;   // a unit list whose parked sums do not fit: dot-product variant
+    }
     switch (batch) {
         case 1: return launch_m<1>(p, stream);
         case 2: return launch_m<2>(p, stream);

@@ -56,8 +56,10 @@ constexpr uint32_t kMfmaUnitRows = 4;
 //            four neighbouring MP-float groups
 __host__ __device__ inline uint32_t mfma_xq_row_pitch(uint32_t nb) { return nb * 32 + 128; }
 __host__ __device__ inline uint32_t mfma_xq_bytes(uint32_t nb, uint32_t batch) { return batch * mfma_xq_row_pitch(nb); }
-inline uint32_t mfma_x_lds_bytes(uint32_t nb, uint32_t batch, uint32_t mg) {
-    return mfma_xq_bytes(nb, batch) + nb * 4 * mg * 4;
+// half_scales: the scale table as fp16 instead of fp32 (half the size, one conversion per use); for
+// activations that would not fit otherwise.
+inline uint32_t mfma_x_lds_bytes(uint32_t nb, uint32_t batch, uint32_t mg, bool half_scales = false) {
+    return mfma_xq_bytes(nb, batch) + nb * 4 * mg * (half_scales ? 2 : 4);
 }
 // Floats one wave parks per touched unit.
 inline uint32_t mfma_park_floats_per_unit(uint32_t mg) { return 4 * kMfmaUnitRows * 4 * mg; }
@@ -68,7 +70,7 @@ struct MfmaItem {
 };
 
 // Copies `batch` rows of Q8_1 activations into the LDS image above.  Ends with a barrier.
-template <int MG, int THREADS>
+template <int MG, int THREADS, bool HS>
 __device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb,
                                              uint32_t batch) {
     constexpr uint32_t MP = 4 * MG;
@@ -82,7 +84,8 @@ __device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__res
     auto put = [&](uint32_t m, uint32_t g, uint32_t word) {   // g: dword index inside row m
         const uint32_t kb = g / 9, part = g % 9;
         if (part == 0) {
-            *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
+            if (HS) *reinterpret_cast<uint16_t *>(xd + (kb * MP + m) * 2) = static_cast<uint16_t>(word & 0xffffu);
+            else *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
         } else {
             *reinterpret_cast<uint32_t *>(xq + m * row_pitch + kb * 32 + (part - 1) * 4) = word;
         }
@@ -120,7 +123,8 @@ __device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__res
         const uint32_t pad = MP - batch;
         for (uint32_t i = threadIdx.x; i < nb * pad; i += THREADS) {
             const uint32_t kb = i / pad, m = batch + i % pad;
-            *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = 0.0f;
+            if (HS) *reinterpret_cast<uint16_t *>(xd + (kb * MP + m) * 2) = 0;
+            else *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = 0.0f;
         }
     }
     __syncthreads();
@@ -135,7 +139,7 @@ __device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__res
 //                          meaningful in the lanes with lane / 16 == (lane % 16) / 4; must not touch
 //                          global memory
 // Must be called by every wave of the workgroup (contains the staging barrier).
-template <int MG, int THREADS, class RowPtr, class Park>
+template <int MG, int THREADS, bool HS, class RowPtr, class Park>
 __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb, uint32_t batch,
                                             const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
                                             Park park) {
@@ -145,7 +149,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, m4 = lane & 3u;
     if (i1 <= i0) {
-        mfma_stage_x<MG, THREADS>(smem, y, nb, batch);
+        mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
         return;
     }
     const uint32_t n_items = i1 - i0;
@@ -176,7 +180,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     };
     issue(items[0]);
     issue(items[1]);
-    mfma_stage_x<MG, THREADS>(smem, y, nb, batch);
+    mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
 
     const uint32_t row_pitch = mfma_xq_row_pitch(nb);
     const uint8_t *xq = smem;
@@ -209,14 +213,28 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
             const uint32_t left = nb - cstep * kMfmaItemBlocks;
             const uint32_t vsteps = left >= kMfmaItemBlocks ? 8u : left / 4;
             const uint8_t *xq_chunk = xq + cstep * 1024;
-            const uint8_t *xd_chunk = xd + (cstep * kMfmaItemBlocks + c) * MP * 4;
+            constexpr uint32_t kSc = HS ? 2 : 4;   // bytes per scale
+            const uint8_t *xd_chunk = xd + (cstep * kMfmaItemBlocks + c) * MP * kSc;
+            auto load_dx = [&](const uint8_t *p) {
+                float4 v;
+                if (HS) {
+                    const uint2 h = *reinterpret_cast<const uint2 *>(p);
+                    v.x = half_bits_to_float(static_cast<uint16_t>(h.x & 0xffffu));
+                    v.y = half_bits_to_float(static_cast<uint16_t>(h.x >> 16));
+                    v.z = half_bits_to_float(static_cast<uint16_t>(h.y & 0xffffu));
+                    v.w = half_bits_to_float(static_cast<uint16_t>(h.y >> 16));
+                } else {
+                    v = *reinterpret_cast<const float4 *>(p);
+                }
+                return v;
+            };
             // activation fragments and scales are fetched one step ahead of the MFMAs that use them
             long a_nxt[MG];
             float4 dx_nxt[MG];
 #pragma unroll
             for (int g = 0; g < MG; ++g) {
                 a_nxt[g] = *reinterpret_cast<const long *>(xq_chunk + a_row[g]);
-                dx_nxt[g] = *reinterpret_cast<const float4 *>(xd_chunk + 16 * g);
+                dx_nxt[g] = load_dx(xd_chunk + 4 * kSc * g);
             }
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
@@ -230,7 +248,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
 #pragma unroll
                     for (int g = 0; g < MG; ++g) {
                         a_nxt[g] = *reinterpret_cast<const long *>(xq_chunk + a_row[g] + sn * 128);
-                        dx_nxt[g] = *reinterpret_cast<const float4 *>(xd_chunk + sn * 4 * MP * 4 + 16 * g);
+                        dx_nxt[g] = load_dx(xd_chunk + sn * 4 * MP * kSc + 4 * kSc * g);
                     }
                 }
                 // halfword 4 s + c of the row's scales: dword 2 s + c / 2 (held by lane 16 r + 2 s + c / 2), half c % 2
