@@ -188,11 +188,11 @@ def cpu_baseline(seconds=12.0):
 
 
 def bench_gemm(q8mi, hip, synth, reps=10):
-    """Prefill GEMM (D4 quantize + MFMA GEMM) at M=2048 on the two FFN shapes."""
+    """Prefill GEMM (D4 quantize + MFMA GEMM): M=2048 on the two FFN shapes, M=8192 on gate/up."""
     L, ok = q8mi.lib(), q8mi.ok
     out = {}
-    m = 2048
-    for name, rows, cols in (("k5120_n17408", FFN, HIDDEN), ("k17408_n5120", HIDDEN, FFN)):
+    for name, rows, cols, m in (("m2048_k5120_n17408", FFN, HIDDEN, 2048), ("m2048_k17408_n5120", HIDDEN, FFN, 2048),
+                                ("m8192_k5120_n17408", FFN, HIDDEN, 8192)):
         w = hip.to_device(synth.q8_0_weight(rows, cols, seed=rows + 7))
         x = hip.to_device(synth.normal(m, cols, seed=cols + 9))
         y = hip.DeviceBuffer(L.q8mi_q8_1_d4_scratch_bytes(m, cols))
@@ -333,7 +333,7 @@ def main():
         for b in l.w.values():
             b.free()
     if not args.quick:
-        result["gemm_int8_m2048"] = bench_gemm(q8mi, hip, synth)
+        result["gemm_int8"] = bench_gemm(q8mi, hip, synth)
         result["lm_head_fused"] = bench_lm_head(q8mi, hip, synth)
     if not (args.quick or args.no_cpu):
         result["cpu_baseline"] = cpu_baseline()

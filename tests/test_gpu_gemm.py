@@ -104,6 +104,32 @@ def test_gemm_large_tilings(gpu, oracle, rows, batch, cols):
         assert_close_fp32(got[j, :rows], ref_c, absum_c, f"gemm column {j}")
 
 
+def test_gemm_heavy_tail_batch_8192(gpu, oracle):
+    """Long-context prefill shape with heavy-tailed activations: batch 8192, Student-t(3) values
+    with 0.1 % of the columns scaled by 20 (outlier channels).  Quantized activations bit-exact on a
+    row sample, per-block int32 dots bit-exact and bounded by 32 * 127 * 127, outputs within
+    tolerance on a seeded sample."""
+    rows, cols, batch = 5120, 5120, 8192
+    w = synth.q8_0_weight(rows, cols, seed=77)
+    x = synth.student_t3(batch, cols, seed=78)
+    assert np.abs(x).max() > 50.0, "the generator must produce outliers"
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    pick = np.array([0, 1, 4095, 4096, 8191], np.int64)
+    rc, yref = oracle.quantize_q8_1_d4(x[pick])
+    yb = y.reshape(cols // 128, batch, 144)
+    assert np.array_equal(yb[:, pick, :].reshape(-1), yref), "D4 blocks of the sampled rows must be bit-exact"
+    got = run_gemm(dw, dy, rows, cols, batch)
+    assert np.isfinite(got).all()
+    rng = np.random.default_rng(79)
+    n = 30000
+    sr = rng.integers(0, rows, n, dtype=np.uint32)
+    sj = rng.integers(0, batch, n, dtype=np.uint32)
+    rc, ref_s, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, sr, sj)
+    assert_close_fp32(got[sj, sr], ref_s, absum, "gemm heavy tail (sampled)")
+    d4_block_dots(oracle, dw, w, dy, y, rows, cols, batch, seed=80, n=1024)
+
+
 def test_gemm_reference_tolerance_restated(gpu):
     """tests/mmq_parity.cu:246-254 restated: output vs fp32 dot of the dequantised
     operands within 5e-3 abs or 1e-3 rel, U(-0.5,0.5) weights and U(-1,1) activations."""
