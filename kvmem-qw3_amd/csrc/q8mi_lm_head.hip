@@ -310,15 +310,23 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
     auto kern = lm_head_mfma_kernel<MG, THREADS>;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     const uint32_t units = (rows + kMfmaUnitRows - 1) / kMfmaUnitRows;
-    uint32_t grid = units < cus ? units : cus;     // the geometry of the GEMV's matrix-core launch
-    if (grid > kMaxPartials) grid = kMaxPartials;
+    // One workgroup per CU, the geometry of the GEMV's matrix-core launch, when the sums its waves
+    // park fit LDS; a very tall weight (the full vocabulary at 5..8 rows) takes 2..4 workgroups per
+    // CU instead, which run one after the other.
     const uint32_t x_bytes = mfma_x_lds_bytes(nb, batch, MG);
     const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
-    const uint32_t per_group = (units + grid - 1) / grid;
-    const uint32_t park_floats = max_units_touched(per_group, nitems, THREADS / kWave) * mfma_park_floats_per_unit(MG);
-    const uint32_t lds = x_bytes + (THREADS / kWave) * park_floats * 4;
     constexpr uint32_t kDynLimit = kLdsLimit - THREADS * 8 - 256;   // static LDS: the argmax tree and a few words
-    if (lds > kDynLimit) return fail(Q8MI_REJECTED, "lm_head (matrix-core variant): %u bytes of LDS needed", lds);
+    uint32_t grid = 0, park_floats = 0, lds = 0;
+    for (uint32_t mult = 1; mult <= 4; ++mult) {
+        uint32_t g = cus * mult;
+        if (g > units) g = units;
+        if (g > kMaxPartials) g = kMaxPartials;
+        const uint32_t per_group = (units + g - 1) / g;
+        const uint32_t pf = max_units_touched(per_group, nitems, THREADS / kWave) * mfma_park_floats_per_unit(MG);
+        const uint32_t need = x_bytes + (THREADS / kWave) * pf * 4;
+        if (need <= kDynLimit) { grid = g; park_floats = pf; lds = need; break; }
+    }
+    if (grid == 0) return fail(Q8MI_REJECTED, "lm_head (matrix-core variant): the parked sums do not fit LDS");
     static thread_local bool granted = false;
     if (lds > 64u * 1024u && !granted) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -334,12 +342,15 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
     return check_launch("lm_head");
 }
 
-// Same routing rule as the GEMV: matrix-core variant from gemv_tuning().mfma_from rows on, when
-// the activations fit LDS in its layout.
-bool lm_head_uses_mfma(uint32_t nb, uint32_t batch) {
+// Matrix-core variant: for weights of up to 65536 rows under the GEMV's own rule (same kernel
+// family and geometry as q8mi_gemv at that batch, so the optional logits are the GEMV's bits), for
+// taller ones (the vocabulary) only from 7 verify rows on: there the dot-product variant streams
+// faster up to 6 rows (measured: 238..257 us against 248..267 us at 4..6 rows, 296 against 279 at 8).
+bool lm_head_uses_mfma(uint32_t rows, uint32_t nb, uint32_t batch) {
     const uint32_t mg = (batch + 3) / 4;
-    return batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) &&
-           mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u <= kLdsLimit - 256;
+    if (batch < static_cast<uint32_t>(gemv_tuning().mfma_from)) return false;
+    if (mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u > kLdsLimit - 256) return false;
+    return rows <= 65536u || batch >= 7;
 }
 
 template <int M>
@@ -393,7 +404,7 @@ extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, 
     const auto *yb = static_cast<const uint8_t *>(y);
     hipStream_t s = as_stream(stream);
     int rc = Q8MI_REJECTED;
-    if (lm_head_uses_mfma(nb, batch)) {
+    if (lm_head_uses_mfma(rows, nb, batch)) {
         rc = batch <= 4 ? launch_lm_head_mfma<1>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s)
                         : launch_lm_head_mfma<2>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s);
     }
