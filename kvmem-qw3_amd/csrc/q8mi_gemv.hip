@@ -190,7 +190,7 @@ __device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, flo
 // ---- matrix-core variant for batch 3..32 (see q8mi_gemv_mfma_core.hpp) --------------------------
 // Unit u covers rows 4u .. 4u+3 of the concatenated row space; for SwiGLU gate rows 2u, 2u+1
 // (fragment rows 0, 1) and the matching up rows (fragment rows 2, 3).
-template <int MG, int THREADS, bool SILU, bool HS>
+template <int MG, int THREADS, bool SILU, bool HS, bool D4>
 __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, uint32_t batch,
                                                             uint32_t park_floats) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
 #ifdef Q8MI_TRACE
     const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
 #endif
-    mfma_stream<MG, THREADS, HS>(smem, p.y, p.nb, batch, useq, i0, i1, row_ptr, park);
+    mfma_stream<MG, THREADS, HS, D4>(smem, p.y, p.nb, batch, useq, i0, i1, row_ptr, park);
 #ifdef Q8MI_TRACE
     const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
 #endif
@@ -407,10 +407,10 @@ int launch_m(const GemvParams &p, hipStream_t stream) {
 
 // One workgroup of 512 threads per CU: its eight waves split the items of its units evenly, so a
 // matrix only needs as many 4-row units as there are CUs to keep the chip busy.
-template <int MG, bool SILU, bool HS>
+template <int MG, bool SILU, bool HS, bool D4 = false>
 int launch_mfma(GemvParams p, uint32_t batch, hipStream_t stream) {
     constexpr int THREADS = 512;
-    auto kern = gemv_mfma_kernel<MG, THREADS, SILU, HS>;
+    auto kern = gemv_mfma_kernel<MG, THREADS, SILU, HS, D4>;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
     p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG, HS);
@@ -545,6 +545,26 @@ GemvTuning gemv_tuning() {
         return t;
     };
     return live ? read() : GemvTuning{2, 1, 0, kMfmaFromBatch};
+}
+
+// D4-quantized activations, batch 1..16, through the matrix-core GEMV: what the GEMM entry points
+// use for batches too small for an MFMA tile.  Q8MI_REJECTED when the activations do not fit LDS.
+int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, uint32_t cols, uint32_t batch,
+                 uint32_t stride_dst_row, hipStream_t stream) {
+    const uint32_t nb = cols / kQK;
+    if (nb % 8 != 0 || batch == 0 || batch > 16)
+        return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): cols %u / batch %u not served", cols, batch);
+    const uint32_t mg = (batch + 3) / 4;
+    // D4 scales are fp32 values: only the fp32 scale table keeps them exact
+    if (mfma_x_lds_bytes(nb, batch, mg, false) + 16u * 1024u > kLdsLimit - 256)
+        return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): activations do not fit LDS");
+    const GemvParams p = single(w, XSource{y_d4, nullptr, 0}, dst, rows, cols, stride_dst_row, kStoreF32);
+    switch (mg) {
+        case 1: return launch_mfma<1, false, false, true>(p, batch, stream);
+        case 2: return launch_mfma<2, false, false, true>(p, batch, stream);
+        case 3: return launch_mfma<3, false, false, true>(p, batch, stream);
+        default: return launch_mfma<4, false, false, true>(p, batch, stream);
+    }
 }
 
 // Any batch through the GEMV kernels, eight activation rows per launch.  Used by

@@ -1,4 +1,4 @@
-// Matrix-core variant of the Q8_0 x Q8_1 GEMV for small batches (3 .. 32
+// Matrix-core variant of the Q8_0 x Q8_1 GEMV for small batches (3 .. 16
 // activation rows), shared by the GEMV family and the fused LM-head kernel.
 //
 // From batch 3 on the dot-product GEMV is bound by its VALU work (eight dot4 per
@@ -130,6 +130,56 @@ __device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__res
     __syncthreads();
 }
 
+// The same LDS image from D4 activation blocks ([k / 128][batch] records of 16 B fp32 scales +
+// 128 B int8, the prefill GEMM's input), for batches the GEMM entry points hand to this kernel.
+template <int MG, int THREADS>
+__device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb,
+                                                uint32_t batch) {
+    constexpr uint32_t MP = 4 * MG;
+    constexpr int kBatch = 4;
+    const uint32_t row_pitch = mfma_xq_row_pitch(nb);
+    uint8_t *xq = smem;
+    uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
+    const uint32_t nsb = nb / 4;
+    const uint32_t per_sb = batch * 9;           // 16-byte chunks per super-block: batch records of 9
+    const uint32_t total = nsb * per_sb;
+    const v4i *src = reinterpret_cast<const v4i *>(y);   // records are 16-byte aligned by construction
+    auto put = [&](uint32_t sb, uint32_t cc, const v4i &v) {   // cc: chunk inside super-block sb
+        const uint32_t j = cc / 9, part = cc % 9;
+        if (part == 0) {
+            const int d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t kb = 4 * sb + t;
+                *reinterpret_cast<int *>(xd + (kb * MP + j) * 4) = d[t];
+            }
+        } else {
+            *reinterpret_cast<v4i *>(xq + j * row_pitch + sb * 128 + (part - 1) * 16) = v;
+        }
+    };
+    for (uint32_t base = 0; base < total; base += THREADS * kBatch) {
+        v4i v[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t c = base + u * THREADS + threadIdx.x;
+            v[u] = src[c < total ? c : 0];
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t c = base + u * THREADS + threadIdx.x;
+            if (c < total) put(c / per_sb, c % per_sb, v[u]);
+        }
+    }
+    if (batch < MP) {
+        const uint32_t pad = MP - batch;
+        for (uint32_t i = threadIdx.x; i < nb * pad; i += THREADS) {
+            const uint32_t kb = i / pad, m = batch + i % pad;
+            *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = 0.0f;
+        }
+    }
+    __syncthreads();
+}
+
 // Streams the items [i0, i1) of the workgroup's unit sequence (item i = part i % nitems of unit
 // i / nitems, nitems = ceil(nb / 32)).
 //   row_ptr(u)             the weight row (scale plane) this lane LOADS for unit u: fragment row lane / 16,
@@ -139,7 +189,7 @@ __device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__res
 //                          meaningful in the lanes with lane / 16 == (lane % 16) / 4; must not touch
 //                          global memory
 // Must be called by every wave of the workgroup (contains the staging barrier).
-template <int MG, int THREADS, bool HS, class RowPtr, class Park>
+template <int MG, int THREADS, bool HS, bool D4, class RowPtr, class Park>
 __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb, uint32_t batch,
                                             const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
                                             Park park) {
@@ -149,7 +199,8 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, m4 = lane & 3u;
     if (i1 <= i0) {
-        mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
+        if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch);
+        else mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
         return;
     }
     const uint32_t n_items = i1 - i0;
@@ -180,7 +231,8 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     };
     issue(items[0]);
     issue(items[1]);
-    mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
+    if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch);
+    else mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
 
     const uint32_t row_pitch = mfma_xq_row_pitch(nb);
     const uint8_t *xq = smem;

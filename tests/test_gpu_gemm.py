@@ -174,6 +174,30 @@ def test_gemm_ragged_and_medium(gpu, oracle, rows, batch, cols):
     assert np.array_equal(got_m.view(np.uint32), got[:, :rows].view(np.uint32))
 
 
+@pytest.mark.parametrize("rows,cols", [(515, 1024), (5120, 5120), (130, 17408), (4, 256)])
+@pytest.mark.parametrize("batch", [1, 3, 4, 7, 8, 9, 12, 13, 16])
+def test_gemm_small_batches_stream_the_weights(gpu, oracle, rows, cols, batch):
+    """Batches of up to 16 rows on D4 activations are served by the weight-streaming matrix-core
+    GEMV (when the activations fit LDS): same contract as the tile kernel."""
+    if rows == 5120 and batch not in (4, 9, 16):
+        pytest.skip("big shape: three batches only")
+    w = synth.q8_0_weight(rows, cols, seed=rows * 5 + cols)
+    x = synth.normal(batch, cols, seed=batch * 3 + cols)
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    rc, ref = oracle.gemm_d4(w, y, rows, cols, batch, threads=8)
+    rr, jj = np.meshgrid(np.arange(rows, dtype=np.uint32), np.arange(batch, dtype=np.uint32))
+    rc, _, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr.reshape(-1), jj.reshape(-1))
+    stride = rows + 5
+    fn = (lambda: run_gemm(dw, dy, rows, cols, batch, stride=stride)) if rows >= 128 else None
+    if fn is None:   # rows < 128 take Q8_1 activations through q8mi_gemm; the D4 form goes through gemm_medium
+        got = run_gemm(dw, dy, rows, cols, batch, stride=stride, medium=True)
+    else:
+        got = fn()
+    assert_close_fp32(got[:, :rows], ref, absum, f"gemm small batch {batch}")
+    assert np.all(got[:, rows:].view(np.uint32) == 0xffffffff), "stores must stay inside the rows"
+
+
 def test_gemm_small_shapes_take_q8_1(gpu, oracle):
     """rows < 128 or cols % 128 != 0: the entry point expects Q8_1 activations, as the
     reference's launcher does for those shapes (src/kernels_cuda.cu:14545-14552)."""
