@@ -41,7 +41,7 @@ namespace q8mi {
 // q8mi_gemv.hip): y is Q8_1, any batch, processed eight activation rows at a time.
 int gemv_any_batch(const uint8_t *w, const void *y_q8_1, float *dst, uint32_t rows, uint32_t cols,
                    uint32_t batch, uint32_t stride_dst_row, hipStream_t stream);
-// Matrix-core GEMV on D4 activations (q8mi_gemv.hip): batch <= 16 that fits LDS, else Q8MI_REJECTED.
+// Matrix-core GEMV on D4 activations (q8mi_gemv.hip): small batches, else Q8MI_REJECTED.
 int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, uint32_t cols, uint32_t batch,
                  uint32_t stride_dst_row, hipStream_t stream);
 
@@ -538,9 +538,9 @@ int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
 
 int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,
                    uint32_t batch, uint32_t stride, hipStream_t stream) {
-    // up to 16 activation rows: the weight-streaming matrix-core GEMV, which reads the weights once
-    // at HBM speed instead of padding the batch to a 128-wide tile
-    if (batch <= 16 && (cols / kQK) % 8 == 0) {
+    // small batches: the weight-streaming matrix-core GEMV, which reads the weights at HBM speed
+    // instead of padding the batch to a 128-wide tile (it declines what tiles serve better)
+    if (batch <= 32 && (cols / kQK) % 8 == 0) {
         const int rc = gemv_mfma_d4(w, y, dst, rows, cols, batch, stride, stream);
         if (rc != Q8MI_REJECTED) return rc;
     }

@@ -237,7 +237,7 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
 #ifdef Q8MI_TRACE
     const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
 #endif
-    mfma_stream<MG, THREADS, HS, D4>(smem, p.y, p.nb, batch, useq, i0, i1, row_ptr, park);
+    mfma_stream<MG, THREADS, HS, D4>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
 #ifdef Q8MI_TRACE
     const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
 #endif
@@ -547,24 +547,37 @@ GemvTuning gemv_tuning() {
     return live ? read() : GemvTuning{2, 1, 0, kMfmaFromBatch};
 }
 
-// D4-quantized activations, batch 1..16, through the matrix-core GEMV: what the GEMM entry points
-// use for batches too small for an MFMA tile.  Q8MI_REJECTED when the activations do not fit LDS.
+// D4-quantized activations through the matrix-core GEMV: what the GEMM entry points use for
+// batches too small for an MFMA tile.  As many activation rows per launch as fit LDS (at most 16);
+// a batch is cut into that many rows at a time, each slice streaming the weights once, for as many
+// passes as measured faster than tiles (two of 16 rows, four of fewer).  Q8MI_REJECTED otherwise
+// (the caller then uses tiles).
 int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, uint32_t cols, uint32_t batch,
                  uint32_t stride_dst_row, hipStream_t stream) {
     const uint32_t nb = cols / kQK;
-    if (nb % 8 != 0 || batch == 0 || batch > 16)
-        return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): cols %u / batch %u not served", cols, batch);
-    const uint32_t mg = (batch + 3) / 4;
+    if (nb % 8 != 0 || batch == 0) return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): cols %u not served", cols);
     // D4 scales are fp32 values: only the fp32 scale table keeps them exact
-    if (mfma_x_lds_bytes(nb, batch, mg, false) + 16u * 1024u > kLdsLimit - 256)
-        return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): activations do not fit LDS");
-    const GemvParams p = single(w, XSource{y_d4, nullptr, 0}, dst, rows, cols, stride_dst_row, kStoreF32);
-    switch (mg) {
-        case 1: return launch_mfma<1, false, false, true>(p, batch, stream);
-        case 2: return launch_mfma<2, false, false, true>(p, batch, stream);
-        case 3: return launch_mfma<3, false, false, true>(p, batch, stream);
-        default: return launch_mfma<4, false, false, true>(p, batch, stream);
+    uint32_t fit = 0;
+    for (uint32_t m = 16; m >= 4; m -= 4) {
+        if (mfma_x_lds_bytes(nb, m, m / 4, false) + 16u * 1024u <= kLdsLimit - 256) { fit = m; break; }
     }
+    if (fit == 0 || batch > (fit >= 16 ? 2u : 4u) * fit)
+        return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): batch %u at %u columns is served by tiles", batch, cols);
+    const auto *y = static_cast<const uint8_t *>(y_d4);
+    for (uint32_t j0 = 0; j0 < batch; j0 += fit) {
+        const uint32_t m = batch - j0 < fit ? batch - j0 : fit;
+        GemvParams p = single(w, XSource{y + static_cast<uint64_t>(j0) * kD4Bytes, nullptr, batch},
+                              dst + static_cast<uint64_t>(j0) * stride_dst_row, rows, cols, stride_dst_row, kStoreF32);
+        int rc;
+        switch ((m + 3) / 4) {
+            case 1: rc = launch_mfma<1, false, false, true>(p, m, stream); break;
+            case 2: rc = launch_mfma<2, false, false, true>(p, m, stream); break;
+            case 3: rc = launch_mfma<3, false, false, true>(p, m, stream); break;
+            default: rc = launch_mfma<4, false, false, true>(p, m, stream); break;
+        }
+        if (rc != Q8MI_OK) return rc;
+    }
+    return Q8MI_OK;
 }
 
 // Any batch through the GEMV kernels, eight activation rows per launch.  Used by

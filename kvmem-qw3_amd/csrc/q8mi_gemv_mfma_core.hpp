@@ -133,8 +133,9 @@ __device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__res
 // The same LDS image from D4 activation blocks ([k / 128][batch] records of 16 B fp32 scales +
 // 128 B int8, the prefill GEMM's input), for batches the GEMM entry points hand to this kernel.
 template <int MG, int THREADS>
+// y points at the first of the `batch` records staged; a super-block holds batch_total records.
 __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb,
-                                                uint32_t batch) {
+                                                uint32_t batch, uint32_t batch_total) {
     constexpr uint32_t MP = 4 * MG;
     constexpr int kBatch = 4;
     const uint32_t row_pitch = mfma_xq_row_pitch(nb);
@@ -162,7 +163,8 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *__
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const uint32_t c = base + u * THREADS + threadIdx.x;
-            v[u] = src[c < total ? c : 0];
+            const uint32_t cc = c < total ? c : 0;
+            v[u] = src[static_cast<uint64_t>(cc / per_sb) * batch_total * 9 + cc % per_sb];
         }
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
@@ -191,7 +193,7 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *__
 // Must be called by every wave of the workgroup (contains the staging barrier).
 template <int MG, int THREADS, bool HS, bool D4, class RowPtr, class Park>
 __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb, uint32_t batch,
-                                            const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
+                                            uint32_t d4_batch_total, const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
                                             Park park) {
     constexpr uint32_t MP = 4 * MG;
     constexpr float kMagic = 12582912.0f;
@@ -199,7 +201,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, m4 = lane & 3u;
     if (i1 <= i0) {
-        if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch);
+        if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch, d4_batch_total);
         else mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
         return;
     }
@@ -231,7 +233,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     };
     issue(items[0]);
     issue(items[1]);
-    if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch);
+    if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch, d4_batch_total);
     else mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
 
     const uint32_t row_pitch = mfma_xq_row_pitch(nb);

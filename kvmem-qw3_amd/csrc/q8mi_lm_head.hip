@@ -159,7 +159,7 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
             }
         }
     };
-    mfma_stream<MG, THREADS, false, false>(smem, y, nb, batch, useq, i0, i1, row_ptr, park);
+    mfma_stream<MG, THREADS, false, false>(smem, y, nb, batch, 0, useq, i0, i1, row_ptr, park);
     __syncthreads();
 
     __shared__ uint32_t s_kf[kWaves], s_kl[kWaves];

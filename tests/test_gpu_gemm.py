@@ -175,11 +175,11 @@ def test_gemm_ragged_and_medium(gpu, oracle, rows, batch, cols):
 
 
 @pytest.mark.parametrize("rows,cols", [(515, 1024), (5120, 5120), (130, 17408), (4, 256)])
-@pytest.mark.parametrize("batch", [1, 3, 4, 7, 8, 9, 12, 13, 16])
+@pytest.mark.parametrize("batch", [1, 3, 4, 7, 8, 9, 12, 13, 16, 17, 29, 32])
 def test_gemm_small_batches_stream_the_weights(gpu, oracle, rows, cols, batch):
     """Batches of up to 16 rows on D4 activations are served by the weight-streaming matrix-core
     GEMV (when the activations fit LDS): same contract as the tile kernel."""
-    if rows == 5120 and batch not in (4, 9, 16):
+    if rows == 5120 and batch not in (4, 9, 16, 29):
         pytest.skip("big shape: three batches only")
     w = synth.q8_0_weight(rows, cols, seed=rows * 5 + cols)
     x = synth.normal(batch, cols, seed=batch * 3 + cols)
