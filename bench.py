@@ -141,6 +141,27 @@ def time_loop(hip, fn, steps, warmup):
     return e0.elapsed_ms(e1) / steps
 
 
+def time_graph_replays(hip, record, steps, warmup):
+    """Device time per replay of the launches `record(stream)` makes, captured once as a HIP graph
+    on a stream of its own (events recorded on that stream)."""
+    stream = hip.Stream()
+    record(stream.handle)            # eager once: first-use set-up of every kernel happens outside the capture
+    stream.synchronize()
+    g = hip.Graph(stream)
+    with g:
+        record(stream.handle)
+    for _ in range(warmup):
+        g.launch()
+    stream.synchronize()
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record(stream)
+    for _ in range(steps):
+        g.launch()
+    e1.record(stream)
+    e1.synchronize()
+    return e0.elapsed_ms(e1) / steps
+
+
 def time_each_launch(hip, fn, n, warmup=5):
     """Average duration of single launches, one event pair per launch."""
     for i in range(warmup):
@@ -322,6 +343,13 @@ def main():
     }
 
     if not args.quick:
+        # the same step captured once as a HIP graph (all four weight sets in one graph) and replayed
+        def record(stream):
+            for l in layers:
+                step.run(l, stream)
+        ms_graph = time_graph_replays(hip, record, max(args.steps // len(layers), 10), 3) / len(layers)
+        result["graph_replay"] = {"ms_per_step": round(ms_graph, 5),
+                                  "gbps": round(step_bytes / (ms_graph * 1e-3) / 1e9, 1)}
         sweep = {}
         for m in (1, 2, 4, 6, 8):
             st = step if m == 1 else DecodeStep(q8mi, hip, m=m)

@@ -142,6 +142,40 @@ class Stream:
             pass
 
 
+class Graph:
+    """A stream capture turned into an executable graph: with Graph(stream): ...launches...; then
+    graph.launch() replays them on that stream."""
+
+    def __init__(self, stream):
+        self._stream = stream
+        self._graph = C.c_void_p(0)
+        self._exec = C.c_void_p(0)
+
+    def __enter__(self):
+        check(rt().hipStreamBeginCapture(self._stream.handle, 1), "hipStreamBeginCapture")   # thread-local mode
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        code = rt().hipStreamEndCapture(self._stream.handle, C.byref(self._graph))
+        if exc_type is None:
+            check(code, "hipStreamEndCapture")
+            check(rt().hipGraphInstantiate(C.byref(self._exec), self._graph, None, None, C.c_size_t(0)),
+                  "hipGraphInstantiate")
+        return False
+
+    def launch(self):
+        check(rt().hipGraphLaunch(self._exec, self._stream.handle), "hipGraphLaunch")
+
+    def __del__(self):
+        try:
+            if self._exec.value:
+                rt().hipGraphExecDestroy(self._exec)
+            if self._graph.value:
+                rt().hipGraphDestroy(self._graph)
+        except Exception:
+            pass
+
+
 class Event:
     def __init__(self):
         self._e = C.c_void_p(0)
