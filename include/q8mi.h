@@ -149,6 +149,26 @@ int q8mi_block_dots(const uint8_t *weight, const void *y, int y_layout, uint32_t
                     const uint32_t *sample_j, const uint32_t *sample_kb, uint32_t n, int32_t *out,
                     void *stream);
 
+/* ---- dequantizing row gather (embedding lookup) ---------------------------- */
+/* out[i] = fp32(d[i / 32]) * q[i] of one row, fp32 or (out_is_bf16) bf16 rounded
+ * to nearest even.  Bit-exact: the product is exact in fp32.  All three need a
+ * 4-byte aligned matrix and a 16-byte (bf16: 8-byte) aligned output.
+ * replaces q8_get_row_kernel / q8_get_row_bf16_kernel, src/kernels_cuda.cu:2075-2108
+ * (launched :10636-10650).  A row outside the matrix is REJECTED. */
+int q8mi_get_row(const uint8_t *weight, uint64_t row, uint64_t rows, uint64_t cols, void *out,
+                 int out_is_bf16, void *stream);
+/* replaces q8_get_row_from_argmax_kernel, src/kernels_cuda.cu:2110-2134 (launched
+ * :10704-10711): the row id is argmaxes[index].index, read on the device; an id
+ * below zero or beyond the matrix gives a row of zeros. */
+int q8mi_get_row_from_argmax(const uint8_t *weight, const q8mi_argmax_pair *argmaxes, uint32_t index,
+                             uint64_t rows, uint64_t cols, float *out, void *stream);
+/* replaces q8_get_rows_batch_kernel / q8_get_rows_batch_bf16_kernel,
+ * src/kernels_cuda.cu:2141-2190 (launched :10747-10755): row_ids is a DEVICE array
+ * of `batch` ids, out holds batch rows of cols elements.  An id beyond the matrix
+ * gives a row of zeros (the reference reads out of bounds there). */
+int q8mi_get_rows(const uint8_t *weight, const uint64_t *row_ids, uint32_t batch, uint64_t rows,
+                  uint64_t cols, void *out, int out_is_bf16, void *stream);
+
 /* ---- argmax -------------------------------------------------------------- */
 /* replaces argmax_kernel, src/kernels_cuda.cu:1693-1734 (launched at :20759):
  * out2[0] = index (-1 if no element is above -inf), out2[1] = bits of the max. */

@@ -84,7 +84,7 @@ HipQ8Backend::HipQ8Backend() {
 
 HipQ8Backend::~HipQ8Backend() {
     if (stream_) (void)hipStreamSynchronize(stream_);
-    for (Scratch *s : {&q8_1_, &d4_, &argmax_partial_, &argmax_result_, &lm_head_, &lm_rows_, &out_f32_}) {
+    for (Scratch *s : {&q8_1_, &d4_, &argmax_partial_, &argmax_result_, &lm_head_, &lm_rows_, &out_f32_, &row_ids_}) {
         if (s->ptr) (void)hipFree(s->ptr);
     }
     if (argmax_dev_) (void)hipFree(argmax_dev_);
@@ -473,6 +473,49 @@ DeviceStatus HipQ8Backend::argmax_to_buffer(const DeviceTensor &x, DeviceArgmaxB
     if (q8mi_argmax_to_pair(T(x).f32(), T(x).count, dst.ptr, index, stream_) != Q8MI_OK)
         return failed("argmax_to_pair");
     return launch_status("hip argmax_to_buffer");
+}
+
+DeviceStatus HipQ8Backend::q8_0_get_row(DeviceTensor &out, const DeviceWeight &weight, uint64_t row) {
+    const auto &w = W(weight);
+    auto &o = T(out);
+    if (w.format != DeviceWeightFormat::Q8_0) return {false, "row lookup requires Q8_0 weight"};
+    if (o.count < w.cols) return {false, "q8_0_get_row: output smaller than a row"};
+    if (row >= w.rows) return {false, "q8_0_get_row: row outside the matrix"};
+    if (q8mi_get_row(w.ptr, row, w.rows, w.cols, o.ptr, o.is_bf16() ? 1 : 0, stream_) != Q8MI_OK)
+        return failed("get_row");
+    return launch_status("hip q8_0_get_row");
+}
+
+DeviceStatus HipQ8Backend::q8_0_get_row_from_argmax(DeviceTensor &out, const DeviceWeight &weight,
+                                                    const DeviceArgmaxBuffer &argmaxes, uint32_t index) {
+    const auto &w = W(weight);
+    auto &o = T(out);
+    const auto &a = static_cast<const HipArgmaxBuffer &>(argmaxes);
+    if (index >= a.count) return {false, "q8_0_get_row_from_argmax index oob"};
+    if (w.format != DeviceWeightFormat::Q8_0) return {false, "argmax row lookup requires Q8_0 weight"};
+    if (o.is_bf16()) return {false, "q8_0_get_row_from_argmax: fp32 output only"};
+    if (o.count < w.cols) return {false, "q8_0_get_row_from_argmax: output smaller than a row"};
+    if (q8mi_get_row_from_argmax(w.ptr, a.ptr, index, w.rows, w.cols, o.f32(), stream_) != Q8MI_OK)
+        return failed("get_row_from_argmax");
+    return launch_status("hip q8_0_get_row_from_argmax");
+}
+
+DeviceStatus HipQ8Backend::q8_0_get_rows_batch(DeviceTensor &out, const DeviceWeight &weight,
+                                               const uint64_t *rows, uint32_t batch) {
+    if (batch == 0) return {};
+    const auto &w = W(weight);
+    auto &o = T(out);
+    if (w.format != DeviceWeightFormat::Q8_0) return {false, "batched row lookup requires Q8_0 weight"};
+    if (o.count < static_cast<uint64_t>(batch) * w.cols) return {false, "q8_0_get_rows_batch: output too small"};
+    // grow-only device copy of the ids (src/kernels_cuda.cu:10722-10727)
+    if (auto st = ensure(row_ids_, batch * sizeof(uint64_t), "row id buffer"); !st.ok) return st;
+    if (auto st = hip_status(hipMemcpyAsync(row_ids_.ptr, rows, batch * sizeof(uint64_t), hipMemcpyHostToDevice,
+                                            stream_), "row id upload"); !st.ok)
+        return st;
+    if (q8mi_get_rows(w.ptr, static_cast<const uint64_t *>(row_ids_.ptr), batch, w.rows, w.cols, o.ptr,
+                      o.is_bf16() ? 1 : 0, stream_) != Q8MI_OK)
+        return failed("get_rows");
+    return launch_status("hip q8_0_get_rows_batch");
 }
 
 DeviceStatus HipQ8Backend::copy_argmax_buffer_to_host(const DeviceArgmaxBuffer &src, DeviceArgmax *host,

@@ -121,6 +121,16 @@ public:
     DeviceStatus argmax_batch(const DeviceTensor &x, uint32_t batch, uint32_t row_stride,
                               std::vector<DeviceArgmax> &out);
 
+    // embedding lookup: dequantized rows of a Q8_0 matrix
+    // (include/qw3/device_backend.hpp:276-299, src/kernels_cuda.cu:10613-10755).
+    // `out` may be fp32 or bf16; the argmax variant is fp32 only and yields zeros
+    // when the slot holds no valid token.  `rows` of the batch variant is a HOST array.
+    DeviceStatus q8_0_get_row(DeviceTensor &out, const DeviceWeight &weight, uint64_t row);
+    DeviceStatus q8_0_get_row_from_argmax(DeviceTensor &out, const DeviceWeight &weight,
+                                          const DeviceArgmaxBuffer &argmaxes, uint32_t index);
+    DeviceStatus q8_0_get_rows_batch(DeviceTensor &out, const DeviceWeight &weight, const uint64_t *rows,
+                                     uint32_t batch);
+
     // New op (no counterpart in the reference): the whole verify tail in one pass
     // over the LM-head weights.  Equivalent to q8_0_matmul(logits, w_out, norm, batch,
     // in_stride, vocab) + argmax_batch + the greedy accept loop
@@ -145,7 +155,7 @@ private:
                             uint32_t out_stride);
 
     hipStream_t stream_ = nullptr;
-    Scratch q8_1_, d4_, argmax_partial_, argmax_result_, lm_head_, lm_rows_, out_f32_;
+    Scratch q8_1_, d4_, argmax_partial_, argmax_result_, lm_head_, lm_rows_, out_f32_, row_ids_;
     int32_t *argmax_dev_ = nullptr;    // {token, logit bits}
     int32_t *argmax_host_ = nullptr;   // pinned mirror
     int32_t *accept_dev_ = nullptr;    // {accepted, next}

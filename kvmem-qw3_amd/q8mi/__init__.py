@@ -48,6 +48,9 @@ SIGNATURES = {
     "q8mi_gemm_medium": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_f32_to_bf16": (_int, [_vp, _vp, _u64, _vp]),
     "q8mi_block_dots": (_int, [_u8p, _vp, _int, _u32, _u32, _u32, _vp, _vp, _vp, _u32, _vp, _vp]),
+    "q8mi_get_row": (_int, [_u8p, _u64, _u64, _u64, _vp, _int, _vp]),
+    "q8mi_get_row_from_argmax": (_int, [_u8p, _vp, _u32, _u64, _u64, _vp, _vp]),
+    "q8mi_get_rows": (_int, [_u8p, _vp, _u32, _u64, _u64, _vp, _int, _vp]),
     "q8mi_argmax": (_int, [_vp, _u64, _vp, _vp]),
     "q8mi_argmax_to_pair": (_int, [_vp, _u64, _vp, _u32, _vp]),
     "q8mi_argmax_rows_scratch_bytes": (C.c_size_t, [_u32, _u32]),

@@ -168,6 +168,19 @@ static float amax32(const float *x) {
     return m;
 }
 
+int q8o_get_row(const uint8_t *w_split, uint64_t row, uint64_t cols, float *out) {
+    if (cols % Q8O_QK != 0) return -1;
+    const uint64_t nb = cols / Q8O_QK;
+    const uint8_t *base = w_split + row * nb * Q8O_Q8_0_BYTES;
+    const int8_t *qs = (const int8_t *)(base + 2 * nb);
+    for (uint64_t i = 0; i < cols; ++i) {
+        uint16_t h;
+        memcpy(&h, base + 2 * (i / Q8O_QK), 2);
+        out[i] = q8o_f16_to_f32(h) * (float)qs[i];
+    }
+    return 0;
+}
+
 int q8o_quantize_q8_1(const float *x, uint32_t batch, uint32_t cols, uint32_t stride_x_row,
                       uint8_t *y) {
     if (cols % Q8O_QK != 0) return -1;

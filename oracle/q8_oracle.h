@@ -18,6 +18,7 @@
  *   q8o_quantize_q8_0 ........... independent numpy restatement, invariants
  *   q8o_repack_split_plane ...... byte-level numpy restatement, round trip
  *   q8o_quantize_q8_1 / _d4 ..... independent numpy restatement, closed forms
+ *   q8o_get_row ................. numpy restatement (d * q is exact in fp32)
  *   q8o_block_dot ............... int64 brute force, extreme values
  *   q8o_gemv*, q8o_gemm_d4 ...... reference closed form (cols*0.5*x), reference
  *                                 tolerance test restated (5e-3 abs / 1e-3 rel
@@ -67,6 +68,10 @@ int q8o_quantize_q8_0(const float *w, uint64_t rows, uint64_t cols, uint8_t *ggu
  * src/kernels_cuda.cu:1566-1594. */
 int q8o_repack_split_plane(const uint8_t *gguf_blocks, uint64_t rows, uint64_t cols,
                            uint8_t *split);
+
+/* Dequantized row `row` of a split-plane weight: out[i] = fp32(d[i / 32]) * (float)q[i]
+ * (exact: an fp16 value times an 8-bit integer).  src/kernels_cuda.cu:2075-2087. */
+int q8o_get_row(const uint8_t *w_split, uint64_t row, uint64_t cols, float *out);
 
 /* ---- activation quantizers ----------------------------------------------- */
 /* src/mmvq_q8.cu:82-112, 623-640.  y: batch * (cols/32) blocks of 36 B. */

@@ -50,6 +50,7 @@ def lib():
             "q8o_bf16_to_f32": (C.c_float, [C.c_uint16]),
             "q8o_quantize_q8_0": (i32, [f32p, u64, u64, u8p]),
             "q8o_repack_split_plane": (i32, [u8p, u64, u64, u8p]),
+            "q8o_get_row": (i32, [u8p, u64, u64, f32p]),
             "q8o_quantize_q8_1": (i32, [f32p, u32, u32, u32, u8p]),
             "q8o_quantize_q8_1_d4": (i32, [f32p, u32, u32, u32, u8p]),
             "q8o_block_dot": (C.c_int32, [u8p, u8p, i32, u32, u32, u32, u32, u32]),
@@ -125,6 +126,15 @@ def repack_split_plane(gguf, rows, cols):
     rc = lib().q8o_repack_split_plane(_p(gguf, C.c_uint8), rows, cols, _p(out, C.c_uint8))
     if rc != 0:
         raise ValueError("q8o_repack_split_plane rejected the shape")
+    return out
+
+
+def get_row(w, row, cols):
+    w = _c(w, np.uint8)
+    out = np.empty(cols, np.float32)
+    rc = lib().q8o_get_row(_p(w, C.c_uint8), row, cols, _p(out, C.c_float))
+    if rc != 0:
+        raise ValueError("q8o_get_row rejected the shape")
     return out
 
 

@@ -398,6 +398,75 @@ void case_argmax(qw3::HipQ8Backend &b) {
     }
 }
 
+// Embedding lookup: every output is an exact product, so the comparison is on bits.
+void case_get_rows(qw3::HipQ8Backend &b) {
+    std::string d;
+    const uint32_t rows = 3000, cols = 5120;
+    const HostWeight w = make_weight(rows, cols, 91);
+    auto weight = b.weight_q8_0(w.gguf.data(), rows, cols, "embed");
+    auto want_row = [&](uint64_t r) {
+        std::vector<float> v(cols);
+        q8o_get_row(w.split.data(), r, cols, v.data());
+        return v;
+    };
+    auto same_bits = [](const std::vector<float> &a, const float *ref, size_t n) {
+        return std::memcmp(a.data(), ref, n * 4) == 0;
+    };
+
+    auto out = b.tensor_f32(cols, "row");
+    bool ok = weight != nullptr;
+    for (uint64_t r : {0ull, 1234ull, 2999ull}) {
+        ok = ok && require(b.q8_0_get_row(*out, *weight, r), "get_row");
+        ok = ok && same_bits(download_f32(b, *out), want_row(r).data(), cols);
+    }
+    ok = ok && !b.q8_0_get_row(*out, *weight, rows).ok;
+    report("get_row_f32", ok);
+
+    auto outb = b.tensor_bf16(cols, "rowb");
+    ok = require(b.q8_0_get_row(*outb, *weight, 77), "get_row bf16");
+    {
+        std::vector<uint16_t> raw(cols);
+        ok = ok && require(b.copy_bytes_to_host(*outb, raw.data(), 0, cols * 2), "download bf16");
+        const auto ref = want_row(77);
+        for (uint32_t i = 0; i < cols && ok; ++i) ok = raw[i] == q8o_f32_to_bf16(ref[i]);
+    }
+    report("get_row_bf16", ok);
+
+    // chained to an argmax slot: the token of a logits row picks the embedding row
+    auto logits = normal_vec(rows, 92);
+    logits[2024] = 50.0f;
+    auto dl = upload_f32(b, logits);
+    auto buf = b.argmax_buffer(3);
+    ok = buf != nullptr && require(b.argmax_to_buffer(*dl, *buf, 1), "argmax_to_buffer");
+    ok = ok && require(b.q8_0_get_row_from_argmax(*out, *weight, *buf, 1), "get_row_from_argmax");
+    ok = ok && same_bits(download_f32(b, *out), want_row(2024).data(), cols);
+    report("get_row_from_argmax", ok);
+
+    // a slot without a token (all logits -inf -> index -1) gives zeros
+    std::vector<float> none(rows, -INFINITY);
+    auto dn = upload_f32(b, none);
+    ok = require(b.argmax_to_buffer(*dn, *buf, 2), "argmax_to_buffer none");
+    ok = ok && require(b.q8_0_get_row_from_argmax(*out, *weight, *buf, 2), "get_row_from_argmax none");
+    {
+        const auto got = download_f32(b, *out);
+        for (uint32_t i = 0; i < cols && ok; ++i) ok = got[i] == 0.0f && !std::signbit(got[i]);
+    }
+    ok = ok && !b.q8_0_get_row_from_argmax(*out, *weight, *buf, 3).ok;
+    report("get_row_from_argmax_no_token", ok);
+
+    const std::vector<uint64_t> ids = {5, 2999, 0, 5, 1500, 42, 2998};
+    const uint32_t batch = static_cast<uint32_t>(ids.size());
+    auto many = b.tensor_f32(static_cast<size_t>(batch) * cols, "rows");
+    ok = require(b.q8_0_get_rows_batch(*many, *weight, ids.data(), batch), "get_rows_batch");
+    {
+        const auto got = download_f32(b, *many);
+        for (uint32_t j = 0; j < batch && ok; ++j)
+            ok = std::memcmp(got.data() + static_cast<size_t>(j) * cols, want_row(ids[j]).data(), cols * 4) == 0;
+    }
+    ok = ok && b.q8_0_get_rows_batch(*many, *weight, ids.data(), 0).ok;
+    report("get_rows_batch", ok);
+}
+
 void case_lm_head_verify(qw3::HipQ8Backend &b) {
     const uint32_t vocab = 30000, cols = 1024, eos = 5;
     const HostWeight w = make_weight(vocab, cols, 81);
@@ -489,7 +558,7 @@ int main(int argc, char **argv) {
     struct Case { const char *name; void (*fn)(qw3::HipQ8Backend &); };
     const Case cases[] = {
         {"closed_form", case_closed_form}, {"matvec", case_matvec_family}, {"matmul", case_matmul},
-        {"argmax", case_argmax}, {"lm_head", case_lm_head_verify}, {"graph", case_graph_replay},
+        {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"lm_head", case_lm_head_verify}, {"graph", case_graph_replay},
     };
     for (const auto &c : cases) {
         if (!only.empty() && only != c.name) continue;

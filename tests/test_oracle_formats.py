@@ -227,3 +227,23 @@ def test_strided_input(oracle):
     assert np.array_equal(y, np_ref.quantize_q8_1(np.ascontiguousarray(x[:, :256])))
     rc, y = oracle.quantize_q8_1_d4(x, cols=256, stride=300)
     assert np.array_equal(y, np_ref.quantize_d4(np.ascontiguousarray(x[:, :256])))
+
+
+def test_get_row_matches_numpy_unpack(oracle):
+    """d * q is exact in fp32, so an independent unpack of the planes must give the same bits."""
+    rng = np.random.default_rng(21)
+    rows, cols = 37, 96          # odd block count: planes of odd rows are not dword aligned
+    w = rng.standard_normal((rows, cols)).astype(np.float32)
+    w[3, :32] = 0.0
+    ws = oracle.make_weight(w)
+    d, q = np_ref.unpack_weight(ws.reshape(rows, -1), cols)
+    want = (d[:, :, None] * q.astype(np.float32)).reshape(rows, cols)
+    for r in range(rows):
+        got = oracle.get_row(ws, r, cols)
+        assert np.array_equal(got.view(np.uint32), want[r].view(np.uint32))
+        # and it is the dequantization of what quantize_q8_0 stored: within half a step of w,
+        # plus the fp16 rounding of the scale (2^-11 relative) on a quant of up to 127
+        step = d[r].repeat(32)
+        assert np.all(np.abs(got - w[r]) <= step * (0.5 + 127 * 2.0 ** -11) * (1 + 1e-3) + 1e-12)
+    with pytest.raises(ValueError):
+        oracle.get_row(ws, 0, 40)
