@@ -208,6 +208,54 @@ def cpu_baseline(seconds=12.0):
             "value_1core": round(one, 3)}
 
 
+def cpu_gemm_sample(rows=2048, m=2048, cols=HIDDEN):
+    """The oracle's scalar GEMM (D4 activations) on a row slice of the M=2048 gate/up shape,
+    row-parallel on the host cores: a bounded sample of the prefill GEMM's CPU rate."""
+    sys.path.insert(0, ROOT)
+    from oracle import q8_oracle as o
+    from q8mi import synth
+    w = synth.q8_0_weight(rows, cols, seed=99)
+    x = synth.normal(m, cols, seed=98)
+    rc, y = o.quantize_q8_1_d4(x)
+    cores = min(16, os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    o.gemm_d4(w, y, rows, cols, m, threads=cores)
+    dt = time.perf_counter() - t0
+    return {"tops": round(2.0 * m * rows * cols / dt / 1e12, 4), "cores": cores, "seconds": round(dt, 2),
+            "sample": f"oracle q8o_gemm_d4, {rows} of 17408 weight rows x M={m} x K={cols}"}
+
+
+def bench_config0(q8mi, hip, synth, copies=48, reps=480):
+    """BASELINE config 0: one 5120x5120 GEMV at M=1 from fp32 activations (quantizer fused).
+    Streaming: cycles through `copies` weight buffers (1.3 GB, no cache hits); resident: one buffer."""
+    L, ok = q8mi.lib(), q8mi.ok
+    host = synth.q8_0_weight(HIDDEN, HIDDEN, seed=31)
+    ws = [hip.to_device(host) for _ in range(copies)]
+    x = hip.to_device(synth.normal(1, HIDDEN, seed=32))
+    dst = hip.DeviceBuffer(4 * HIDDEN)
+    fn = lambda i: ok(L.q8mi_qgemv(ws[i % copies].ptr, x.ptr, HIDDEN, dst.ptr, 0, HIDDEN, HIDDEN, 1, HIDDEN, None),
+                      "qgemv")
+    one = lambda i: ok(L.q8mi_qgemv(ws[0].ptr, x.ptr, HIDDEN, dst.ptr, 0, HIDDEN, HIDDEN, 1, HIDDEN, None), "qgemv")
+    t_stream = time_loop(hip, fn, reps, copies)
+    t_res = time_loop(hip, one, reps, 10)
+    nbytes = w_bytes(HIDDEN, HIDDEN) + q81_bytes(1, HIDDEN) + 4 * HIDDEN
+    for b in ws + [x, dst]:
+        b.free()
+    return {"bytes": nbytes, "streaming_us": round(t_stream * 1e3, 3),
+            "streaming_gbps": round(nbytes / (t_stream * 1e-3) / 1e9, 1),
+            "resident_us": round(t_res * 1e3, 3), "resident_gbps": round(nbytes / (t_res * 1e-3) / 1e9, 1)}
+
+
+def bench_read_probe(q8mi, hip, nbytes=1 << 30, reps=20):
+    """Measured ceiling of a plain streaming read (every lane 16 bytes per load, grid-stride)."""
+    buf, sink = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(64)
+    fn = lambda i: q8mi.ok(q8mi.lib().q8mi_probe_read(buf.ptr, nbytes, 8, sink.ptr, None), "probe_read")
+    t = time_loop(hip, fn, reps, 3)
+    buf.free()
+    sink.free()
+    return round(nbytes / (t * 1e-3) / 1e9, 1)
+
+
 def bench_gemm(q8mi, hip, synth, reps=10):
     """Prefill GEMM (D4 quantize + MFMA GEMM): M=2048 on the two FFN shapes, M=8192 on gate/up."""
     L, ok = q8mi.lib(), q8mi.ok
@@ -361,10 +409,13 @@ def main():
         for b in l.w.values():
             b.free()
     if not args.quick:
+        result["config0_gemv_m1"] = bench_config0(q8mi, hip, synth)
+        result["hbm_read_probe_gbps"] = bench_read_probe(q8mi, hip)
         result["gemm_int8"] = bench_gemm(q8mi, hip, synth)
         result["lm_head_fused"] = bench_lm_head(q8mi, hip, synth)
     if not (args.quick or args.no_cpu):
         result["cpu_baseline"] = cpu_baseline()
+        result["cpu_baseline"]["gemm_int8"] = cpu_gemm_sample()
     else:
         result["cpu_baseline"] = None
     try:

@@ -393,6 +393,8 @@ int launch_ms(const GemvParams &p, hipStream_t stream) {
         if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXF32, SILU>(p, xb, stream);
         return fail(Q8MI_REJECTED, "qgemv: %u activation rows of %u columns do not fit LDS", M, p.nb * 32);
     }
+    // the LDS staging loads 16 bytes at a time: activations on a 4-byte boundary are read by the lanes
+    if (reinterpret_cast<uintptr_t>(p.y) % 16 != 0) return launch_inst<M, 256, kXGlobal, SILU>(p, 0, stream);
     if (forced == 256 && xb + park_256 <= kLdsLimit) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);
     if (forced == 1024 && xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds, SILU>(p, xb, stream);
     if (xb + park_256 <= 76u * 1024u) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);   // two per CU fit
@@ -469,7 +471,8 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         gemv_unaligned_kernel<<<grid, 256, 0, stream>>>(p, batch);
         return check_launch("gemv_unaligned");
     }
-    if (p.xf == nullptr && batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) &&
+    if (p.xf == nullptr && reinterpret_cast<uintptr_t>(p.y) % 16 == 0 &&
+        batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) &&
         (mfma_fits(p.nb, batch, false) || mfma_fits(p.nb, batch, true))) {
         const int rc = launch_mfma_any(p, batch, stream);
         if (rc != Q8MI_REJECTED) return rc;   // a unit list whose parked sums do not fit: dot-product variant

@@ -76,112 +76,163 @@ __device__ __forceinline__ v4i load_x16_global(const uint8_t *y, uint32_t blk, u
 // before the first one is consumed: staging costs one memory round trip, not
 // one per trip of a load-use loop.  Ends with a workgroup barrier.
 template <int M, int THREADS>
-__device__ __forceinline__ void stage_x_lds(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb) {
-    constexpr int kBatch = 4;   // 16-byte loads in flight per thread
-    const uint32_t nsteps = (nb * 2 + 127) / 128;
-    int *wq = reinterpret_cast<int *>(smem);
-    float *wd = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
-    const uint32_t blocks_padded = nsteps * 64;
-    const uint32_t total_dw = static_cast<uint32_t>(M) * nb * 9;   // multiple of 4: nb % 8 == 0 here
-    const uint32_t total_ch = total_dw / 4;
+struct StageLds {
+    static constexpr int kBatch = 4;   // 16-byte loads in flight per thread
+    v4i v[kBatch];
 
-    auto put = [&](uint32_t g, uint32_t word) {   // g: dword index in the global layout
-        const uint32_t blk_g = g / 9, part = g % 9;
-        const uint32_t m = blk_g / nb, kb = blk_g % nb;
-        const uint32_t blk = m * blocks_padded + kb;
-        if (part == 0) {
-            wd[blk] = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
-        } else {
-            wq[blk * 8 + (part - 1)] = static_cast<int>(word);
-        }
-    };
-    if (reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+    // First trip of loads only: nothing is consumed here, so the caller can put further
+    // loads (its first weight items) behind these before finish() waits for them.
+    // y must be 16-byte aligned (launchers send other activations to the global-memory mode).
+    __device__ __forceinline__ void issue(const uint8_t *y, uint32_t nb) {
+        const uint32_t total_ch = static_cast<uint32_t>(M) * nb * 9 / 4;
         const v4i *src = reinterpret_cast<const v4i *>(y);
-        for (uint32_t base = 0; base < total_ch; base += THREADS * kBatch) {
-            v4i v[kBatch];
 #pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const uint32_t c = base + u * THREADS + threadIdx.x;
-                v[u] = src[c < total_ch ? c : 0];
-            }
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const uint32_t c = base + u * THREADS + threadIdx.x;
-                if (c < total_ch) {
-                    put(4 * c + 0, static_cast<uint32_t>(v[u].x));
-                    put(4 * c + 1, static_cast<uint32_t>(v[u].y));
-                    put(4 * c + 2, static_cast<uint32_t>(v[u].z));
-                    put(4 * c + 3, static_cast<uint32_t>(v[u].w));
-                }
-            }
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t c = u * THREADS + threadIdx.x;
+            v[u] = src[c < total_ch ? c : 0];
         }
-    } else {   // activations that are only 4-byte aligned
-        const uint32_t *src = reinterpret_cast<const uint32_t *>(y);
-        for (uint32_t g = threadIdx.x; g < total_dw; g += THREADS) put(g, src[g]);
     }
-    // zero the padding up to whole steps (blocks nb .. blocks_padded of every row)
-    const uint32_t pad = blocks_padded - nb;
-    for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(M) * pad * 9; i += THREADS) {
-        const uint32_t b = i / 9, part = i % 9;
-        const uint32_t blk = (b / pad) * blocks_padded + nb + b % pad;
-        if (part == 0) wd[blk] = 0.0f; else wq[blk * 8 + (part - 1)] = 0;
-    }
-    __syncthreads();
-}
 
-// Same LDS image as stage_x_lds, produced from fp32 activations: every workgroup quantizes
+    __device__ __forceinline__ void finish(uint8_t *smem, const uint8_t *y, uint32_t nb) {
+        const uint32_t nsteps = (nb * 2 + 127) / 128;
+        int *wq = reinterpret_cast<int *>(smem);
+        float *wd = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
+        const uint32_t blocks_padded = nsteps * 64;
+        const uint32_t total_dw = static_cast<uint32_t>(M) * nb * 9;   // multiple of 4: nb % 8 == 0 here
+        const uint32_t total_ch = total_dw / 4;
+
+        auto put = [&](uint32_t g, uint32_t word) {   // g: dword index in the global layout
+            const uint32_t blk_g = g / 9, part = g % 9;
+            const uint32_t m = blk_g / nb, kb = blk_g % nb;
+            const uint32_t blk = m * blocks_padded + kb;
+            if (part == 0) {
+                wd[blk] = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
+            } else {
+                wq[blk * 8 + (part - 1)] = static_cast<int>(word);
+            }
+        };
+        auto put4 = [&](uint32_t c, const v4i &q) {
+            if (c < total_ch) {
+                put(4 * c + 0, static_cast<uint32_t>(q.x));
+                put(4 * c + 1, static_cast<uint32_t>(q.y));
+                put(4 * c + 2, static_cast<uint32_t>(q.z));
+                put(4 * c + 3, static_cast<uint32_t>(q.w));
+            }
+        };
+        const v4i *src = reinterpret_cast<const v4i *>(y);
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) put4(u * THREADS + threadIdx.x, v[u]);
+        for (uint32_t base = THREADS * kBatch; base < total_ch; base += THREADS * kBatch) {
+            v4i t[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const uint32_t c = base + u * THREADS + threadIdx.x;
+                t[u] = src[c < total_ch ? c : 0];
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) put4(base + u * THREADS + threadIdx.x, t[u]);
+        }
+        // zero the padding up to whole steps (blocks nb .. blocks_padded of every row)
+        const uint32_t pad = blocks_padded - nb;
+        for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(M) * pad * 9; i += THREADS) {
+            const uint32_t b = i / 9, part = i % 9;
+            const uint32_t blk = (b / pad) * blocks_padded + nb + b % pad;
+            if (part == 0) wd[blk] = 0.0f; else wq[blk * 8 + (part - 1)] = 0;
+        }
+        __syncthreads();
+    }
+};
+
+// Same LDS image as StageLds, produced from fp32 activations: every workgroup quantizes
 // the M rows itself (M * cols / 4 float4 loads spread over the workgroup), with the code the
 // stand-alone quantizer uses, so the int8 values and the fp16-rounded scales are the same bits.
 // The block sum `s` of Q8_1 is not needed by Q8_0 dots and is not formed.  x rows are
 // stride_x floats apart; cols = 32 * nb.  Ends with a workgroup barrier.
 template <int M, int THREADS>
-__device__ __forceinline__ void stage_x_f32(uint8_t *smem, const float *__restrict__ x, uint32_t stride_x,
-                                            uint32_t nb) {
-    constexpr int kBatch = 6;   // float4 loads in flight per thread: one trip for a 6144-column row at 256 threads
-    const uint32_t nsteps = (nb * 2 + 127) / 128;
-    uint32_t *wq = reinterpret_cast<uint32_t *>(smem);
-    float *wd = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
-    const uint32_t blocks_padded = nsteps * 64;
-    const uint32_t per_row = nb * 8;                        // float4 chunks per activation row
-    const uint32_t total = static_cast<uint32_t>(M) * per_row;   // multiple of 8: lanes of a block stay together
-    const bool vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride_x % 4 == 0);
-    for (uint32_t base = 0; base < total; base += THREADS * kBatch) {
-        Float4 v[kBatch];
+struct StageF32 {
+    static constexpr int kBatch = 6;   // float4 loads in flight per thread: one trip for a 6144-column row at 256 threads
+    Float4 v[kBatch];
+
+    __device__ __forceinline__ static Float4 fetch(const float *x, uint32_t stride_x, uint32_t per_row,
+                                                   uint32_t total, uint32_t c, bool vec) {
+        const uint32_t cc = c < total ? c : 0;
+        const float *src = x + static_cast<uint64_t>(cc / per_row) * stride_x + (cc % per_row) * 4;
+        return vec ? load4<true>(src) : load4<false>(src);
+    }
+
+    // First trip of loads only (see StageLds::issue).
+    __device__ __forceinline__ void issue(const float *x, uint32_t stride_x, uint32_t nb) {
+        const uint32_t per_row = nb * 8, total = static_cast<uint32_t>(M) * per_row;
+        const bool vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride_x % 4 == 0);
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const uint32_t c = base + u * THREADS + threadIdx.x;
-            const uint32_t cc = c < total ? c : 0;
-            const float *src = x + static_cast<uint64_t>(cc / per_row) * stride_x + (cc % per_row) * 4;
-            v[u] = vec ? load4<true>(src) : load4<false>(src);
-        }
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const uint32_t c = base + u * THREADS + threadIdx.x;
+        for (int u = 0; u < kBatch; ++u) v[u] = fetch(x, stride_x, per_row, total, u * THREADS + threadIdx.x, vec);
+    }
+
+    __device__ __forceinline__ void finish(uint8_t *smem, const float *x, uint32_t stride_x,
+                                           uint32_t nb) {
+        const uint32_t nsteps = (nb * 2 + 127) / 128;
+        uint32_t *wq = reinterpret_cast<uint32_t *>(smem);
+        float *wd = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
+        const uint32_t blocks_padded = nsteps * 64;
+        const uint32_t per_row = nb * 8;                        // float4 chunks per activation row
+        const uint32_t total = static_cast<uint32_t>(M) * per_row;   // multiple of 8: lanes of a block stay together
+        const bool vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride_x % 4 == 0);
+        auto quantize_put = [&](uint32_t c, const Float4 &f) {
             float d;
-            const uint32_t packed = quantize4_q8_1(v[u], d);   // all lanes take part in the exchanges
+            const uint32_t packed = quantize4_q8_1(f, d);   // all lanes take part in the exchanges
             if (c < total) {
                 const uint32_t m = c / per_row, within = c % per_row;
                 const uint32_t blk = m * blocks_padded + within / 8;
                 wq[blk * 8 + within % 8] = packed;
                 if (within % 8 == 0) wd[blk] = half_bits_to_float(float_to_half_bits(d));
             }
+        };
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) quantize_put(u * THREADS + threadIdx.x, v[u]);
+        for (uint32_t base = THREADS * kBatch; base < total; base += THREADS * kBatch) {
+            Float4 t[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) t[u] = fetch(x, stride_x, per_row, total, base + u * THREADS + threadIdx.x, vec);
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) quantize_put(base + u * THREADS + threadIdx.x, t[u]);
         }
+        const uint32_t pad = blocks_padded - nb;
+        for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(M) * pad * 9; i += THREADS) {
+            const uint32_t b = i / 9, part = i % 9;
+            const uint32_t blk = (b / pad) * blocks_padded + nb + b % pad;
+            if (part == 0) wd[blk] = 0.0f; else wq[blk * 8 + (part - 1)] = 0u;
+        }
+        __syncthreads();
     }
-    const uint32_t pad = blocks_padded - nb;
-    for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(M) * pad * 9; i += THREADS) {
-        const uint32_t b = i / 9, part = i % 9;
-        const uint32_t blk = (b / pad) * blocks_padded + nb + b % pad;
-        if (part == 0) wd[blk] = 0.0f; else wq[blk * 8 + (part - 1)] = 0u;
-    }
-    __syncthreads();
-}
+};
 
-// Activations of the workgroup into LDS, by mode (no-op when lanes read them from global memory).
+// Activations of the workgroup into LDS, by mode, in two halves: issue() puts the first trip of
+// activation loads in flight, finish() consumes them (and any further trips) and ends with a
+// workgroup barrier.  Loads return in order, so the weight loads a caller issues between the two
+// stay in flight while the activations are converted.  No-op when lanes read the activations
+// from global memory.
 template <int M, int THREADS, int XMODE>
-__device__ __forceinline__ void stage_x(uint8_t *smem, const uint8_t *__restrict__ y, const float *__restrict__ xf,
+struct XStage {
+    StageLds<M, THREADS> lds;
+    StageF32<M, THREADS> f32;
+    __device__ __forceinline__ void issue(const uint8_t *y, const float *xf,
+                                          uint32_t stride_x, uint32_t nb) {
+        if constexpr (XMODE == kXLds) lds.issue(y, nb);
+        if constexpr (XMODE == kXF32) f32.issue(xf, stride_x, nb);
+    }
+    __device__ __forceinline__ void finish(uint8_t *smem, const uint8_t *y,
+                                           const float *xf, uint32_t stride_x, uint32_t nb) {
+        if constexpr (XMODE == kXLds) lds.finish(smem, y, nb);
+        if constexpr (XMODE == kXF32) f32.finish(smem, xf, stride_x, nb);
+    }
+};
+
+template <int M, int THREADS, int XMODE>
+__device__ __forceinline__ void stage_x(uint8_t *smem, const uint8_t *y, const float *xf,
                                         uint32_t stride_x, uint32_t nb) {
-    if (XMODE == kXLds) stage_x_lds<M, THREADS>(smem, y, nb);
-    if (XMODE == kXF32) stage_x_f32<M, THREADS>(smem, xf, stride_x, nb);
+    XStage<M, THREADS, XMODE> xs;
+    xs.issue(y, xf, stride_x, nb);
+    xs.finish(smem, y, xf, stride_x, nb);
 }
 
 // Weight bytes of one item held by a lane.
@@ -224,7 +275,7 @@ struct XOperand {
 
 template <int XMODE>
 __device__ __forceinline__ XOperand load_x(uint32_t m, uint32_t p1, uint32_t p2, uint32_t kb, bool v1, bool v2,
-                                           bool vk, uint32_t nb, uint32_t nsteps, const uint8_t *__restrict__ y,
+                                           bool vk, uint32_t nb, uint32_t nsteps, const uint8_t *y,
                                            const int *lds_q, const float *lds_d) {
     XOperand o;
     o.x1 = v4i{0, 0, 0, 0};
@@ -253,7 +304,7 @@ __device__ __forceinline__ XOperand load_x(uint32_t m, uint32_t p1, uint32_t p2,
 // while row m is being consumed.
 template <int M, int R, int XMODE>
 __device__ __forceinline__ void compute_item(const Item<R> &it, uint32_t step, uint32_t lane, uint32_t nb,
-                                             uint32_t nsteps, const uint8_t *__restrict__ y, const int *lds_q,
+                                             uint32_t nsteps, const uint8_t *y, const int *lds_q,
                                              const float *lds_d, float (&acc)[M][R]) {
     const uint32_t npieces = nb * 2;
     const uint32_t pa = step * 128 + lane, pb = pa + 64;
@@ -329,8 +380,8 @@ __device__ __forceinline__ UnitSeq group_units(uint32_t units, uint32_t group, u
 // the last item and whose sums are never parked.
 // Must be called by every wave of the workgroup (it contains the staging barrier).
 template <int M, int R, int THREADS, int XMODE, class RowsOf, class Park>
-__device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__restrict__ y,
-                                            const float *__restrict__ xf, uint32_t stride_x, uint32_t nb,
+__device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *y,
+                                            const float *xf, uint32_t stride_x, uint32_t nb,
                                             const UnitSeq &useq, uint32_t i0, uint32_t i1,
                                             RowsOf rows_of, Park park) {
     const uint32_t nsteps = (nb * 2 + 127) / 128;
@@ -345,6 +396,11 @@ __device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__rest
     const uint32_t n_padded = (n_items + kDepth - 1) / kDepth * kDepth;
     const uint32_t k0 = i0 / nsteps, s0 = i0 % nsteps;
 
+    // activation loads first, the first weight items behind them: the activations arrive first
+    // and are converted while the weight loads are still in flight
+    XStage<M, THREADS, XMODE> xs;
+    xs.issue(y, xf, stride_x, nb);
+    asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
     Item<R> items[kDepth];
     // issue cursor: unit ordinal, step, items left to issue for real
     uint32_t ik = k0, istep = s0, ileft = n_items;
@@ -365,7 +421,10 @@ __device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *__rest
         issue_item(items[d], irows, istep, lane, nb);
         advance_issue();
     }
-    stage_x<M, THREADS, XMODE>(smem, y, xf, stride_x, nb);
+    // keeps the loads above where they are: without it the compiler sinks them below the staging
+    // barrier and the first weight bytes are requested only after the activations are in LDS
+    asm volatile("" ::: "memory");
+    xs.finish(smem, y, xf, stride_x, nb);
 
     float acc[M][R];
 #pragma unroll

@@ -69,72 +69,93 @@ struct MfmaItem {
     int d;      // fp16 scales 2 (L % 16), 2 (L % 16) + 1 of the item's 32, row L / 16
 };
 
-// Copies `batch` rows of Q8_1 activations into the LDS image above.  Ends with a barrier.
+// Copies `batch` rows of Q8_1 activations into the LDS image above, in two halves: issue() puts
+// the first trip of loads in flight and consumes nothing, finish() converts them, runs any further
+// trips and ends with a barrier.  Loads return in order, so weight loads the caller issues between
+// the two stay in flight while the first trip is converted.
 template <int MG, int THREADS, bool HS>
-__device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb,
-                                             uint32_t batch) {
-    constexpr uint32_t MP = 4 * MG;
-    constexpr int kBatch = 4;
-    const uint32_t row_pitch = mfma_xq_row_pitch(nb);
-    uint8_t *xq = smem;
-    uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
-    // row by row (a row is nb * 36 bytes, a multiple of 16: nb % 8 == 0), so that locating a dword
-    // needs no division by nb; all loads of a trip are issued before the first is used
-    const uint32_t row_dw = nb * 9, row_ch = row_dw / 4;
-    auto put = [&](uint32_t m, uint32_t g, uint32_t word) {   // g: dword index inside row m
-        const uint32_t kb = g / 9, part = g % 9;
-        if (part == 0) {
-            if (HS) *reinterpret_cast<uint16_t *>(xd + (kb * MP + m) * 2) = static_cast<uint16_t>(word & 0xffffu);
-            else *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
-        } else {
-            *reinterpret_cast<uint32_t *>(xq + m * row_pitch + kb * 32 + (part - 1) * 4) = word;
+struct MfmaStage {
+    static constexpr uint32_t MP = 4 * MG;
+    static constexpr int kBatch = 4;
+    v4i v[kBatch];
+
+    // y must be 16-byte aligned (the launchers use the dot-product kernel otherwise)
+    __device__ __forceinline__ void issue(const uint8_t *y, uint32_t nb, uint32_t batch) {
+        const v4i *src = reinterpret_cast<const v4i *>(y);
+        const uint32_t total_ch = batch * (nb * 9 / 4);
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const uint32_t c = u * THREADS + threadIdx.x;
+            v[u] = src[c < total_ch ? c : 0];
         }
-    };
-    if (reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+    }
+
+    __device__ __forceinline__ void finish(uint8_t *smem, const uint8_t *y, uint32_t nb, uint32_t batch) {
+        const uint32_t row_pitch = mfma_xq_row_pitch(nb);
+        uint8_t *xq = smem;
+        uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
+        // row by row (a row is nb * 36 bytes, a multiple of 16: nb % 8 == 0), so that locating a dword
+        // needs no division by nb; all loads of a trip are issued before the first is used
+        const uint32_t row_dw = nb * 9, row_ch = row_dw / 4;
+        auto put = [&](uint32_t m, uint32_t g, uint32_t word) {   // g: dword index inside row m
+            const uint32_t kb = g / 9, part = g % 9;
+            if (part == 0) {
+                if (HS) *reinterpret_cast<uint16_t *>(xd + (kb * MP + m) * 2) = static_cast<uint16_t>(word & 0xffffu);
+                else *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
+            } else {
+                *reinterpret_cast<uint32_t *>(xq + m * row_pitch + kb * 32 + (part - 1) * 4) = word;
+            }
+        };
         const v4i *src = reinterpret_cast<const v4i *>(y);
         const uint32_t total_ch = batch * row_ch;
-        for (uint32_t base = 0; base < total_ch; base += THREADS * kBatch) {
-            v4i v[kBatch];
+        auto put4 = [&](uint32_t c, const v4i &w) {
+            if (c < total_ch) {
+                uint32_t m = 0, cc = c;                 // batch <= 32: a short subtract loop beats a division
+                while (cc >= row_ch) { cc -= row_ch; ++m; }
+                put(m, 4 * cc + 0, static_cast<uint32_t>(w.x));
+                put(m, 4 * cc + 1, static_cast<uint32_t>(w.y));
+                put(m, 4 * cc + 2, static_cast<uint32_t>(w.z));
+                put(m, 4 * cc + 3, static_cast<uint32_t>(w.w));
+            }
+        };
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) put4(u * THREADS + threadIdx.x, v[u]);
+        for (uint32_t base = THREADS * kBatch; base < total_ch; base += THREADS * kBatch) {
+            v4i t[kBatch];
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 const uint32_t c = base + u * THREADS + threadIdx.x;
-                v[u] = src[c < total_ch ? c : 0];
+                t[u] = src[c < total_ch ? c : 0];
             }
 #pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const uint32_t c = base + u * THREADS + threadIdx.x;
-                if (c < total_ch) {
-                    uint32_t m = 0, cc = c;                 // batch <= 32: a short subtract loop beats a division
-                    while (cc >= row_ch) { cc -= row_ch; ++m; }
-                    put(m, 4 * cc + 0, static_cast<uint32_t>(v[u].x));
-                    put(m, 4 * cc + 1, static_cast<uint32_t>(v[u].y));
-                    put(m, 4 * cc + 2, static_cast<uint32_t>(v[u].z));
-                    put(m, 4 * cc + 3, static_cast<uint32_t>(v[u].w));
-                }
+            for (int u = 0; u < kBatch; ++u) put4(base + u * THREADS + threadIdx.x, t[u]);
+        }
+        // scales of the padding rows batch .. 4 MG - 1 (their products are never stored; keep them finite)
+        if (batch < MP) {
+            const uint32_t pad = MP - batch;
+            for (uint32_t i = threadIdx.x; i < nb * pad; i += THREADS) {
+                const uint32_t kb = i / pad, m = batch + i % pad;
+                if (HS) *reinterpret_cast<uint16_t *>(xd + (kb * MP + m) * 2) = 0;
+                else *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = 0.0f;
             }
         }
-    } else {
-        const uint32_t *src = reinterpret_cast<const uint32_t *>(y);
-        for (uint32_t m = 0; m < batch; ++m)
-            for (uint32_t g = threadIdx.x; g < row_dw; g += THREADS) put(m, g, src[m * row_dw + g]);
+        __syncthreads();
     }
-    // scales of the padding rows batch .. 4 MG - 1 (their products are never stored; keep them finite)
-    if (batch < MP) {
-        const uint32_t pad = MP - batch;
-        for (uint32_t i = threadIdx.x; i < nb * pad; i += THREADS) {
-            const uint32_t kb = i / pad, m = batch + i % pad;
-            if (HS) *reinterpret_cast<uint16_t *>(xd + (kb * MP + m) * 2) = 0;
-            else *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = 0.0f;
-        }
-    }
-    __syncthreads();
+};
+
+template <int MG, int THREADS, bool HS>
+__device__ __forceinline__ void mfma_stage_x(uint8_t *smem, const uint8_t *y, uint32_t nb,
+                                             uint32_t batch) {
+    MfmaStage<MG, THREADS, HS> st;
+    st.issue(y, nb, batch);
+    st.finish(smem, y, nb, batch);
 }
 
 // The same LDS image from D4 activation blocks ([k / 128][batch] records of 16 B fp32 scales +
 // 128 B int8, the prefill GEMM's input), for batches the GEMM entry points hand to this kernel.
 template <int MG, int THREADS>
 // y points at the first of the `batch` records staged; a super-block holds batch_total records.
-__device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb,
+__device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *y, uint32_t nb,
                                                 uint32_t batch, uint32_t batch_total) {
     constexpr uint32_t MP = 4 * MG;
     constexpr int kBatch = 4;
@@ -192,7 +213,7 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *__
 //                          global memory
 // Must be called by every wave of the workgroup (contains the staging barrier).
 template <int MG, int THREADS, bool HS, bool D4, class RowPtr, class Park>
-__device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__restrict__ y, uint32_t nb, uint32_t batch,
+__device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uint32_t nb, uint32_t batch,
                                             uint32_t d4_batch_total, const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
                                             Park park) {
     constexpr uint32_t MP = 4 * MG;
@@ -208,6 +229,11 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     const uint32_t n_items = i1 - i0;
     const uint32_t n_padded = (n_items + 1) / 2 * 2;
 
+    // activation loads first, the first weight items behind them (they stay in flight while the
+    // activations are converted)
+    MfmaStage<MG, THREADS, HS> xstage;
+    if constexpr (!D4) xstage.issue(y, nb, batch);
+    asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
     MfmaItem items[2];
     uint32_t ik = i0 / nitems, istep = i0 % nitems, ileft = n_items;
     const uint8_t *irow = row_ptr(useq.unit(ik));
@@ -233,8 +259,9 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *__rest
     };
     issue(items[0]);
     issue(items[1]);
+    asm volatile("" ::: "memory");   // keeps the loads above from being moved below the staging barrier
     if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch, d4_batch_total);
-    else mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
+    else xstage.finish(smem, y, nb, batch);
 
     const uint32_t row_pitch = mfma_xq_row_pitch(nb);
     const uint8_t *xq = smem;

@@ -360,6 +360,8 @@ int launch_lm_head(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t n
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
     const uint32_t tree_256 = 256 * 8, tree_1024 = 1024 * 8;   // static LDS of the argmax tree
     const int forced = gemv_tuning().threads;
+    if (reinterpret_cast<uintptr_t>(y) % 16 != 0)   // the LDS staging loads 16 bytes at a time
+        return launch_inst<M, 256, kXGlobal>(w, y, rows, nb, 0, partial, logits, stride_logits, grid_out, stream);
     if (forced == 256 && xb + park_256 + tree_256 <= kLdsLimit)
         return launch_inst<M, 256, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
     if (forced == 1024 && xb + park_1024 + tree_1024 <= kLdsLimit)
@@ -404,7 +406,7 @@ extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, 
     const auto *yb = static_cast<const uint8_t *>(y);
     hipStream_t s = as_stream(stream);
     int rc = Q8MI_REJECTED;
-    if (lm_head_uses_mfma(rows, nb, batch)) {
+    if (reinterpret_cast<uintptr_t>(yb) % 16 == 0 && lm_head_uses_mfma(rows, nb, batch)) {
         rc = batch <= 4 ? launch_lm_head_mfma<1>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s)
                         : launch_lm_head_mfma<2>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s);
     }

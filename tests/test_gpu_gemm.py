@@ -104,12 +104,14 @@ def test_gemm_large_tilings(gpu, oracle, rows, batch, cols):
         assert_close_fp32(got[j, :rows], ref_c, absum_c, f"gemm column {j}")
 
 
-def test_gemm_heavy_tail_batch_8192(gpu, oracle):
-    """Long-context prefill shape with heavy-tailed activations: batch 8192, Student-t(3) values
+# the layer's projections: QKV, O, gate/up (one shape), down
+@pytest.mark.parametrize("rows,cols", [(5120, 5120), (8192, 5120), (5120, 6144), (17408, 5120), (5120, 17408)])
+def test_gemm_heavy_tail_batch_8192(gpu, oracle, rows, cols):
+    """Long-context prefill shapes with heavy-tailed activations: batch 8192, Student-t(3) values
     with 0.1 % of the columns scaled by 20 (outlier channels).  Quantized activations bit-exact on a
     row sample, per-block int32 dots bit-exact and bounded by 32 * 127 * 127, outputs within
     tolerance on a seeded sample."""
-    rows, cols, batch = 5120, 5120, 8192
+    batch = 8192
     w = synth.q8_0_weight(rows, cols, seed=77)
     x = synth.student_t3(batch, cols, seed=78)
     assert np.abs(x).max() > 50.0, "the generator must produce outliers"
