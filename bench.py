@@ -249,7 +249,7 @@ def bench_config0(q8mi, hip, synth, copies=48, reps=480):
 def bench_read_probe(q8mi, hip, nbytes=1 << 30, reps=20):
     """Measured ceiling of a plain streaming read (every lane 16 bytes per load, grid-stride)."""
     buf, sink = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(64)
-    fn = lambda i: q8mi.ok(q8mi.lib().q8mi_probe_read(buf.ptr, nbytes, 8, sink.ptr, None), "probe_read")
+    fn = lambda i: q8mi.ok(q8mi.lib().q8mi_probe_read(buf.ptr, nbytes, 2, sink.ptr, None), "probe_read")
     t = time_loop(hip, fn, reps, 3)
     buf.free()
     sink.free()

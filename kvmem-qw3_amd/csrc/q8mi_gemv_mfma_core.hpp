@@ -48,14 +48,18 @@ constexpr uint32_t kMfmaItemBlocks = 32;   // blocks of a row per item: 4 chunks
 constexpr uint32_t kMfmaUnitRows = 4;
 
 // LDS image of the activations:
-//   quants   [batch rows][nb][32 B], rows row_pitch = 32 nb + 128 bytes apart.  A fragment read
-//            (lane = activation row m, chunk c, k-quarter q) touches m * row_pitch + 32 c + 8 q
-//            (+ the step's offset): 128 contiguous bytes per activation row, and the odd
-//            multiple of 128 in the pitch puts rows m and m + 1 on the two halves of the banks
+//   quants   [batch rows][nb][32 B], row m at mfma_xq_row_base(m).  A fragment read (lane =
+//            activation row m, chunk c, k-quarter q) touches row_base(m) + 32 c + 8 q (+ the
+//            step's offset).  The 32 lanes of a half-wave (four rows, four chunks, two quarters)
+//            read 8 bytes each: per row the slots {0, 8} + 32 c of a 128-byte window, so row
+//            bases that are 0, 16, 128 and 144 modulo 256 give 32 different slots of a 256-byte
+//            span (no two lanes on one bank, whether the LDS has 32 or 64 of them)
 //   scales   [nb][MP] fp32 (MP = 4 MG activation rows, padded): the four chunks of a step read
 //            four neighbouring MP-float groups
-__host__ __device__ inline uint32_t mfma_xq_row_pitch(uint32_t nb) { return nb * 32 + 128; }
-__host__ __device__ inline uint32_t mfma_xq_bytes(uint32_t nb, uint32_t batch) { return batch * mfma_xq_row_pitch(nb); }
+__host__ __device__ inline uint32_t mfma_xq_row_base(uint32_t m, uint32_t nb) {   // nb % 8 == 0
+    return m * (nb * 32 + 256) + 16 * (m & 1u) + 128 * ((m >> 1) & 1u);
+}
+__host__ __device__ inline uint32_t mfma_xq_bytes(uint32_t nb, uint32_t batch) { return batch * (nb * 32 + 256); }
 // half_scales: the scale table as fp16 instead of fp32 (half the size, one conversion per use); for
 // activations that would not fit otherwise.
 inline uint32_t mfma_x_lds_bytes(uint32_t nb, uint32_t batch, uint32_t mg, bool half_scales = false) {
@@ -65,8 +69,9 @@ inline uint32_t mfma_x_lds_bytes(uint32_t nb, uint32_t batch, uint32_t mg, bool 
 inline uint32_t mfma_park_floats_per_unit(uint32_t mg) { return 4 * kMfmaUnitRows * 4 * mg; }
 
 struct MfmaItem {
-    v2i q[8];   // per step: bytes 8 (L % 16) .. +8 of the step's 128 bytes of row L / 16 (memory order)
-    int d;      // fp16 scales 2 (L % 16), 2 (L % 16) + 1 of the item's 32, row L / 16
+    v2i q[8];   // per step: bytes 8 t .. 8 t + 7 of the step's 128 bytes of row L / 16 (memory order),
+                // t = (L % 16) ^ 2 for rows 2 and 3, L % 16 for rows 0 and 1
+    int d;      // fp16 scales 2 t, 2 t + 1 of the item's 32, row L / 16
 };
 
 // Copies `batch` rows of Q8_1 activations into the LDS image above, in two halves: issue() puts
@@ -91,7 +96,6 @@ struct MfmaStage {
     }
 
     __device__ __forceinline__ void finish(uint8_t *smem, const uint8_t *y, uint32_t nb, uint32_t batch) {
-        const uint32_t row_pitch = mfma_xq_row_pitch(nb);
         uint8_t *xq = smem;
         uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
         // row by row (a row is nb * 36 bytes, a multiple of 16: nb % 8 == 0), so that locating a dword
@@ -103,7 +107,7 @@ struct MfmaStage {
                 if (HS) *reinterpret_cast<uint16_t *>(xd + (kb * MP + m) * 2) = static_cast<uint16_t>(word & 0xffffu);
                 else *reinterpret_cast<float *>(xd + (kb * MP + m) * 4) = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
             } else {
-                *reinterpret_cast<uint32_t *>(xq + m * row_pitch + kb * 32 + (part - 1) * 4) = word;
+                *reinterpret_cast<uint32_t *>(xq + mfma_xq_row_base(m, nb) + kb * 32 + (part - 1) * 4) = word;
             }
         };
         const v4i *src = reinterpret_cast<const v4i *>(y);
@@ -159,7 +163,6 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *y,
                                                 uint32_t batch, uint32_t batch_total) {
     constexpr uint32_t MP = 4 * MG;
     constexpr int kBatch = 4;
-    const uint32_t row_pitch = mfma_xq_row_pitch(nb);
     uint8_t *xq = smem;
     uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
     const uint32_t nsb = nb / 4;
@@ -176,7 +179,7 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *y,
                 *reinterpret_cast<int *>(xd + (kb * MP + j) * 4) = d[t];
             }
         } else {
-            *reinterpret_cast<v4i *>(xq + j * row_pitch + sb * 128 + (part - 1) * 16) = v;
+            *reinterpret_cast<v4i *>(xq + mfma_xq_row_base(j, nb) + sb * 128 + (part - 1) * 16) = v;
         }
     };
     for (uint32_t base = 0; base < total; base += THREADS * kBatch) {
@@ -237,7 +240,10 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
     MfmaItem items[2];
     uint32_t ik = i0 / nitems, istep = i0 % nitems, ileft = n_items;
     const uint8_t *irow = row_ptr(useq.unit(ik));
-    const uint32_t l16 = lane & 15u;
+    // Lane L loads slot (L % 16) ^ swz of row L / 16, swz = 2 for rows 2 and 3: the operand shuffle
+    // below then reads, per half-wave, source lanes that differ modulo 32 (rows m and m + 2 would
+    // otherwise meet on the same banks of the shuffle network).
+    const uint32_t l16 = (lane & 15u) ^ ((lane >> 4) & 2u);
     auto issue = [&](MfmaItem &it) {
         const uint32_t left = nb - istep * kMfmaItemBlocks;          // blocks of the row from this item on
         const uint32_t vsteps = left >= kMfmaItemBlocks ? 8u : left / 4;   // steps with real blocks (nb % 8 == 0)
@@ -263,7 +269,6 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
     if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch, d4_batch_total);
     else xstage.finish(smem, y, nb, batch);
 
-    const uint32_t row_pitch = mfma_xq_row_pitch(nb);
     const uint8_t *xq = smem;
     const uint8_t *xd = smem + mfma_xq_bytes(nb, batch);
     // activation fragment rows of this lane, one per MFMA group (clamped: rows past the batch are never stored)
@@ -271,11 +276,11 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
 #pragma unroll
     for (int g = 0; g < MG; ++g) {
         const uint32_t m = 4 * g + m4;
-        a_row[g] = (m < batch ? m : batch - 1) * row_pitch + 32 * c + 8 * q;
+        a_row[g] = mfma_xq_row_base(m < batch ? m : batch - 1, nb) + 32 * c + 8 * q;
     }
     // source lanes of the operand shuffle (byte addresses for ds_bpermute)
-    const int src_q = static_cast<int>((16 * m4 + 4 * c + q) * 4);
-    const int src_d = static_cast<int>((16 * m4 + (c >> 1)) * 4);
+    const uint32_t swz = m4 & 2u;
+    const int src_q = static_cast<int>((16 * m4 + ((4 * c + q) ^ swz)) * 4);
     v4i seed;
     seed.x = seed.y = seed.z = seed.w = 0x4B400000;   // 1.5 * 2^23: the int32 result read as fp32 is 12582912 + S
     asm volatile("" : "+v"(seed));
@@ -333,7 +338,8 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
                     }
                 }
                 // halfword 4 s + c of the row's scales: dword 2 s + c / 2 (held by lane 16 r + 2 s + c / 2), half c % 2
-                const uint32_t dword = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(src_d + 8 * s, it.d));
+                const uint32_t dword = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(
+                    static_cast<int>((16 * m4 + ((2 * s + (c >> 1)) ^ swz)) * 4), it.d));
                 const uint16_t hbits = static_cast<uint16_t>((c & 1u) ? (dword >> 16) : (dword & 0xffffu));
                 const float dw = static_cast<uint32_t>(s) < vsteps ? half_bits_to_float(hbits) : 0.0f;
                 const float cw = -kMagic * dw;
