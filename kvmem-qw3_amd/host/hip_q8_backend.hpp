@@ -131,6 +131,49 @@ public:
     DeviceStatus q8_0_get_rows_batch(DeviceTensor &out, const DeviceWeight &weight, const uint64_t *rows,
                                      uint32_t batch);
 
+    // Format-neutral forwards with the reference's default bodies
+    // (include/qw3/device_backend.hpp:541-607): the executor calls these; for Q8_0
+    // weights they are the q8_0_* operators.  linear_matmul_add is left to the base
+    // class there (it needs the backend's elementwise add, which is outside this path).
+    DeviceStatus linear_get_row(DeviceTensor &out, const DeviceWeight &weight, uint64_t row) {
+        return q8_0_get_row(out, weight, row);
+    }
+    DeviceStatus linear_get_row_from_argmax(DeviceTensor &out, const DeviceWeight &weight,
+                                            const DeviceArgmaxBuffer &argmaxes, uint32_t index) {
+        return q8_0_get_row_from_argmax(out, weight, argmaxes, index);
+    }
+    DeviceStatus linear_get_rows_batch(DeviceTensor &out, const DeviceWeight &weight, const uint64_t *rows,
+                                       uint32_t batch) {
+        return q8_0_get_rows_batch(out, weight, rows, batch);
+    }
+    DeviceStatus linear_matvec(DeviceTensor &out, const DeviceWeight &weight, const DeviceTensor &x) {
+        return q8_0_matvec(out, weight, x);
+    }
+    DeviceStatus linear_matvec_add(DeviceTensor &accum, const DeviceWeight &weight, const DeviceTensor &x) {
+        return q8_0_matvec_add(accum, weight, x);
+    }
+    DeviceStatus linear_matvec_silu_mul(DeviceTensor &out, const DeviceWeight &weight_gate,
+                                        const DeviceWeight &weight_up, const DeviceTensor &x) {
+        return q8_0_matvec_silu_mul(out, weight_gate, weight_up, x);
+    }
+    DeviceStatus linear_matvec_fanout(DeviceTensor *const *outs, const DeviceWeight *const *weights, uint32_t n,
+                                      const DeviceTensor &x) {
+        for (uint32_t i = 0; i < n; ++i)
+            if (auto st = linear_matvec(*outs[i], *weights[i], x); !st.ok) return st;
+        return {};
+    }
+    DeviceStatus linear_matmul(DeviceTensor &out, const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
+                               uint32_t in_stride, uint32_t out_stride) {
+        return q8_0_matmul(out, weight, x, batch, in_stride, out_stride);
+    }
+    DeviceStatus linear_matmul_fanout(DeviceTensor *const *outs, const DeviceWeight *const *weights,
+                                      const uint32_t *out_strides, uint32_t n, const DeviceTensor &x,
+                                      uint32_t batch, uint32_t in_stride) {
+        for (uint32_t i = 0; i < n; ++i)
+            if (auto st = linear_matmul(*outs[i], *weights[i], x, batch, in_stride, out_strides[i]); !st.ok) return st;
+        return {};
+    }
+
     // New op (no counterpart in the reference): the whole verify tail in one pass
     // over the LM-head weights.  Equivalent to q8_0_matmul(logits, w_out, norm, batch,
     // in_stride, vocab) + argmax_batch + the greedy accept loop

@@ -6,10 +6,14 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
 #include <string>
 #include <vector>
 
+#include <unistd.h>
+
 #include "../../kvmem-qw3_amd/host/hip_q8_backend.hpp"
+#include "../../kvmem-qw3_amd/host/gguf_q8.hpp"
 #include "../../oracle/q8_oracle.h"
 
 namespace {
@@ -261,6 +265,22 @@ void case_matvec_family(qw3::HipQ8Backend &b) {
         ok = close_fp32(download_f32(b, *outs[i]), ref, mag, 1, hw[i]->rows, hw[i]->rows, d);
     }
     report("matvec_fanout3", ok, d);
+
+    // format-neutral forwards: the same operators under the names the executor calls
+    auto la = b.tensor_f32(wa.rows, "la"), lb = b.tensor_f32(wb.rows, "lb"), lc = b.tensor_f32(wc.rows, "lc");
+    qw3::DeviceTensor *louts[3] = {la.get(), lb.get(), lc.get()};
+    ok = require(b.linear_matvec_fanout(louts, ws, 3, *dx), "linear_matvec_fanout");
+    for (int i = 0; i < 3 && ok; ++i) {
+        oracle_linear(*hw[i], x.data(), 1, cols, hw[i]->rows, ref, mag);
+        ok = close_fp32(download_f32(b, *louts[i]), ref, mag, 1, hw[i]->rows, hw[i]->rows, d);
+    }
+    auto lo = b.tensor_f32(rows, "lo");
+    ok = ok && require(b.linear_matvec(*lo, *dw, *dx), "linear_matvec") && require(b.q8_0_matvec(*out, *dw, *dx), "matvec");
+    ok = ok && download_f32(b, *lo) == download_f32(b, *out);
+    ok = ok && require(b.linear_matmul(*lo, *dw, *dx, 1, cols, rows), "linear_matmul");
+    oracle_linear(w, x.data(), 1, cols, rows, ref, mag);
+    ok = ok && close_fp32(download_f32(b, *lo), ref, mag, 1, rows, rows, d);
+    report("linear_forwards", ok, d);
 }
 
 void case_matmul(qw3::HipQ8Backend &b) {
@@ -467,6 +487,57 @@ void case_get_rows(qw3::HipQ8Backend &b) {
     report("get_rows_batch", ok);
 }
 
+// A Q8_0 tensor travels file -> GgufFile -> split-plane device weight -> GEMV and must give what
+// the same blocks give when handed to weight_q8_0 directly.
+void case_gguf(qw3::HipQ8Backend &b) {
+    std::string d;
+    const uint32_t rows = 640, cols = 1024;
+    const HostWeight w = make_weight(rows, cols, 301);
+    const std::string path = "/tmp/q8mi_backend_parity_" + std::to_string(static_cast<long>(getpid())) + ".gguf";
+    {
+        std::vector<uint8_t> f;
+        auto put = [&](const void *p, size_t n) { f.insert(f.end(), static_cast<const uint8_t *>(p), static_cast<const uint8_t *>(p) + n); };
+        auto u32 = [&](uint32_t v) { put(&v, 4); };
+        auto u64 = [&](uint64_t v) { put(&v, 8); };
+        auto str = [&](const char *t) { u64(std::strlen(t)); put(t, std::strlen(t)); };
+        put("GGUF", 4); u32(3); u64(2); u64(1);
+        str("general.architecture"); u32(8); str("qwen3");
+        str("pad.bias"); u32(1); u64(5); u32(0); u64(0);                 // 20 bytes of F32 first, so the weight is not at offset 0
+        str("blk.0.attn_output.weight"); u32(2); u64(cols); u64(rows); u32(8); u64(32);
+        while (f.size() % 32) f.push_back(0);
+        const float bias[5] = {1, 2, 3, 4, 5};
+        put(bias, 20);
+        while (f.size() % 32) f.push_back(0);
+        put(w.gguf.data(), w.gguf.size());
+        FILE *fp = std::fopen(path.c_str(), "wb");
+        if (fp) { std::fwrite(f.data(), 1, f.size(), fp); std::fclose(fp); }
+    }
+    bool ok = true;
+    try {
+        const qw3::GgufFile file(path);
+        const qw3::GgufTensorInfo *t = file.find_tensor("blk.0.attn_output.weight");
+        ok = t != nullptr && t->type == 8 && qw3::gguf_tensor_rows(*t) == rows && qw3::gguf_tensor_cols(*t) == cols &&
+             t->bytes == w.gguf.size() && std::memcmp(file.data() + t->abs_offset, w.gguf.data(), t->bytes) == 0;
+        ok = ok && qw3::gguf_upload_q8_0(b, file, "pad.bias") == nullptr && qw3::gguf_upload_q8_0(b, file, "absent") == nullptr;
+        auto from_file = qw3::gguf_upload_q8_0(b, file, "blk.0.attn_output.weight");
+        auto direct = b.weight_q8_0(w.gguf.data(), rows, cols, "direct");
+        ok = ok && from_file != nullptr && direct != nullptr && from_file->rows == rows && from_file->cols == cols;
+        const auto x = normal_vec(cols, 302);
+        auto dx = upload_f32(b, x);
+        auto o1 = b.tensor_f32(rows, "o1"), o2 = b.tensor_f32(rows, "o2");
+        ok = ok && require(b.q8_0_matvec(*o1, *from_file, *dx), "matvec gguf") && require(b.q8_0_matvec(*o2, *direct, *dx), "matvec direct");
+        std::vector<float> ref, mag;
+        oracle_linear(w, x.data(), 1, cols, rows, ref, mag);
+        const auto g1 = download_f32(b, *o1);
+        ok = ok && g1 == download_f32(b, *o2) && close_fp32(g1, ref, mag, 1, rows, rows, d);
+    } catch (const std::exception &e) {
+        ok = false;
+        d = e.what();
+    }
+    std::remove(path.c_str());
+    report("gguf_tensor_to_matvec", ok, d);
+}
+
 void case_lm_head_verify(qw3::HipQ8Backend &b) {
     const uint32_t vocab = 30000, cols = 1024, eos = 5;
     const HostWeight w = make_weight(vocab, cols, 81);
@@ -558,7 +629,7 @@ int main(int argc, char **argv) {
     struct Case { const char *name; void (*fn)(qw3::HipQ8Backend &); };
     const Case cases[] = {
         {"closed_form", case_closed_form}, {"matvec", case_matvec_family}, {"matmul", case_matmul},
-        {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"lm_head", case_lm_head_verify}, {"graph", case_graph_replay},
+        {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"gguf", case_gguf}, {"lm_head", case_lm_head_verify}, {"graph", case_graph_replay},
     };
     for (const auto &c : cases) {
         if (!only.empty() && only != c.name) continue;
