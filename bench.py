@@ -342,7 +342,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's throughput; run with --gpus 1 "
-                 "(the path shards by weight rows, see DESIGN.md)")
+                 "(the path would shard by weight rows: each GPU keeps rows/N of every weight)")
 
     import q8mi
     from q8mi import hip, synth

@@ -40,9 +40,10 @@ struct GatherParams {
 
 template <RowSource SRC, bool BF16>
 __global__ __launch_bounds__(kThreads) void get_rows_kernel(const GatherParams p) {
-    const uint64_t i = (static_cast<uint64_t>(blockIdx.x) * kThreads + threadIdx.x) * kPerThread;
+    // grid.x carries the batch (a long prompt gathers more rows than grid.y may count)
+    const uint64_t i = (static_cast<uint64_t>(blockIdx.y) * kThreads + threadIdx.x) * kPerThread;
     if (i >= p.cols) return;
-    const uint32_t b = blockIdx.y;
+    const uint32_t b = blockIdx.x;
 
     uint64_t row;
     bool valid;
@@ -91,9 +92,9 @@ __global__ __launch_bounds__(kThreads) void get_rows_kernel(const GatherParams p
 
 template <RowSource SRC>
 int launch(const GatherParams &p, uint32_t batch, bool bf16, void *stream, const char *what) {
-    const uint64_t gx = (p.cols / kPerThread + kThreads - 1) / kThreads;
-    if (gx > 0x7fffffffull || batch > 65535u) return fail(Q8MI_REJECTED, "%s: grid too large", what);
-    const dim3 grid(static_cast<uint32_t>(gx), batch);
+    const uint64_t gy = (p.cols / kPerThread + kThreads - 1) / kThreads;
+    if (gy > 65535u || batch > 0x7fffffffu) return fail(Q8MI_REJECTED, "%s: grid too large", what);
+    const dim3 grid(batch, static_cast<uint32_t>(gy));
     if (bf16)
         get_rows_kernel<SRC, true><<<grid, kThreads, 0, as_stream(stream)>>>(p);
     else

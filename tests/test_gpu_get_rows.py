@@ -95,6 +95,22 @@ def test_argmax_then_embedding_chain(gpu, oracle):
     assert np.array_equal(out.download(np.uint32), oracle.get_row(w, tok, cols).view(np.uint32))
 
 
+def test_get_rows_long_prompt(gpu, oracle):
+    """A prompt's worth of rows in one call: 100 000 ids (more than a grid's y extent)."""
+    rows, cols = 512, 256
+    w = make(oracle, rows, cols, seed=14)
+    dw = dev(w)
+    n = 100000
+    ids = np.random.default_rng(15).integers(0, rows, n).astype(np.uint64)
+    dids = dev(ids)
+    out = hip.DeviceBuffer(n * cols * 4)
+    ok(q8mi.lib().q8mi_get_rows(dw.ptr, dids.ptr, n, rows, cols, out.ptr, 0, NULL), "get_rows")
+    hip.synchronize()
+    got = out.download(np.uint32).reshape(n, cols)
+    table = np.stack([oracle.get_row(w, r, cols) for r in range(rows)]).view(np.uint32)
+    assert np.array_equal(got, table[ids.astype(np.int64)])
+
+
 def test_get_rows_rejections(gpu):
     L = q8mi.lib()
     buf = hip.DeviceBuffer(4096)
