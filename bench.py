@@ -7,7 +7,7 @@ One "step" = one pass over the decode GEMV set of one 27B-style layer at M=1
     qgemv_fanout4(x[5120])   Q 5120x6144, K 5120x1024, V 5120x1024   (quantizer fused into the GEMV)
     qgemv_add(a[6144])       O 6144x5120, residual add               (fused)
     qgemv_silu_mul(x[5120])  gate, up 5120x17408 each                (fused)
-    quantize_q8_1(f[17408])  -> gemv_add   down 17408x5120           (two launches: rows above 8192 columns)
+    qgemv_add(f[17408])      down 17408x5120, residual add           (fused, one 1024-thread workgroup per CU)
 
 which is the routing of the host layer (HipQ8Backend) at batch 1; for batch 2..8 every op is
 quantize_q8_1 + GEMV (two launches), as in the reference.
@@ -88,7 +88,7 @@ class DecodeStep:
 
     @property
     def launches(self):
-        return 5 if self.fused else 8
+        return 4 if self.fused else 8
 
     def run(self, layer, stream=None):
         L, m, w = self.L, self.m, layer.w
@@ -100,8 +100,7 @@ class DecodeStep:
             ok(L.q8mi_qgemv_add(w["o"].ptr, self.attn.ptr, ATTN_OUT, self.h.ptr, 0, HIDDEN, ATTN_OUT, m, HIDDEN,
                                 stream), "qo")
             self.run_silu(layer, stream)
-            ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, m, FFN, FFN, stream), "quantize")
-            ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, m, HIDDEN, stream), "down")
+            ok(L.q8mi_qgemv_add(w["down"].ptr, self.ffn.ptr, FFN, self.h.ptr, 0, HIDDEN, FFN, m, HIDDEN, stream), "qdown")
             return
         ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize")
         ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.y5120.ptr,

@@ -95,10 +95,13 @@ int q8mi_gemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uint
                       void *stream);
 
 /* ---- GEMV with the Q8_1 quantizer fused in (batch 1..2) --------------------
- * Same results, bit for bit, as q8mi_quantize_q8_1 followed by the matching
- * q8mi_gemv* call, in one launch: every workgroup quantizes the fp32
- * activations (x: [batch][stride_x_row] floats) while it stages them in LDS,
- * so no Q8_1 scratch buffer and no quantizer launch are needed.  This is what
+ * The results of q8mi_quantize_q8_1 followed by the matching q8mi_gemv* call,
+ * in one launch: every workgroup quantizes the fp32 activations
+ * (x: [batch][stride_x_row] floats) while it stages them in LDS, so no Q8_1
+ * scratch buffer and no quantizer launch are needed.  The quantized values
+ * and the per-block products are the same bits; for rows of up to 8192
+ * columns so are the outputs, longer rows run with another workgroup size and
+ * add the same products in another order (inside the GEMV's tolerance).  This is what
  * the reference's operators do in two steps (src/kernels_cuda.cu:10764-10888,
  * 11244-11302, 12035-12069, 12227-12258: launch_quantize_q8_1 then the
  * launcher); the fusion itself has no counterpart in the reference.

@@ -389,7 +389,10 @@ int launch_ms(const GemvParams &p, hipStream_t stream) {
     const int forced = gemv_tuning().threads;
     if (p.xf != nullptr) {   // fused quantizer: the activations must fit LDS
         if (M > 2) return fail(Q8MI_REJECTED, "qgemv: batch %d above 2 (quantize once and use the GEMV instead)", M);
-        if (xb + park_256 <= 76u * 1024u && forced != 1024) return launch_inst<M, 256, kXF32, SILU>(p, xb, stream);
+        // rows above 8192 columns: one 1024-thread workgroup per CU quantizes them once per CU instead of twice
+        const bool long_rows = p.nb * kQK > 8192u && xb + park_1024 <= kLdsLimit;
+        if (xb + park_256 <= 76u * 1024u && forced != 1024 && !long_rows)
+            return launch_inst<M, 256, kXF32, SILU>(p, xb, stream);
         if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXF32, SILU>(p, xb, stream);
         return fail(Q8MI_REJECTED, "qgemv: %u activation rows of %u columns do not fit LDS", M, p.nb * 32);
     }

@@ -215,9 +215,10 @@ DeviceStatus HipQ8Backend::quantize_q8_1(const float *x, uint32_t batch, uint32_
     return {};
 }
 
-// Batch-1 ops on rows of at most 8192 columns quantize inside the GEMV (one launch instead of
-// two, same bits); longer rows and batches above 1 are faster with the stand-alone quantizer.
-static bool fuse_quantizer(uint32_t batch, uint32_t cols) { return batch == 1 && cols % 256 == 0 && cols <= 8192; }
+// Batch-1 ops quantize inside the GEMV (one launch instead of two, same bits) whenever the library
+// accepts the shape (it rejects rows that do not fit LDS, and the two-step form below runs);
+// batches above 1 are faster with the stand-alone quantizer.
+static bool fuse_quantizer(uint32_t batch, uint32_t cols) { return batch == 1 && cols % 256 == 0; }
 
 // dispatch_q8_matvec, src/kernels_cuda.cu:14617-14658: any batch as GEMV slices of <= 8 rows
 DeviceStatus HipQ8Backend::gemv_route(float *out, const DeviceWeight &weight, const float *x, uint32_t batch,
