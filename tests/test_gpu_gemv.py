@@ -54,6 +54,38 @@ def test_gemv_matches_oracle(gpu, oracle, rows, cols, batch):
         block_dot_check(oracle, dw, w, dy, y, rows, cols, batch, seed=rows + batch, n=1024)
 
 
+@pytest.mark.parametrize("offset", [4, 8, 12])
+@pytest.mark.parametrize("batch", [1, 2, 4, 8])
+def test_gemv_activations_on_a_4_byte_boundary(gpu, oracle, offset, batch):
+    """Q8_1 blocks are only 4-byte aligned by type (36 bytes each): an activation buffer that does
+    not start on a 16-byte boundary must give the same results (the lanes then read it from
+    global memory instead of a 16-byte-wide LDS staging copy)."""
+    rows, cols = 777, 2048
+    w = synth.q8_0_weight(rows, cols, seed=5)
+    x = synth.normal(batch, cols, seed=6 + batch)
+    dw = dev(w)
+    _, y = quantize_q8_1(x)
+    shifted = hip.DeviceBuffer(len(y) + 16)
+    shifted.upload(y, offset)
+    L = q8mi.lib()
+    out = hip.DeviceBuffer(4 * batch * rows).fill(0xff)
+    ok(L.q8mi_gemv(dw.ptr, shifted.ptr + offset, out.ptr, rows, cols, batch, rows, NULL), "gemv")
+    hip.synchronize()
+    rc, ref = oracle.gemv(w, y, rows, cols, batch)
+    rc, absum = oracle.gemv_abs(w, y, rows, cols, batch)
+    assert_close_fp32(out.download(np.float32).reshape(batch, rows), ref, absum, f"gemv y+{offset} M={batch}")
+    # the fused LM head takes the same buffer
+    scratch = hip.DeviceBuffer(L.q8mi_lm_head_scratch_bytes(rows, cols, batch))
+    pairs, acc = hip.DeviceBuffer(8 * batch), hip.DeviceBuffer(8)
+    drafts = np.zeros(8, np.int32)
+    ok(L.q8mi_lm_head_argmax_accept(dw.ptr, shifted.ptr + offset, rows, cols, batch, drafts.ctypes.data_as(C.c_void_p),
+                                    0, 0, pairs.ptr, acc.ptr, None, rows, scratch.ptr, NULL), "lm_head")
+    hip.synchronize()
+    tok = pairs.download(np.dtype([("value", np.float32), ("index", np.int32)]))["index"]
+    want = oracle.argmax_rows_scan(ref, batch, rows)["index"]
+    assert np.array_equal(tok, want)
+
+
 @pytest.mark.parametrize("cols", [32, 96, 160, 992])
 @pytest.mark.parametrize("batch", [1, 3, 8])
 def test_gemv_unaligned_planes(gpu, oracle, cols, batch):
