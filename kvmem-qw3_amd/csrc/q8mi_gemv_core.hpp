@@ -69,6 +69,20 @@ __device__ __forceinline__ v4i load_x16_global(const uint8_t *y, uint32_t blk, u
     return v;
 }
 
+// idx = m * per + within with m < M: the quotient by a run of compare-and-subtract steps (M is a
+// small compile-time bound; a 32-bit division by a run-time value costs some twenty instructions).
+template <int M>
+__device__ __forceinline__ void split_index(uint32_t idx, uint32_t per, uint32_t &m, uint32_t &within) {
+    m = 0;
+    within = idx;
+#pragma unroll
+    for (int i = 1; i < M; ++i) {
+        const bool over = within >= per;
+        within = over ? within - per : within;
+        m += over ? 1u : 0u;
+    }
+}
+
 // Copies M rows of Q8_1 activations from global memory into LDS, split into a
 // packed int8 area and an fp32 scale area.  Dword 0 of each 36-B block is
 // {d, s}; dwords 1..8 are the quants.  The M rows are contiguous in memory
@@ -103,7 +117,8 @@ struct StageLds {
 
         auto put = [&](uint32_t g, uint32_t word) {   // g: dword index in the global layout
             const uint32_t blk_g = g / 9, part = g % 9;
-            const uint32_t m = blk_g / nb, kb = blk_g % nb;
+            uint32_t m, kb;
+            split_index<M>(blk_g, nb, m, kb);
             const uint32_t blk = m * blocks_padded + kb;
             if (part == 0) {
                 wd[blk] = half_bits_to_float(static_cast<uint16_t>(word & 0xffffu));
@@ -156,7 +171,9 @@ struct StageF32 {
     __device__ __forceinline__ static Float4 fetch(const float *x, uint32_t stride_x, uint32_t per_row,
                                                    uint32_t total, uint32_t c, bool vec) {
         const uint32_t cc = c < total ? c : 0;
-        const float *src = x + static_cast<uint64_t>(cc / per_row) * stride_x + (cc % per_row) * 4;
+        uint32_t m, within;
+        split_index<M>(cc, per_row, m, within);
+        const float *src = x + static_cast<uint64_t>(m) * stride_x + within * 4;
         return vec ? load4<true>(src) : load4<false>(src);
     }
 
@@ -181,7 +198,8 @@ struct StageF32 {
             float d;
             const uint32_t packed = quantize4_q8_1(f, d);   // all lanes take part in the exchanges
             if (c < total) {
-                const uint32_t m = c / per_row, within = c % per_row;
+                uint32_t m, within;
+                split_index<M>(c, per_row, m, within);
                 const uint32_t blk = m * blocks_padded + within / 8;
                 wq[blk * 8 + within % 8] = packed;
                 if (within % 8 == 0) wd[blk] = half_bits_to_float(float_to_half_bits(d));
