@@ -55,9 +55,11 @@ template <bool VEC>
 __global__ __launch_bounds__(kQuantThreads) void quantize_q8_1_d4_kernel(
         const float *__restrict__ x, uint8_t *__restrict__ y, uint32_t cols,
         uint32_t stride_x_row, uint32_t batch) {
-    const uint32_t i0 = (blockIdx.x * kQuantThreads + threadIdx.x) * kElemsPerLane;
+    // grid.x carries the batch, as in the reference's launch (src/mmvq_q8.cu:749): a prefill chunk
+    // may hold more rows than grid.y can count
+    const uint32_t i0 = (blockIdx.y * kQuantThreads + threadIdx.x) * kElemsPerLane;
     if (i0 >= cols) return;
-    const uint32_t j = blockIdx.y;
+    const uint32_t j = blockIdx.x;
     const Float4 v = load4<VEC>(x + static_cast<uint64_t>(j) * stride_x_row + i0);
 
     const float amax = group8_amax(v);
@@ -117,8 +119,9 @@ extern "C" int q8mi_quantize_q8_1_d4(const float *x, void *y, uint32_t batch, ui
                                      uint32_t stride_x_row, void *stream) {
     if (cols % 128 != 0) return fail(Q8MI_REJECTED, "quantize_q8_1_d4: cols %u not a multiple of 128", cols);
     if (batch == 0 || cols == 0) return Q8MI_OK;
-    if (batch > 65535u) return fail(Q8MI_REJECTED, "quantize_q8_1_d4: batch %u above 65535", batch);
-    const dim3 grid((cols + kQuantThreads * kElemsPerLane - 1) / (kQuantThreads * kElemsPerLane), batch);
+    const uint32_t col_groups = (cols + kQuantThreads * kElemsPerLane - 1) / (kQuantThreads * kElemsPerLane);
+    if (col_groups > 65535u || batch > 0x7fffffffu) return fail(Q8MI_REJECTED, "quantize_q8_1_d4: shape too large for one launch");
+    const dim3 grid(batch, col_groups);
     if (vec_ok(x, stride_x_row)) {
         quantize_q8_1_d4_kernel<true><<<grid, kQuantThreads, 0, as_stream(stream)>>>(
             x, static_cast<uint8_t *>(y), cols, stride_x_row, batch);

@@ -132,6 +132,25 @@ def test_gemm_heavy_tail_batch_8192(gpu, oracle, rows, cols):
     d4_block_dots(oracle, dw, w, dy, y, rows, cols, batch, seed=80, n=1024)
 
 
+def test_gemm_prompt_longer_than_a_grid_extent(gpu, oracle):
+    """70 000 activation rows in one call (more than a grid's y extent): D4 quantizer bit-exact
+    on the whole buffer, GEMM outputs within tolerance on a seeded sample."""
+    rows, cols, batch = 256, 256, 70000
+    w = synth.q8_0_weight(rows, cols, seed=91)
+    x = synth.normal(batch, cols, seed=92)
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    rc, yref = oracle.quantize_q8_1_d4(x)
+    assert np.array_equal(y, yref)
+    got = run_gemm(dw, dy, rows, cols, batch)
+    rng = np.random.default_rng(93)
+    n = 20000
+    sr = rng.integers(0, rows, n, dtype=np.uint32)
+    sj = np.concatenate([rng.integers(0, batch, n - 4, dtype=np.uint32), np.array([0, 65535, 65536, batch - 1], np.uint32)])
+    rc, ref_s, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, sr, sj)
+    assert_close_fp32(got[sj, sr], ref_s, absum, "gemm, 70000 rows (sampled)")
+
+
 def test_gemm_reference_tolerance_restated(gpu):
     """tests/mmq_parity.cu:246-254 restated: output vs fp32 dot of the dequantised
     operands within 5e-3 abs or 1e-3 rel, U(-0.5,0.5) weights and U(-1,1) activations."""
