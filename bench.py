@@ -255,6 +255,21 @@ def bench_read_probe(q8mi, hip, nbytes=1 << 30, reps=20):
     return round(nbytes / (t * 1e-3) / 1e9, 1)
 
 
+def bench_mfma_ceilings(q8mi, hip, iters=20000):
+    """Measured issue-rate ceilings of the matrix unit: int8 MFMAs alone, and with the scalar fp32
+    FMAs that rescaling their results costs (2 per int32 sum; packed fp32 math is not available)."""
+    L = q8mi.lib()
+    sink = hip.DeviceBuffer(L.q8mi_probe_mfma_sink_bytes())
+    ops = C.c_uint64(0)
+    out = {}
+    for name, flag in (("mfma_only_tops", 0), ("mfma_with_rescale_tops", 1)):
+        fn = lambda i: q8mi.ok(L.q8mi_probe_mfma(flag, iters, sink.ptr, C.byref(ops), None), "probe_mfma")
+        t = time_loop(hip, fn, 3, 1)
+        out[name] = round(ops.value / (t * 1e-3) / 1e12, 1)
+    sink.free()
+    return out
+
+
 def bench_gemm(q8mi, hip, synth, reps=10):
     """Prefill GEMM (D4 quantize + MFMA GEMM): M=2048 on the two FFN shapes, M=8192 on gate/up."""
     L, ok = q8mi.lib(), q8mi.ok
@@ -411,6 +426,10 @@ def main():
         result["config0_gemv_m1"] = bench_config0(q8mi, hip, synth)
         result["hbm_read_probe_gbps"] = bench_read_probe(q8mi, hip)
         result["gemm_int8"] = bench_gemm(q8mi, hip, synth)
+        ceil = bench_mfma_ceilings(q8mi, hip)
+        for v in result["gemm_int8"].values():
+            v["frac_of_rescale_ceiling"] = round(v["tops"] / ceil["mfma_with_rescale_tops"], 4)
+        result["gemm_int8"]["measured_ceilings"] = ceil
         result["lm_head_fused"] = bench_lm_head(q8mi, hip, synth)
     if not (args.quick or args.no_cpu):
         result["cpu_baseline"] = cpu_baseline()

@@ -232,6 +232,16 @@ int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per_cu, uint32
  * writes `bytes`): the known-size launch that hardware memory-traffic counters
  * are calibrated against.  No counterpart in the reference. */
 int q8mi_probe_copy(const void *src, void *dst, uint64_t bytes, void *stream);
+/* Matrix-unit ceilings the GEMM is compared with: two workgroups of four waves
+ * per CU, every wave running `iters` rounds of four independent
+ * v_mfma_i32_32x32x32_i8 (what one wave issues per 32-block of a 128 x 128 GEMM
+ * tile) plus, when with_rescale is nonzero, the 128 scalar fp32 FMAs that
+ * rescaling those four results costs with packed fp32 math unavailable.
+ * *ops_out (host) receives the int8 operations launched,
+ * 2 * 32 * 32 * 32 * 4 * iters per wave; the caller times the launch.  No
+ * counterpart in the reference.  sink: 2 * CUs * 256 device int32. */
+int q8mi_probe_mfma(int with_rescale, uint32_t iters, int32_t *sink, uint64_t *ops_out, void *stream);
+size_t q8mi_probe_mfma_sink_bytes(void);
 
 /* ---- synthetic inputs (host side, for benches and tests) ----------------- */
 /* Counter-based generator: element i of stream `seed` depends only on

@@ -141,6 +141,33 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const v4i *__restrict__
     for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
+// ---- measurement helper: matrix-unit ceilings -----------------------------------
+// Four independent int8 MFMAs per round, optionally with NV independent scalar FMAs:
+// nothing else (no loads, no LDS), so the time is the issue rate of the two pipes.
+template <int NV>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(int *__restrict__ out, uint32_t iters, float a, float b) {
+    v4i va = {static_cast<int>(threadIdx.x), 1, 2, 3}, vb = {4, 5, 6, static_cast<int>(threadIdx.x)};
+    v16i c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+    float x[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) x[k] = static_cast<float>(threadIdx.x + k);
+    for (uint32_t i = 0; i < iters; ++i) {
+        c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c3, 0, 0, 0);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) x[k % 8] = fmaf(x[k % 8], a, b);
+    }
+    int s = 0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s += c0[v] + c1[v] + c2[v] + c3[v];
+    float f = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) f += x[k];
+    out[blockIdx.x * 256 + threadIdx.x] = s + static_cast<int>(f);
+}
+
 // ---- synthetic inputs --------------------------------------------------------
 inline uint64_t splitmix64(uint64_t z) {
     z += 0x9E3779B97F4A7C15ull;
@@ -264,6 +291,21 @@ extern "C" int q8mi_probe_copy(const void *src, void *dst, uint64_t bytes, void 
     probe_copy_kernel<<<grid, 256, 0, as_stream(stream)>>>(static_cast<const v4i *>(src), static_cast<v4i *>(dst),
                                                            bytes / 16);
     return check_launch("probe_copy");
+}
+
+extern "C" size_t q8mi_probe_mfma_sink_bytes(void) {
+    return static_cast<size_t>(device_cu_count()) * 2 * 256 * sizeof(int32_t);
+}
+
+extern "C" int q8mi_probe_mfma(int with_rescale, uint32_t iters, int32_t *sink, uint64_t *ops_out, void *stream) {
+    if (sink == nullptr || iters == 0) return fail(Q8MI_REJECTED, "probe_mfma: null sink or zero rounds");
+    const uint32_t grid = static_cast<uint32_t>(device_cu_count()) * 2;
+    if (with_rescale)
+        probe_mfma_kernel<128><<<grid, 256, 0, as_stream(stream)>>>(sink, iters, 1.0001f, 0.5f);
+    else
+        probe_mfma_kernel<0><<<grid, 256, 0, as_stream(stream)>>>(sink, iters, 1.0001f, 0.5f);
+    if (ops_out) *ops_out = static_cast<uint64_t>(grid) * 4 * iters * 4 * 2ull * 32 * 32 * 32;
+    return check_launch("probe_mfma");
 }
 
 extern "C" int q8mi_synth_f32(float *out, uint64_t rows, uint64_t cols, uint64_t seed, int kind,

@@ -61,6 +61,8 @@ SIGNATURES = {
     "q8mi_repack_q8_0_split_host": (_int, [_vp, _u64, _u64, _vp]),
     "q8mi_repack_q8_0_split": (_int, [_vp, _u64, _u64, _vp, _vp]),
     "q8mi_probe_read": (_int, [_vp, _u64, _u32, _vp, _vp]),
+    "q8mi_probe_mfma": (_int, [_int, _u32, _vp, C.POINTER(C.c_uint64), _vp]),
+    "q8mi_probe_mfma_sink_bytes": (C.c_size_t, []),
     "q8mi_qgemv": (_int, [_vp, _vp, _u32, _vp, _int, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_qgemv_add": (_int, [_vp, _vp, _u32, _vp, _int, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_qgemv_silu_mul": (_int, [_vp, _vp, _vp, _u32, _vp, _u32, _u32, _u32, _u32, _vp]),
