@@ -38,6 +38,8 @@
 // different activation fragments.
 #pragma once
 
+#include <type_traits>
+
 #include "q8mi_gemv_core.hpp"
 
 namespace q8mi {
@@ -322,30 +324,53 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
                 a_nxt[g] = *reinterpret_cast<const long *>(xq_chunk + a_row[g]);
                 dx_nxt[g] = load_dx(xd_chunk + 4 * kSc * g);
             }
+            // the operand and scale shuffles run one step ahead as well: LDS operations complete in
+            // order, so a shuffle issued right before its use would expose the whole LDS latency
+            // (and that of the reads issued just before it) in every step
+            auto shuffle_scale = [&](int s) {
+                // halfword 4 s + c of the row's scales: dword 2 s + c / 2 (held by lane 16 r + 2 s + c / 2), half c % 2
+                return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(
+                    static_cast<int>((16 * m4 + ((2 * s + (c >> 1)) ^ swz)) * 4), it.d));
+            };
+            auto shuffle_quants = [&](int s) {
+                v2i bq;
+                bq.x = __builtin_amdgcn_ds_bpermute(src_q, it.q[s].x);
+                bq.y = __builtin_amdgcn_ds_bpermute(src_q, it.q[s].y);
+                return bq;
+            };
+            // Items with all eight steps inside the row (every item when nb % 32 == 0, as for all layer
+            // shapes) take a copy of the loop in which the step count is a constant: the selects that
+            // guard the row's end and the address arithmetic behind them fold away (about ten of the
+            // fifty-odd instructions of a step).
+            auto run_steps = [&](auto full_tag) {
+            constexpr bool kFull = decltype(full_tag)::value;
+            const uint32_t nvalid = kFull ? 8u : vsteps;
+            uint32_t dword_nxt = shuffle_scale(0);
+            v2i bq_nxt = shuffle_quants(0);
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
                 long a_cur[MG];
                 float4 dx_cur[MG];
 #pragma unroll
                 for (int g = 0; g < MG; ++g) { a_cur[g] = a_nxt[g]; dx_cur[g] = dx_nxt[g]; }
+                const uint32_t dword = dword_nxt;
+                const v2i bq = bq_nxt;
                 if (s < 7) {
                     // steps past the row's end read step 0 again (finite values; their weight scale is zero)
-                    const uint32_t sn = static_cast<uint32_t>(s + 1) < vsteps ? s + 1 : 0;
+                    const uint32_t sn = static_cast<uint32_t>(s + 1) < nvalid ? s + 1 : 0;
 #pragma unroll
                     for (int g = 0; g < MG; ++g) {
                         a_nxt[g] = *reinterpret_cast<const long *>(xq_chunk + a_row[g] + sn * 128);
                         dx_nxt[g] = load_dx(xd_chunk + sn * 4 * MP * kSc + 4 * kSc * g);
                     }
+                    dword_nxt = shuffle_scale(s + 1);
+                    bq_nxt = shuffle_quants(s + 1);
                 }
-                // halfword 4 s + c of the row's scales: dword 2 s + c / 2 (held by lane 16 r + 2 s + c / 2), half c % 2
-                const uint32_t dword = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(
-                    static_cast<int>((16 * m4 + ((2 * s + (c >> 1)) ^ swz)) * 4), it.d));
+                // keeps the compiler's scheduler from sinking the look-ahead above back to its uses
+                __builtin_amdgcn_sched_barrier(0);
                 const uint16_t hbits = static_cast<uint16_t>((c & 1u) ? (dword >> 16) : (dword & 0xffffu));
-                const float dw = static_cast<uint32_t>(s) < vsteps ? half_bits_to_float(hbits) : 0.0f;
+                const float dw = static_cast<uint32_t>(s) < nvalid ? half_bits_to_float(hbits) : 0.0f;
                 const float cw = -kMagic * dw;
-                v2i bq;
-                bq.x = __builtin_amdgcn_ds_bpermute(src_q, it.q[s].x);
-                bq.y = __builtin_amdgcn_ds_bpermute(src_q, it.q[s].y);
                 const long b = __builtin_bit_cast(long, bq);
                 v4i r[MG];
 #pragma unroll
@@ -358,6 +383,9 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
                     acc[g][3] = fmaf(fmaf(as_f32(r[g].w), dw, cw), dx_cur[g].w, acc[g][3]);
                 }
             }
+            };
+            if (vsteps == 8) run_steps(std::true_type{});
+            else run_steps(std::false_type{});
             ++cstep;
             const uint32_t done = t + d + 1;
             if (done <= n_items && (cstep == nitems || done == n_items)) {

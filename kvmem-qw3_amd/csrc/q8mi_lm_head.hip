@@ -120,15 +120,22 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
 // Matrix-core variant for 3 or more verify rows (see q8mi_gemv_mfma_core.hpp): same unit and
 // item decomposition as the GEMV's matrix-core kernel at the same grid, so the logits are the
 // same bits as that GEMV's.
+//
+// A wave keeps a running (max, lowest index) per activation row for the units it streams from
+// their first to their last item: the four chunk sums of such a unit are brought together with
+// three lane shuffles and never go to LDS.  Only the units a wave shares with a neighbour (at most
+// the first and the last of its range) are parked, two slots per wave, and added up in wave order
+// after the stream.  LDS use does not grow with the number of rows, so one workgroup per CU
+// covers a vocabulary of any size in a single pass.
 template <int MG, int THREADS>
 __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
         const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, uint32_t rows, uint32_t nb, uint32_t batch,
         q8mi_argmax_pair *__restrict__ partial, float *__restrict__ logits, uint32_t stride_logits,
-        int interleave, uint32_t x_bytes, uint32_t park_floats) {
+        int interleave, uint32_t x_bytes) {
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr uint32_t MP = 4 * MG;
     constexpr uint32_t kWaves = THREADS / kWave;
-    constexpr uint32_t kPerUnit = 4 * kMfmaUnitRows * MP;
+    constexpr uint32_t kPerUnit = 4 * kMfmaUnitRows * MP;   // [chunk][row][activation row]
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, r = lane & 3u;
@@ -140,8 +147,15 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
     const uint32_t n_items = ucount * nitems;
     uint32_t i0, i1;
     wave_items(n_items, wave, kWaves, i0, i1);
-    float *park_base = reinterpret_cast<float *>(smem + x_bytes);
-    float *my_park = park_base + wave * park_floats;
+    float *park_base = reinterpret_cast<float *>(smem + x_bytes);   // [wave][2][kPerUnit]
+    float *my_park = park_base + wave * 2 * kPerUnit;
+    const uint32_t kf_mine = i0 / nitems;
+
+    // running best of the rows this lane finishes (lanes 0..3: row 4 u + lane of every whole unit)
+    float bv[MP];
+    int bi[MP];
+#pragma unroll
+    for (uint32_t m = 0; m < MP; ++m) { bv[m] = -INFINITY; bi[m] = -1; }
 
     auto row_ptr = [&](uint32_t u) -> const uint8_t * {
         uint32_t row = kMfmaUnitRows * u + q;
@@ -149,8 +163,29 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
         return w + row * row_bytes;
     };
     auto park = [&](uint32_t kk, auto &acc) {
-        if (q == c) {
-            float *dst = my_park + kk * kPerUnit + (c * kMfmaUnitRows + r) * MP;
+        const uint32_t k = kf_mine + kk;
+        const bool whole = k * nitems >= i0 && (k + 1) * nitems <= i1;   // wave-uniform
+        if (whole) {
+            const int row = static_cast<int>(kMfmaUnitRows * useq.unit(k) + r);
+#pragma unroll
+            for (int g = 0; g < MG; ++g) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    // chunk c of fragment row r sits in lane 20 c + r
+                    const float e0 = acc[g][v];
+                    const float e1 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((20 + r) * 4), as_i32(e0)));
+                    const float e2 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((40 + r) * 4), as_i32(e0)));
+                    const float e3 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((60 + r) * 4), as_i32(e0)));
+                    const float s = 0.0f + (((e0 + e1) + e2) + e3);   // the sum the combine below forms
+                    const uint32_t m = 4 * g + v;
+                    if (lane < kMfmaUnitRows && static_cast<uint32_t>(row) < rows && m < batch) {
+                        if (beats(s, row, bv[m], bi[m])) { bv[m] = s; bi[m] = row; }
+                        if (logits != nullptr) logits[static_cast<uint64_t>(m) * stride_logits + row] = s;
+                    }
+                }
+            }
+        } else if (q == c) {
+            float *dst = my_park + (k == kf_mine ? 0 : 1) * kPerUnit + (c * kMfmaUnitRows + r) * MP;
 #pragma unroll
             for (int g = 0; g < MG; ++g) {
                 float4 v;
@@ -160,43 +195,62 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
         }
     };
     mfma_stream<MG, THREADS, false, false>(smem, y, nb, batch, 0, useq, i0, i1, row_ptr, park);
-    __syncthreads();
 
-    __shared__ uint32_t s_kf[kWaves], s_kl[kWaves];
+    // item ranges of the waves, for the shared units
+    __shared__ uint32_t s_i0[kWaves], s_i1[kWaves];
     if (threadIdx.x < kWaves) {
         uint32_t a0, a1;
         wave_items(n_items, threadIdx.x, kWaves, a0, a1);
-        s_kf[threadIdx.x] = a1 > a0 ? a0 / nitems : 1u;
-        s_kl[threadIdx.x] = a1 > a0 ? (a1 - 1) / nitems : 0u;
+        s_i0[threadIdx.x] = a0;
+        s_i1[threadIdx.x] = a1;
     }
     __syncthreads();
-    auto total_of = [&](uint32_t k, uint32_t rr, uint32_t m) {
-        float t = 0.0f;
+    // Shared units: candidate (wave wv, slot sl, fragment row rr) is handled by thread 8 wv + 4 sl + rr
+    // when wave wv holds the unit's first item; the partial sums of every wave that touched the unit
+    // are added in wave order, each as ((c0 + c1) + c2) + c3.
+    if (threadIdx.x < kWaves * 8) {
+        const uint32_t wv = threadIdx.x / 8, sl = (threadIdx.x / 4) % 2, rr = threadIdx.x % 4;
+        const uint32_t a0 = s_i0[wv], a1 = s_i1[wv];
+        if (a1 > a0) {
+            const uint32_t kf = a0 / nitems, kl = (a1 - 1) / nitems;
+            const uint32_t k = sl == 0 ? kf : kl;
+            const bool whole = k * nitems >= a0 && (k + 1) * nitems <= a1;
+            const bool first_holder = k * nitems >= a0;       // the unit's first item is in this wave's range
+            if (!whole && first_holder && (sl == 0 || kl != kf)) {
+                const uint32_t row = kMfmaUnitRows * useq.unit(k) + rr;
+                if (row < rows) {
+                    for (uint32_t m = 0; m < batch; ++m) {
+                        float t = 0.0f;
+                        for (uint32_t w2 = wv; w2 < kWaves; ++w2) {
+                            const uint32_t b0 = s_i0[w2], b1 = s_i1[w2];
+                            if (b1 <= b0) continue;
+                            const uint32_t kf2 = b0 / nitems, kl2 = (b1 - 1) / nitems;
+                            if (k < kf2) break;
+                            if (k > kl2) continue;
+                            const float *e = park_base + (w2 * 2 + (k == kf2 ? 0 : 1)) * kPerUnit + rr * MP + m;
+                            t += ((e[0] + e[kMfmaUnitRows * MP]) + e[2 * kMfmaUnitRows * MP]) + e[3 * kMfmaUnitRows * MP];
+                        }
+                        if (logits != nullptr) logits[static_cast<uint64_t>(m) * stride_logits + row] = t;
+                        // fold into this thread's running best (its own, if any, stays valid: lowest index wins ties)
 #pragma unroll
-        for (uint32_t wv = 0; wv < kWaves; ++wv) {
-            const uint32_t kf = s_kf[wv], kl = s_kl[wv];
-            if (k < kf || k > kl) continue;
-            const float *e = park_base + wv * park_floats + (k - kf) * kPerUnit + rr * MP + m;
-            t += ((e[0] + e[kMfmaUnitRows * MP]) + e[2 * kMfmaUnitRows * MP]) + e[3 * kMfmaUnitRows * MP];
+                        for (uint32_t mm = 0; mm < MP; ++mm)
+                            if (mm == m && beats(t, static_cast<int>(row), bv[mm], bi[mm])) { bv[mm] = t; bi[mm] = static_cast<int>(row); }
+                    }
+                }
+            }
         }
-        return t;
-    };
+    }
 
     __shared__ float sv[THREADS];
     __shared__ int si[THREADS];
     for (uint32_t m = 0; m < batch; ++m) {
-        float bv = -INFINITY;
-        int bi = -1;
-        for (uint32_t e = threadIdx.x; e < ucount * kMfmaUnitRows; e += THREADS) {   // rows in ascending order
-            const uint32_t k = e / kMfmaUnitRows, rr = e % kMfmaUnitRows;
-            const uint32_t row = kMfmaUnitRows * useq.unit(k) + rr;
-            if (row >= rows) continue;
-            const float s = total_of(k, rr, m);
-            if (beats(s, static_cast<int>(row), bv, bi)) { bv = s; bi = static_cast<int>(row); }
-            if (logits != nullptr) logits[static_cast<uint64_t>(m) * stride_logits + row] = s;
-        }
-        sv[threadIdx.x] = bv;
-        si[threadIdx.x] = bi;
+        float v = -INFINITY;
+        int i = -1;
+#pragma unroll
+        for (uint32_t mm = 0; mm < MP; ++mm)
+            if (mm == m) { v = bv[mm]; i = bi[mm]; }
+        sv[threadIdx.x] = v;
+        si[threadIdx.x] = i;
         __syncthreads();
         for (uint32_t stride = THREADS / 2; stride > 0; stride >>= 1) {
             if (threadIdx.x < stride) {
@@ -310,23 +364,14 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
     auto kern = lm_head_mfma_kernel<MG, THREADS>;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     const uint32_t units = (rows + kMfmaUnitRows - 1) / kMfmaUnitRows;
-    // One workgroup per CU, the geometry of the GEMV's matrix-core launch, when the sums its waves
-    // park fit LDS; a very tall weight (the full vocabulary at 5..8 rows) takes 2..4 workgroups per
-    // CU instead, which run one after the other.
+    // One workgroup per CU, the geometry of the GEMV's matrix-core launch; the kernel parks only the
+    // units its waves share (two slots per wave), so the LDS need does not depend on the row count.
     const uint32_t x_bytes = mfma_x_lds_bytes(nb, batch, MG);
-    const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
     constexpr uint32_t kDynLimit = kLdsLimit - THREADS * 8 - 256;   // static LDS: the argmax tree and a few words
-    uint32_t grid = 0, park_floats = 0, lds = 0;
-    for (uint32_t mult = 1; mult <= 4; ++mult) {
-        uint32_t g = cus * mult;
-        if (g > units) g = units;
-        if (g > kMaxPartials) g = kMaxPartials;
-        const uint32_t per_group = (units + g - 1) / g;
-        const uint32_t pf = max_units_touched(per_group, nitems, THREADS / kWave) * mfma_park_floats_per_unit(MG);
-        const uint32_t need = x_bytes + (THREADS / kWave) * pf * 4;
-        if (need <= kDynLimit) { grid = g; park_floats = pf; lds = need; break; }
-    }
-    if (grid == 0) return fail(Q8MI_REJECTED, "lm_head (matrix-core variant): the parked sums do not fit LDS");
+    uint32_t grid = cus < units ? cus : units;
+    if (grid > kMaxPartials) grid = kMaxPartials;
+    const uint32_t lds = x_bytes + (THREADS / kWave) * 2 * mfma_park_floats_per_unit(MG) * 4;
+    if (lds > kDynLimit) return fail(Q8MI_REJECTED, "lm_head (matrix-core variant): the activations do not fit LDS");
     static thread_local bool granted = false;
     if (lds > 64u * 1024u && !granted) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -338,7 +383,7 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
     }
     *grid_out = grid;
     kern<<<grid, THREADS, lds, stream>>>(w, y, rows, nb, batch, partial, logits, stride_logits,
-                                         gemv_tuning().interleave, x_bytes, park_floats);
+                                         gemv_tuning().interleave, x_bytes);
     return check_launch("lm_head");
 }
 
@@ -350,7 +395,8 @@ bool lm_head_uses_mfma(uint32_t rows, uint32_t nb, uint32_t batch) {
     const uint32_t mg = (batch + 3) / 4;
     if (batch < static_cast<uint32_t>(gemv_tuning().mfma_from)) return false;
     if (mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u > kLdsLimit - 256) return false;
-    return rows <= 65536u || batch >= 7;
+    static const uint32_t tall_from = [] { const char *e = getenv("Q8MI_EXP_LMHEAD_MFMA_FROM"); return e ? static_cast<uint32_t>(atoi(e)) : 7u; }();
+    return rows <= 65536u || batch >= tall_from;
 }
 
 template <int M>
