@@ -390,13 +390,12 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
 // Matrix-core variant: for weights of up to 65536 rows under the GEMV's own rule (same kernel
 // family and geometry as q8mi_gemv at that batch, so the optional logits are the GEMV's bits), for
 // taller ones (the vocabulary) only from 7 verify rows on: there the dot-product variant streams
-// faster up to 6 rows (measured: 238..257 us against 248..267 us at 4..6 rows, 296 against 279 at 8).
+// faster up to 6 rows (measured: 237..257 us against 245..265 us at 4..6 rows, 296 against 265 at 8).
 bool lm_head_uses_mfma(uint32_t rows, uint32_t nb, uint32_t batch) {
     const uint32_t mg = (batch + 3) / 4;
     if (batch < static_cast<uint32_t>(gemv_tuning().mfma_from)) return false;
     if (mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u > kLdsLimit - 256) return false;
-    static const uint32_t tall_from = [] { const char *e = getenv("Q8MI_EXP_LMHEAD_MFMA_FROM"); return e ? static_cast<uint32_t>(atoi(e)) : 7u; }();
-    return rows <= 65536u || batch >= tall_from;
+    return rows <= 65536u || batch >= 7;
 }
 
 template <int M>
