@@ -255,7 +255,7 @@ def bench_read_probe(q8mi, hip, nbytes=1 << 30, reps=20):
     return round(nbytes / (t * 1e-3) / 1e9, 1)
 
 
-def bench_mfma_ceilings(q8mi, hip, iters=20000):
+def bench_mfma_ceilings(q8mi, hip, iters=5000):
     """Measured issue-rate ceilings of the matrix unit: int8 MFMAs alone, and with the scalar fp32
     FMAs that rescaling their results costs (2 per int32 sum; packed fp32 math is not available)."""
     L = q8mi.lib()
