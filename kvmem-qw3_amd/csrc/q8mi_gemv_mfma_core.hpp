@@ -70,6 +70,12 @@ inline uint32_t mfma_x_lds_bytes(uint32_t nb, uint32_t batch, uint32_t mg, bool 
 // Floats one wave parks per touched unit.
 inline uint32_t mfma_park_floats_per_unit(uint32_t mg) { return 4 * kMfmaUnitRows * 4 * mg; }
 
+// Items a wave keeps in flight (each 4 rows x 1 KiB of quants + their scales).
+#ifndef Q8MI_MFMA_DEPTH
+#define Q8MI_MFMA_DEPTH 2
+#endif
+constexpr int kMfmaDepth = Q8MI_MFMA_DEPTH;
+
 struct MfmaItem {
     v2i q[8];   // per step: bytes 8 t .. 8 t + 7 of the step's 128 bytes of row L / 16 (memory order),
                 // t = (L % 16) ^ 2 for rows 2 and 3, L % 16 for rows 0 and 1
@@ -232,14 +238,14 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
         return;
     }
     const uint32_t n_items = i1 - i0;
-    const uint32_t n_padded = (n_items + 1) / 2 * 2;
+
 
     // activation loads first, the first weight items behind them (they stay in flight while the
     // activations are converted)
     MfmaStage<MG, THREADS, HS> xstage;
     if constexpr (!D4) xstage.issue(y, nb, batch);
     asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
-    MfmaItem items[2];
+    MfmaItem items[kMfmaDepth];
     uint32_t ik = i0 / nitems, istep = i0 % nitems, ileft = n_items;
     const uint8_t *irow = row_ptr(useq.unit(ik));
     // Lane L loads slot (L % 16) ^ swz of row L / 16, swz = 2 for rows 2 and 3: the operand shuffle
@@ -265,8 +271,8 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
             }
         }
     };
-    issue(items[0]);
-    issue(items[1]);
+#pragma unroll
+    for (int d = 0; d < kMfmaDepth; ++d) issue(items[d]);
     asm volatile("" ::: "memory");   // keeps the loads above from being moved below the staging barrier
     if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch, d4_batch_total);
     else xstage.finish(smem, y, nb, batch);
@@ -294,10 +300,8 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
         for (int v = 0; v < 4; ++v) acc[g][v] = 0.0f;
 
     uint32_t cstep = i0 % nitems, kk = 0;
-    for (uint32_t t = 0; t < n_padded; t += 2) {
-#pragma unroll
-        for (int d = 0; d < 2; ++d) {
-            const MfmaItem &it = items[d];
+    // one item: `done` counts the items consumed so far, this one included
+    auto consume = [&](const MfmaItem &it, uint32_t done) {
             const uint32_t left = nb - cstep * kMfmaItemBlocks;
             const uint32_t vsteps = left >= kMfmaItemBlocks ? 8u : left / 4;
             const uint8_t *xq_chunk = xq + cstep * 1024;
@@ -387,8 +391,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
             if (vsteps == 8) run_steps(std::true_type{});
             else run_steps(std::false_type{});
             ++cstep;
-            const uint32_t done = t + d + 1;
-            if (done <= n_items && (cstep == nitems || done == n_items)) {
+            if (cstep == nitems || done == n_items) {
                 park(kk, acc);
                 ++kk;
 #pragma unroll
@@ -397,9 +400,21 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
                     for (int v = 0; v < 4; ++v) acc[g][v] = 0.0f;
             }
             if (cstep == nitems) cstep = 0;
+    };
+    // Whole rounds of kMfmaDepth items, each slot refilled as soon as it is consumed (past the
+    // last item the refills re-read it, so the loop stays branch-free and the load counters
+    // exact); then the items of a last, partial round, without refills.
+    uint32_t t = 0;
+    for (; t + kMfmaDepth <= n_items; t += kMfmaDepth) {
+#pragma unroll
+        for (int d = 0; d < kMfmaDepth; ++d) {
+            consume(items[d], t + d + 1);
             issue(items[d]);
         }
     }
+#pragma unroll
+    for (int d = 0; d < kMfmaDepth - 1; ++d)
+        if (t + d < n_items) consume(items[d], t + d + 1);
 }
 
 }  // namespace q8mi
