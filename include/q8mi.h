@@ -121,6 +121,49 @@ int q8mi_qgemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uin
                        uint32_t cols, uint32_t batch, uint32_t stride_dst0, uint32_t stride_dst1,
                        uint32_t stride_dst2, uint32_t stride_dst3, void *stream);
 
+/* ---- RMS norm in front of the quantizer ------------------------------------
+ * out[j][i] = (x[j][i] * scale_j) * weight[i], scale_j = 1 / sqrt(mean_i x[j][i]^2 + eps):
+ * replaces rms_norm_kernel_vec / rms_norm_kernel (src/kernels_cuda.cu:1945-2010,
+ * 2057-2073) as launched by rms_norm and rms_norm_batch (:14748-14816); rows of x
+ * are stride_x_row floats apart (the reference's are dense, stride = cols).  Any
+ * cols and alignment (16-byte aligned pointers and strides that are multiples of 4
+ * take vector loads).  The reference's sum of squares follows its block size and its
+ * root is the GPU's approximate rsqrtf, so its last bits are not restated: this
+ * kernel sums in a fixed order (256 strided partials of 4-float chunks, then a
+ * balanced tree) and takes an IEEE root and quotient, which a CPU follows bit for
+ * bit; against the reference that is a difference of a few units in the last place. */
+int q8mi_rms_norm(const float *x, const float *weight, float *out, uint32_t batch, uint32_t cols,
+                  uint32_t stride_x_row, uint32_t stride_out_row, float eps, void *stream);
+/* q8mi_rms_norm followed by q8mi_quantize_q8_1 of its output, in one pass over x
+ * (same bits as the two calls): the step between the executor's rms_norm and
+ * launch_quantize_q8_1 inside every q8_0_matvec* / q8_0_matmul* operator
+ * (src/kernels_cuda.cu:11250, 12047, 12241).  `normalized` (rows
+ * stride_normalized_row floats apart) also receives the fp32 rows unless NULL.
+ * Rejects cols % 32 != 0. */
+int q8mi_rms_norm_quantize_q8_1(const float *x, const float *weight, float *normalized, void *y_q8_1,
+                                uint32_t batch, uint32_t cols, uint32_t stride_x_row,
+                                uint32_t stride_normalized_row, float eps, void *stream);
+/* One activation row normalised, quantized and multiplied in ONE launch: what
+ * rms_norm_q8_0_matmul_fanout (include/qw3/device_backend.hpp:421-444) and the
+ * rms_norm + q8_0_matvec / q8_0_matvec_silu_mul pairs of the decode loop
+ * (src/qwen_executor.cpp:5734-5792) do in three.  Every workgroup repeats the norm
+ * and the quantization on its own copy of the row while its first weight bytes are
+ * in flight; workgroup 0 also writes the fp32 row to `normalized` unless NULL.  The
+ * outputs are the bits of q8mi_rms_norm followed by the matching q8mi_qgemv* call.
+ * Outputs are dense (one row).  Q8MI_REJECTED (nothing launched; use
+ * q8mi_rms_norm_quantize_q8_1 and the GEMV) when batch != 1, cols is above 6144 or
+ * not a multiple of 256, or x / weight / normalized are not 16-byte aligned. */
+int q8mi_nqgemv(const uint8_t *weight, const float *x, const float *norm_weight, float eps, float *normalized,
+                void *dst, int dst_is_bf16, uint32_t rows, uint32_t cols, uint32_t batch, void *stream);
+int q8mi_nqgemv_silu_mul(const uint8_t *weight_gate, const uint8_t *weight_up, const float *x,
+                         const float *norm_weight, float eps, float *normalized, float *dst, uint32_t rows,
+                         uint32_t cols, uint32_t batch, void *stream);
+int q8mi_nqgemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uint8_t *weight2,
+                        const uint8_t *weight3, const float *x, const float *norm_weight, float eps,
+                        float *normalized, float *dst0, float *dst1, float *dst2, float *dst3, uint32_t rows0,
+                        uint32_t rows1, uint32_t rows2, uint32_t rows3, uint32_t cols, uint32_t batch,
+                        void *stream);
+
 /* ---- D4 activation quantizer + int8 MFMA GEMM ---------------------------- */
 /* replaces q8_1_mmq_scratch_bytes, src/mmvq_q8.cu:726-729 */
 size_t q8mi_q8_1_d4_scratch_bytes(uint32_t batch, uint32_t cols);

@@ -34,6 +34,9 @@ struct GemvParams {
     const uint8_t *y;     // Q8_1 blocks, [batch][nb] (null when xf is set)
     const float *xf;      // fp32 activations to be quantized while staging (fused entry points)
     uint32_t x_stride;    // floats between rows of xf
+    const float *norm_w;  // RMS-norm weights: xf is one raw row, normalised while staging (else null)
+    float *normalized;    // where the normalised row is also written (may be null)
+    float eps;
     uint32_t total_rows;  // rows of the concatenated space (SwiGLU: rows of one weight)
     uint32_t units;
     uint32_t nb;
@@ -122,7 +125,10 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
     auto park = [&](uint32_t kk, float total) {
         if (lane < kPerUnit) my_park[kk * kPerUnit + lane] = total;
     };
-    gemv_stream<M, R, THREADS, XMODE>(smem, p.y, p.xf, p.x_stride, p.nb, useq, i0, i1, rows_of, park);
+    // the reduction of the fused norm borrows the first floats of the park area, which is not
+    // written before the staging barrier
+    const XIn in{p.y, p.xf, p.x_stride, p.norm_w, p.eps, p.normalized, park_base};
+    gemv_stream<M, R, THREADS, XMODE>(smem, in, p.nb, useq, i0, i1, rows_of, park);
 #ifdef Q8MI_TRACE
     const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
 #endif
@@ -387,6 +393,20 @@ int launch_ms(const GemvParams &p, hipStream_t stream) {
     const uint32_t xb = x_lds_bytes(p.nb, M);
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
     const int forced = gemv_tuning().threads;
+    if (p.norm_w != nullptr) {   // fused norm + quantizer: one row, held in registers between the two passes
+        if constexpr (M == 1) {
+            const uint32_t cols = p.nb * kQK;
+            if (cols > StageF32<1, 256, true>::kBatch * 256u * 4u || xb + park_256 > 76u * 1024u)
+                return fail(Q8MI_REJECTED, "nqgemv: rows of %u columns are not served (at most %u)", cols,
+                            StageF32<1, 256, true>::kBatch * 256u * 4u);
+            auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+            if (!al(p.xf) || !al(p.norm_w) || (p.normalized != nullptr && !al(p.normalized)))
+                return fail(Q8MI_REJECTED, "nqgemv: activations, norm weights and normalised output must be 16-byte aligned");
+            return launch_inst<1, 256, kXNormF32, SILU>(p, xb, stream);
+        } else {
+            return fail(Q8MI_REJECTED, "nqgemv: batch %d above 1 (normalise and quantize once, then use the GEMV)", M);
+        }
+    }
     if (p.xf != nullptr) {   // fused quantizer: the activations must fit LDS
         if (M > 2) return fail(Q8MI_REJECTED, "qgemv: batch %d above 2 (quantize once and use the GEMV instead)", M);
         // rows above 8192 columns: one 1024-thread workgroup per CU quantizes them once per CU instead of twice
@@ -507,6 +527,9 @@ struct XSource {
     const void *y_q8_1;
     const float *xf;
     uint32_t stride_x;
+    const float *norm_w = nullptr;   // set: xf is one raw row to be RMS-normalised first
+    float eps = 0.0f;
+    float *normalized = nullptr;
 };
 
 GemvParams single(const uint8_t *w, const XSource &x, void *dst, uint32_t rows, uint32_t cols,
@@ -519,6 +542,9 @@ GemvParams single(const uint8_t *w, const XSource &x, void *dst, uint32_t rows, 
     p.y = static_cast<const uint8_t *>(x.y_q8_1);
     p.xf = x.xf;
     p.x_stride = x.stride_x;
+    p.norm_w = x.norm_w;
+    p.eps = x.eps;
+    p.normalized = x.normalized;
     p.total_rows = rows;
     p.units = 0;   // set per batch size at launch
     p.nb = cols / kQK;
@@ -680,6 +706,9 @@ static int run_fanout4(const uint8_t *w0, const uint8_t *w1, const uint8_t *w2, 
     p.y = static_cast<const uint8_t *>(y.y_q8_1);
     p.xf = y.xf;
     p.x_stride = y.stride_x;
+    p.norm_w = y.norm_w;
+    p.eps = y.eps;
+    p.normalized = y.normalized;
     p.total_rows = total;
     p.units = 0;
     p.nb = cols / kQK;
@@ -730,4 +759,35 @@ extern "C" int q8mi_gemv_two(const uint8_t *w0, const uint8_t *w1, const void *y
     if (rows == 0) return Q8MI_OK;
     return q8mi_gemv_fanout4(w0, w1, nullptr, nullptr, y, dst0, dst1, nullptr, nullptr, rows, rows,
                              0, 0, cols, batch, stride, stride, 0, 0, stream);
+}
+
+// ---- entry points that RMS-normalise and quantize one activation row inside the GEMV ----------
+static int norm_gate(const char *what, const float *x, const float *norm_weight, uint32_t batch) {
+    if (x == nullptr || norm_weight == nullptr) return fail(Q8MI_REJECTED, "%s: null pointer", what);
+    if (batch != 1) return fail(Q8MI_REJECTED, "%s: batch %u (one row only)", what, batch);
+    return Q8MI_OK;
+}
+
+extern "C" int q8mi_nqgemv(const uint8_t *w, const float *x, const float *norm_weight, float eps, float *normalized,
+                           void *dst, int dst_is_bf16, uint32_t rows, uint32_t cols, uint32_t batch, void *stream) {
+    if (int rc = norm_gate("nqgemv", x, norm_weight, batch)) return rc;
+    return run_single("nqgemv", dst_is_bf16 ? kStoreBF16 : kStoreF32, w, XSource{nullptr, x, cols, norm_weight, eps, normalized},
+                      dst, rows, cols, batch, rows, stream);
+}
+
+extern "C" int q8mi_nqgemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const float *x, const float *norm_weight,
+                                    float eps, float *normalized, float *dst, uint32_t rows, uint32_t cols,
+                                    uint32_t batch, void *stream) {
+    if (int rc = norm_gate("nqgemv_silu_mul", x, norm_weight, batch)) return rc;
+    return run_silu_mul(wg, wu, XSource{nullptr, x, cols, norm_weight, eps, normalized}, dst, rows, cols, batch, rows,
+                        stream);
+}
+
+extern "C" int q8mi_nqgemv_fanout4(const uint8_t *w0, const uint8_t *w1, const uint8_t *w2, const uint8_t *w3,
+                                   const float *x, const float *norm_weight, float eps, float *normalized, float *d0,
+                                   float *d1, float *d2, float *d3, uint32_t rows0, uint32_t rows1, uint32_t rows2,
+                                   uint32_t rows3, uint32_t cols, uint32_t batch, void *stream) {
+    if (int rc = norm_gate("nqgemv_fanout4", x, norm_weight, batch)) return rc;
+    return run_fanout4(w0, w1, w2, w3, XSource{nullptr, x, cols, norm_weight, eps, normalized}, d0, d1, d2, d3, rows0,
+                       rows1, rows2, rows3, cols, batch, rows0, rows1, rows2, rows3, stream);
 }

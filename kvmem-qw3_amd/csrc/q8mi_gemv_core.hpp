@@ -46,8 +46,20 @@ constexpr uint32_t kLdsLimit = 160u * 1024u;    // LDS per CU on gfx950
 constexpr uint32_t kParkFloats = 1024;           // per-wave LDS area (floats) for the sums of the units it touched
 
 // Where a lane finds the activations: Q8_1 blocks staged in LDS, Q8_1 blocks read from
-// global memory, or fp32 activations quantized to Q8_1 while they are staged in LDS.
-enum XMode : int { kXLds = 0, kXGlobal = 1, kXF32 = 2 };
+// global memory, fp32 activations quantized to Q8_1 while they are staged in LDS, or one fp32
+// row that is RMS-normalised and then quantized while it is staged.
+enum XMode : int { kXLds = 0, kXGlobal = 1, kXF32 = 2, kXNormF32 = 3 };
+
+// The activations of a launch as the staging code sees them.
+struct XIn {
+    const uint8_t *y;      // Q8_1 blocks (kXLds, kXGlobal)
+    const float *xf;       // fp32 rows (kXF32, kXNormF32)
+    uint32_t stride_x;     // floats between rows of xf
+    const float *norm_w;   // kXNormF32: the norm's weights, one per column
+    float eps;
+    float *normalized;     // kXNormF32: where workgroup 0 leaves the normalised row (may be null)
+    float *red;            // kXNormF32: four floats of LDS for the reduction
+};
 
 // LDS footprint of `batch` activation rows: per 64-block step 128 16-byte
 // pieces of int8 and 64 fp32 scales, zero-padded to whole steps.
@@ -163,10 +175,16 @@ struct StageLds {
 // stand-alone quantizer uses, so the int8 values and the fp16-rounded scales are the same bits.
 // The block sum `s` of Q8_1 is not needed by Q8_0 dots and is not formed.  x rows are
 // stride_x floats apart; cols = 32 * nb.  Ends with a workgroup barrier.
-template <int M, int THREADS>
+//
+// NORM: the single row (M == 1, at most kBatch * THREADS * 4 columns, THREADS == 256) is
+// RMS-normalised first, with the stand-alone kernel's arithmetic: the sum of squares over the
+// registers already loaded, one more workgroup barrier, then (x * scale) * weight.
+template <int M, int THREADS, bool NORM = false>
 struct StageF32 {
     static constexpr int kBatch = 6;   // float4 loads in flight per thread: one trip for a 6144-column row at 256 threads
+    static_assert(!NORM || (M == 1 && THREADS == kNormThreads), "the fused norm handles one row per 256-thread workgroup");
     Float4 v[kBatch];
+    Float4 nw[NORM ? kBatch : 1];
 
     __device__ __forceinline__ static Float4 fetch(const float *x, uint32_t stride_x, uint32_t per_row,
                                                    uint32_t total, uint32_t c, bool vec) {
@@ -178,15 +196,39 @@ struct StageF32 {
     }
 
     // First trip of loads only (see StageLds::issue).
-    __device__ __forceinline__ void issue(const float *x, uint32_t stride_x, uint32_t nb) {
+    __device__ __forceinline__ void issue(const XIn &in, uint32_t nb) {
+        const float *x = in.xf;
+        const uint32_t stride_x = in.stride_x;
         const uint32_t per_row = nb * 8, total = static_cast<uint32_t>(M) * per_row;
         const bool vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride_x % 4 == 0);
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) v[u] = fetch(x, stride_x, per_row, total, u * THREADS + threadIdx.x, vec);
+        if constexpr (NORM) {   // the host only takes this path with 16-byte aligned weights
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) nw[u] = fetch(in.norm_w, 0, per_row, total, u * THREADS + threadIdx.x, true);
+        }
     }
 
-    __device__ __forceinline__ void finish(uint8_t *smem, const float *x, uint32_t stride_x,
-                                           uint32_t nb) {
+    __device__ __forceinline__ void finish(uint8_t *smem, const XIn &in, uint32_t nb) {
+        const float *x = in.xf;
+        const uint32_t stride_x = in.stride_x;
+        if constexpr (NORM) {
+            const uint32_t chunks = nb * 8;   // <= kBatch * THREADS, checked on the host
+            float partial = 0.0f;
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const float q = chunk_squares(v[u]);
+                partial += (u * THREADS + threadIdx.x < chunks) ? q : 0.0f;   // fetch() re-reads chunk 0 past the end
+            }
+            const float scale = rms_scale(block_tree_sum_256(partial, in.red), nb * 32, in.eps);
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                v[u] = rms_apply(v[u], scale, nw[u]);
+                const uint32_t c = u * THREADS + threadIdx.x;
+                if (in.normalized != nullptr && blockIdx.x == 0 && c < chunks)
+                    *reinterpret_cast<float4 *>(in.normalized + c * 4) = make_float4(v[u].x, v[u].y, v[u].z, v[u].w);
+            }
+        }
         const uint32_t nsteps = (nb * 2 + 127) / 128;
         uint32_t *wq = reinterpret_cast<uint32_t *>(smem);
         float *wd = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
@@ -232,25 +274,22 @@ struct StageF32 {
 template <int M, int THREADS, int XMODE>
 struct XStage {
     StageLds<M, THREADS> lds;
-    StageF32<M, THREADS> f32;
-    __device__ __forceinline__ void issue(const uint8_t *y, const float *xf,
-                                          uint32_t stride_x, uint32_t nb) {
-        if constexpr (XMODE == kXLds) lds.issue(y, nb);
-        if constexpr (XMODE == kXF32) f32.issue(xf, stride_x, nb);
+    StageF32<M, THREADS, XMODE == kXNormF32> f32;
+    __device__ __forceinline__ void issue(const XIn &in, uint32_t nb) {
+        if constexpr (XMODE == kXLds) lds.issue(in.y, nb);
+        if constexpr (XMODE == kXF32 || XMODE == kXNormF32) f32.issue(in, nb);
     }
-    __device__ __forceinline__ void finish(uint8_t *smem, const uint8_t *y,
-                                           const float *xf, uint32_t stride_x, uint32_t nb) {
-        if constexpr (XMODE == kXLds) lds.finish(smem, y, nb);
-        if constexpr (XMODE == kXF32) f32.finish(smem, xf, stride_x, nb);
+    __device__ __forceinline__ void finish(uint8_t *smem, const XIn &in, uint32_t nb) {
+        if constexpr (XMODE == kXLds) lds.finish(smem, in.y, nb);
+        if constexpr (XMODE == kXF32 || XMODE == kXNormF32) f32.finish(smem, in, nb);
     }
 };
 
 template <int M, int THREADS, int XMODE>
-__device__ __forceinline__ void stage_x(uint8_t *smem, const uint8_t *y, const float *xf,
-                                        uint32_t stride_x, uint32_t nb) {
+__device__ __forceinline__ void stage_x(uint8_t *smem, const XIn &in, uint32_t nb) {
     XStage<M, THREADS, XMODE> xs;
-    xs.issue(y, xf, stride_x, nb);
-    xs.finish(smem, y, xf, stride_x, nb);
+    xs.issue(in, nb);
+    xs.finish(smem, in, nb);
 }
 
 // Weight bytes of one item held by a lane.
@@ -398,16 +437,16 @@ __device__ __forceinline__ UnitSeq group_units(uint32_t units, uint32_t group, u
 // the last item and whose sums are never parked.
 // Must be called by every wave of the workgroup (it contains the staging barrier).
 template <int M, int R, int THREADS, int XMODE, class RowsOf, class Park>
-__device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *y,
-                                            const float *xf, uint32_t stride_x, uint32_t nb,
+__device__ __forceinline__ void gemv_stream(uint8_t *smem, const XIn &in, uint32_t nb,
                                             const UnitSeq &useq, uint32_t i0, uint32_t i1,
                                             RowsOf rows_of, Park park) {
+    const uint8_t *y = in.y;
     const uint32_t nsteps = (nb * 2 + 127) / 128;
     const uint32_t lane = threadIdx.x % kWave;
     const int *lds_q = reinterpret_cast<const int *>(smem);
     const float *lds_d = reinterpret_cast<const float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
     if (i1 <= i0) {   // wave-uniform; idle waves still take part in the staging barrier
-        stage_x<M, THREADS, XMODE>(smem, y, xf, stride_x, nb);
+        stage_x<M, THREADS, XMODE>(smem, in, nb);
         return;
     }
     const uint32_t n_items = i1 - i0;
@@ -417,7 +456,7 @@ __device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *y,
     // activation loads first, the first weight items behind them: the activations arrive first
     // and are converted while the weight loads are still in flight
     XStage<M, THREADS, XMODE> xs;
-    xs.issue(y, xf, stride_x, nb);
+    xs.issue(in, nb);
     asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
     Item<R> items[kDepth];
     // issue cursor: unit ordinal, step, items left to issue for real
@@ -442,7 +481,7 @@ __device__ __forceinline__ void gemv_stream(uint8_t *smem, const uint8_t *y,
     // keeps the loads above where they are: without it the compiler sinks them below the staging
     // barrier and the first weight bytes are requested only after the activations are in LDS
     asm volatile("" ::: "memory");
-    xs.finish(smem, y, xf, stride_x, nb);
+    xs.finish(smem, in, nb);
 
     float acc[M][R];
 #pragma unroll

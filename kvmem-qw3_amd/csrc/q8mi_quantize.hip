@@ -30,15 +30,7 @@ __global__ __launch_bounds__(kQuantThreads) void quantize_q8_1_kernel(
     float d;
     const uint32_t packed = quantize4_q8_1(v, d);
 
-    // level 1..3 of the reference tree across lanes, component-wise
-    float s0 = v.x, s1 = v.y, s2 = v.z, s3 = v.w;
-    s0 += swizzle_xor4(s0); s1 += swizzle_xor4(s1); s2 += swizzle_xor4(s2); s3 += swizzle_xor4(s3);
-    s0 += dpp_f32<kDppXor2>(s0); s1 += dpp_f32<kDppXor2>(s1);
-    s2 += dpp_f32<kDppXor2>(s2); s3 += dpp_f32<kDppXor2>(s3);
-    s0 += dpp_f32<kDppXor1>(s0); s1 += dpp_f32<kDppXor1>(s1);
-    s2 += dpp_f32<kDppXor1>(s2); s3 += dpp_f32<kDppXor1>(s3);
-    // level 4 and 5 inside the lane
-    const float sum = (s0 + s2) + (s1 + s3);
+    const float sum = block_sum_q8_1(v);
 
     const uint32_t kb = i0 / kQK;
     const uint32_t sub = (i0 % kQK) / kElemsPerLane;  // 0..7

@@ -75,4 +75,54 @@ __device__ __forceinline__ uint32_t quantize4_q8_1(const Float4 &v, float &d_out
     return pack4(q0, q1, q2, q3);
 }
 
+// Block sum of Q8_1 (the `s` field) for the lane's four values, with the reference's pairing
+// (i, i+16), (i, i+8), (i, i+4), (i, i+2), (i, i+1) of its 32-lane xor butterfly
+// (src/cuda_helpers.cuh:44-51): lane exchanges xor 4, 2, 1 cover the first three levels
+// component-wise, the last two are the in-lane adds.  Same calling rules as quantize4_q8_1.
+__device__ __forceinline__ float block_sum_q8_1(const Float4 &v) {
+    float s0 = v.x, s1 = v.y, s2 = v.z, s3 = v.w;
+    s0 += swizzle_xor4(s0); s1 += swizzle_xor4(s1); s2 += swizzle_xor4(s2); s3 += swizzle_xor4(s3);
+    s0 += dpp_f32<kDppXor2>(s0); s1 += dpp_f32<kDppXor2>(s1);
+    s2 += dpp_f32<kDppXor2>(s2); s3 += dpp_f32<kDppXor2>(s3);
+    s0 += dpp_f32<kDppXor1>(s0); s1 += dpp_f32<kDppXor1>(s1);
+    s2 += dpp_f32<kDppXor1>(s2); s3 += dpp_f32<kDppXor1>(s3);
+    return (s0 + s2) + (s1 + s3);
+}
+
+// ---- RMS norm pieces (shared by the stand-alone kernels and the GEMV that normalises while
+// staging, which must produce the same bits) ------------------------------------------------
+// A row is cut into chunks of four consecutive floats (the last one zero-padded).  Thread t of
+// the 256 adds the squares of chunks t, t + 256, t + 512, ... in that order, each chunk as
+// fma(w, w, fma(z, z, fma(y, y, x * x))); the 256 partials are added as a balanced binary tree
+// over the thread index (neighbours first).  scale = 1 / sqrt(sum / n + eps) with IEEE
+// division and square root; an output is (x * scale) * weight, rounded after each product
+// (the reference's expression, src/kernels_cuda.cu:1995-2007).
+constexpr uint32_t kNormThreads = 256;
+
+__device__ __forceinline__ float chunk_squares(const Float4 &v) {
+    return fmaf(v.w, v.w, fmaf(v.z, v.z, fmaf(v.y, v.y, v.x * v.x)));
+}
+
+// Total of the 256 per-thread partials; `red` = four floats of LDS nobody else touches until
+// the barrier that follows the caller's use of the result.  Contains one workgroup barrier.
+__device__ __forceinline__ float block_tree_sum_256(float partial, float *red) {
+    const float s = wave_sum(partial);   // balanced tree over the wave's 64 lanes
+    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__device__ __forceinline__ float rms_scale(float sum_squares, uint32_t n, float eps) {
+    return 1.0f / sqrtf(sum_squares / static_cast<float>(n) + eps);
+}
+
+__device__ __forceinline__ Float4 rms_apply(const Float4 &v, float scale, const Float4 &w) {
+    Float4 r;
+    r.x = (v.x * scale) * w.x;
+    r.y = (v.y * scale) * w.y;
+    r.z = (v.z * scale) * w.z;
+    r.w = (v.w * scale) * w.w;
+    return r;
+}
+
 }  // namespace q8mi

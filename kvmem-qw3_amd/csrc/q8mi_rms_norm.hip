@@ -1,0 +1,157 @@
+// RMS norm of activation rows, alone or fused with the Q8_1 quantizer that feeds the
+// Q8_0 GEMVs (the step in front of every projection group and of the LM head).
+// Reference: rms_norm_kernel_vec / rms_norm_kernel (src/kernels_cuda.cu:1945-2010,
+// 2057-2073), launched by rms_norm / rms_norm_batch (:14748-14816); the operators that
+// pair it with the projections are rms_norm_q8_0_matmul_*fanout
+// (include/qw3/device_backend.hpp:421-523).
+//
+//   out[j][i] = (x[j][i] * scale_j) * weight[i],  scale_j = 1 / sqrt(mean_i(x[j][i]^2) + eps)
+//
+// The reference leaves the order of the sum of squares to its block size and takes the
+// root with the hardware's approximate reciprocal square root, so its last bits cannot be
+// restated; this kernel fixes an order of its own (q8mi_quantize_core.hpp) and uses IEEE
+// division and square root, which a CPU can follow bit for bit.
+//
+// One 256-thread workgroup per row.  The first six chunks of a thread stay in registers
+// between the two passes (rows of up to 6144 columns are read once); longer rows are read
+// again, from cache.
+#include "q8mi_internal.hpp"
+#include "q8mi_quantize_core.hpp"
+
+namespace q8mi {
+namespace {
+
+constexpr uint32_t kHeld = 6;
+
+struct NormParams {
+    const float *x;
+    const float *weight;
+    float *out;      // may be null when y is set
+    uint8_t *y;      // Q8_1 blocks [batch][cols / 32], or null
+    uint32_t cols;
+    uint32_t stride_x;
+    uint32_t stride_out;
+    float eps;
+};
+
+// Chunk c of a row of n floats; elements past the row's end read as zero.
+template <bool VEC>
+__device__ __forceinline__ Float4 load_chunk(const float *row, uint32_t c, uint32_t n) {
+    if (VEC) return load4<true>(row + c * 4);   // n % 4 == 0
+    Float4 v;
+    const uint32_t i = c * 4;
+    v.x = i < n ? row[i] : 0.0f;
+    v.y = i + 1 < n ? row[i + 1] : 0.0f;
+    v.z = i + 2 < n ? row[i + 2] : 0.0f;
+    v.w = i + 3 < n ? row[i + 3] : 0.0f;
+    return v;
+}
+
+template <bool VEC>
+__device__ __forceinline__ void store_chunk(float *row, uint32_t c, uint32_t n, const Float4 &v) {
+    const uint32_t i = c * 4;
+    if (VEC) {
+        *reinterpret_cast<float4 *>(row + i) = make_float4(v.x, v.y, v.z, v.w);
+        return;
+    }
+    if (i < n) row[i] = v.x;
+    if (i + 1 < n) row[i + 1] = v.y;
+    if (i + 2 < n) row[i + 2] = v.z;
+    if (i + 3 < n) row[i + 3] = v.w;
+}
+
+template <bool VEC, bool QUANT>
+__global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const NormParams p) {
+    __shared__ float red[4];
+    const uint32_t j = blockIdx.x, t = threadIdx.x;
+    const float *x = p.x + static_cast<uint64_t>(j) * p.stride_x;
+    const uint32_t n = p.cols;
+    const uint32_t chunks = (n + 3) / 4;
+    const Float4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    Float4 held[kHeld];
+    float partial = 0.0f;
+#pragma unroll
+    for (uint32_t u = 0; u < kHeld; ++u) {
+        const uint32_t c = u * kNormThreads + t;
+        held[u] = c < chunks ? load_chunk<VEC>(x, c, n) : zero;
+        partial += chunk_squares(held[u]);   // + 0 for chunks past the end
+    }
+    for (uint32_t c = kHeld * kNormThreads + t; c < chunks; c += kNormThreads)
+        partial += chunk_squares(load_chunk<VEC>(x, c, n));
+    const float scale = rms_scale(block_tree_sum_256(partial, red), n, p.eps);
+
+    // All lanes walk the same trips: the quantizer's lane exchanges need wave-uniform control flow
+    // (cols % 32 == 0 there, so the eight lanes of a block are in or out together).
+    auto emit = [&](uint32_t c, const Float4 &v) {
+        const bool live = c < chunks;
+        const Float4 r = rms_apply(v, scale, live ? load_chunk<VEC>(p.weight, c, n) : zero);
+        if (live && p.out != nullptr) store_chunk<VEC>(p.out + static_cast<uint64_t>(j) * p.stride_out, c, n, r);
+        if constexpr (QUANT) {
+            float d;
+            const uint32_t packed = quantize4_q8_1(r, d);
+            const float sum = block_sum_q8_1(r);
+            if (live) {
+                uint32_t *blk = reinterpret_cast<uint32_t *>(
+                    p.y + (static_cast<uint64_t>(j) * (n / kQK) + c / 8) * kQ81Bytes);
+                blk[1 + c % 8] = packed;
+                if (c % 8 == 0)
+                    blk[0] = static_cast<uint32_t>(float_to_half_bits(d)) |
+                             (static_cast<uint32_t>(float_to_half_bits(sum)) << 16);
+            }
+        }
+    };
+#pragma unroll
+    for (uint32_t u = 0; u < kHeld; ++u) {
+        if (u * kNormThreads < chunks) emit(u * kNormThreads + t, held[u]);   // uniform
+    }
+    for (uint32_t base = kHeld * kNormThreads; base < chunks; base += kNormThreads) {
+        const uint32_t c = base + t;
+        emit(c, c < chunks ? load_chunk<VEC>(x, c, n) : zero);
+    }
+}
+
+bool aligned16(const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+int launch(const char *what, const NormParams &p, uint32_t batch, void *stream) {
+    if (p.x == nullptr || p.weight == nullptr) return fail(Q8MI_REJECTED, "%s: null pointer", what);
+    if (batch == 0 || p.cols == 0) return Q8MI_OK;
+    if (batch > 0x7fffffffu) return fail(Q8MI_REJECTED, "%s: batch %u too large for one launch", what, batch);
+    const bool quant = p.y != nullptr;
+    const bool vec = p.cols % 4 == 0 && aligned16(p.x) && aligned16(p.weight) && p.stride_x % 4 == 0 &&
+                     (p.out == nullptr || (aligned16(p.out) && p.stride_out % 4 == 0));
+    hipStream_t s = as_stream(stream);
+    if (quant) {
+        if (vec) rms_norm_kernel<true, true><<<batch, kNormThreads, 0, s>>>(p);
+        else rms_norm_kernel<false, true><<<batch, kNormThreads, 0, s>>>(p);
+    } else {
+        if (vec) rms_norm_kernel<true, false><<<batch, kNormThreads, 0, s>>>(p);
+        else rms_norm_kernel<false, false><<<batch, kNormThreads, 0, s>>>(p);
+    }
+    return check_launch(what);
+}
+
+}  // namespace
+}  // namespace q8mi
+
+using namespace q8mi;
+
+extern "C" int q8mi_rms_norm(const float *x, const float *weight, float *out, uint32_t batch, uint32_t cols,
+                             uint32_t stride_x_row, uint32_t stride_out_row, float eps, void *stream) {
+    if (out == nullptr) return fail(Q8MI_REJECTED, "rms_norm: null output");
+    NormParams p{};
+    p.x = x; p.weight = weight; p.out = out; p.y = nullptr;
+    p.cols = cols; p.stride_x = stride_x_row; p.stride_out = stride_out_row; p.eps = eps;
+    return launch("rms_norm", p, batch, stream);
+}
+
+extern "C" int q8mi_rms_norm_quantize_q8_1(const float *x, const float *weight, float *normalized, void *y,
+                                           uint32_t batch, uint32_t cols, uint32_t stride_x_row,
+                                           uint32_t stride_normalized_row, float eps, void *stream) {
+    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "rms_norm_quantize_q8_1: cols %u not a multiple of 32", cols);
+    if (y == nullptr) return fail(Q8MI_REJECTED, "rms_norm_quantize_q8_1: null output");
+    NormParams p{};
+    p.x = x; p.weight = weight; p.out = normalized; p.y = static_cast<uint8_t *>(y);
+    p.cols = cols; p.stride_x = stride_x_row; p.stride_out = stride_normalized_row; p.eps = eps;
+    return launch("rms_norm_quantize_q8_1", p, batch, stream);
+}

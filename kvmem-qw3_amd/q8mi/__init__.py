@@ -68,6 +68,12 @@ SIGNATURES = {
     "q8mi_qgemv_silu_mul": (_int, [_vp, _vp, _vp, _u32, _vp, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_qgemv_fanout4": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32,
                                   _u32, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_rms_norm": (_int, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_float, _vp]),
+    "q8mi_rms_norm_quantize_q8_1": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_float, _vp]),
+    "q8mi_nqgemv": (_int, [_vp, _vp, _vp, C.c_float, _vp, _vp, _int, _u32, _u32, _u32, _vp]),
+    "q8mi_nqgemv_silu_mul": (_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _u32, _u32, _u32, _vp]),
+    "q8mi_nqgemv_fanout4": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,
+                                   _u32, _u32, _u32, _vp]),
     "q8mi_probe_copy": (_int, [_vp, _vp, _u64, _vp]),
     "q8mi_synth_f32": (_int, [_vp, _u64, _u64, _u64, _int, C.c_float, _u32, C.c_float, _int]),
     "q8mi_synth_q8_0_weight": (_int, [_vp, _u64, _u64, _u64, C.c_float, _int]),

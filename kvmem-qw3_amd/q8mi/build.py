@@ -15,6 +15,7 @@ SOURCES = [
     "q8mi_lm_head.hip",
     "q8mi_argmax.hip",
     "q8mi_get_rows.hip",
+    "q8mi_rms_norm.hip",
     "q8mi_gemm.hip",
 ]
 

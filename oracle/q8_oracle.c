@@ -149,6 +149,35 @@ static inline const int8_t *w_quants(const uint8_t *w, uint64_t nb, uint64_t row
 }
 
 /* ------------------------------------------------------------------------- */
+/* RMS norm (expression: src/kernels_cuda.cu:1995-2007; order of the sum: see header) */
+
+int q8o_rms_norm(const float *x, const float *weight, float *out, uint32_t batch, uint32_t n,
+                 uint32_t stride_x_row, uint32_t stride_out_row, float eps) {
+    if (n == 0) return -1;
+    const uint32_t chunks = (n + 3) / 4;
+    for (uint32_t j = 0; j < batch; ++j) {
+        const float *row = x + (size_t)j * stride_x_row;
+        float partial[256];
+        for (uint32_t t = 0; t < 256; ++t) partial[t] = 0.0f;
+        for (uint32_t c = 0; c < chunks; ++c) {
+            float v[4];
+            for (uint32_t e = 0; e < 4; ++e) v[e] = (c * 4 + e < n) ? row[c * 4 + e] : 0.0f;
+            const float q = fmaf(v[3], v[3], fmaf(v[2], v[2], fmaf(v[1], v[1], v[0] * v[0])));
+            partial[c % 256] = partial[c % 256] + q;
+        }
+        for (uint32_t w = 1; w < 256; w *= 2)
+            for (uint32_t t = 0; t < 256; t += 2 * w) partial[t] = partial[t] + partial[t + w];
+        const float scale = 1.0f / sqrtf(partial[0] / (float)n + eps);
+        float *o = out + (size_t)j * stride_out_row;
+        for (uint32_t i = 0; i < n; ++i) {
+            const float xs = row[i] * scale;
+            o[i] = xs * weight[i];
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
 /* activation quantizers                                                     */
 
 /* The reference reduces 32 lanes with xor offsets 16, 8, 4, 2, 1

@@ -19,6 +19,9 @@
  *   q8o_repack_split_plane ...... byte-level numpy restatement, round trip
  *   q8o_quantize_q8_1 / _d4 ..... independent numpy restatement, closed forms
  *   q8o_get_row ................. numpy restatement (d * q is exact in fp32)
+ *   q8o_rms_norm ................ float64 truth within 4 ulp, closed forms
+ *                                 (constant rows, unit weights, scaling law),
+ *                                 independent numpy restatement of the order
  *   q8o_block_dot ............... int64 brute force, extreme values
  *   q8o_gemv*, q8o_gemm_d4 ...... reference closed form (cols*0.5*x), reference
  *                                 tolerance test restated (5e-3 abs / 1e-3 rel
@@ -28,7 +31,11 @@
  *   q8o_accept .................. brute force over all (M, prefix) pairs
  * Parity unpinned (needs the reference's GPU): the last-bit value of the
  * reference's own fp32 reduction tree and of `__expf`; both lie inside the
- * 1e-5 relative tolerance the GPU tests use.
+ * 1e-5 relative tolerance the GPU tests use.  q8o_rms_norm: parity unpinned
+ * against the reference's bits for the same reason (its sum of squares
+ * follows its block size and nvcc's contraction, its root is the GPU's
+ * approximate rsqrtf): the function fixes an order and IEEE operations of
+ * its own and is pinned against the mathematics only.
  */
 #ifndef Q8_ORACLE_H
 #define Q8_ORACLE_H
@@ -72,6 +79,18 @@ int q8o_repack_split_plane(const uint8_t *gguf_blocks, uint64_t rows, uint64_t c
 /* Dequantized row `row` of a split-plane weight: out[i] = fp32(d[i / 32]) * (float)q[i]
  * (exact: an fp16 value times an 8-bit integer).  src/kernels_cuda.cu:2075-2087. */
 int q8o_get_row(const uint8_t *w_split, uint64_t row, uint64_t cols, float *out);
+
+/* ---- RMS norm --------------------------------------------------------------- */
+/* out[i] = (x[i] * scale) * weight[i], scale = 1 / sqrtf(sum_i x[i]^2 / n + eps): the
+ * expression of src/kernels_cuda.cu:1995-2007 (and :2070-2072) with an IEEE root and
+ * quotient in place of rsqrtf, and with this order for the sum of squares (the
+ * reference's, :1966-1992, follows its block size): the row is cut into chunks of
+ * four floats (the last one zero-padded); partial t of 256 adds, in ascending order,
+ * fmaf(w,w, fmaf(z,z, fmaf(y,y, x*x))) of chunks t, t+256, ...; the partials are added
+ * as a balanced binary tree, neighbours first.  batch rows, stride_x / stride_out
+ * floats apart. */
+int q8o_rms_norm(const float *x, const float *weight, float *out, uint32_t batch, uint32_t n,
+                 uint32_t stride_x_row, uint32_t stride_out_row, float eps);
 
 /* ---- activation quantizers ----------------------------------------------- */
 /* src/mmvq_q8.cu:82-112, 623-640.  y: batch * (cols/32) blocks of 36 B. */

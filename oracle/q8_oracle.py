@@ -51,6 +51,7 @@ def lib():
             "q8o_quantize_q8_0": (i32, [f32p, u64, u64, u8p]),
             "q8o_repack_split_plane": (i32, [u8p, u64, u64, u8p]),
             "q8o_get_row": (i32, [u8p, u64, u64, f32p]),
+            "q8o_rms_norm": (i32, [f32p, f32p, f32p, u32, u32, u32, u32, C.c_float]),
             "q8o_quantize_q8_1": (i32, [f32p, u32, u32, u32, u8p]),
             "q8o_quantize_q8_1_d4": (i32, [f32p, u32, u32, u32, u8p]),
             "q8o_block_dot": (C.c_int32, [u8p, u8p, i32, u32, u32, u32, u32, u32]),
@@ -145,6 +146,21 @@ def make_weight(w):
 
 
 # ---- activations ----------------------------------------------------------
+def rms_norm(x, weight, eps, cols=None, stride=None):
+    """Rows of x ([batch, stride] fp32) normalised over their first `cols` columns."""
+    x = _c(np.atleast_2d(x), np.float32)
+    weight = _c(weight, np.float32)
+    batch = x.shape[0]
+    stride = x.shape[1] if stride is None else stride
+    cols = x.shape[1] if cols is None else cols
+    out = np.zeros((batch, cols), np.float32)
+    rc = lib().q8o_rms_norm(_p(x, C.c_float), _p(weight, C.c_float), _p(out, C.c_float), batch, cols, stride,
+                            cols, float(eps))
+    if rc != 0:
+        raise ValueError("q8o_rms_norm rejected the shape")
+    return out
+
+
 def quantize_q8_1(x, cols=None, stride=None):
     x = _c(x, np.float32)
     batch = x.shape[0]
