@@ -113,6 +113,35 @@ class DecodeStep:
         ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, m, FFN, FFN, stream), "quantize")
         ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, m, HIDDEN, stream), "down")
 
+    def run_with_norms(self, layer, one_launch, stream=None):
+        """The same four GEMVs at M=1 preceded by the layer's two RMS norms: inside the fan-out and
+        SwiGLU launches (4 launches), or as two launches of their own (6)."""
+        L, w, ok = self.L, layer.w, self.ok
+        if not hasattr(self, "norm_w"):
+            import numpy as np
+            from q8mi import hip
+            self.norm_w = hip.to_device(np.ones(HIDDEN, np.float32))
+            self.h_in = hip.to_device(np.linspace(-2.0, 2.0, HIDDEN, dtype=np.float32))
+        eps = 1e-6
+        if one_launch:
+            ok(L.q8mi_nqgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.h_in.ptr, self.norm_w.ptr, eps,
+                                     self.x.ptr, self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
+                                     HIDDEN, 1, stream), "nqfanout4")
+        else:
+            ok(L.q8mi_rms_norm(self.h_in.ptr, self.norm_w.ptr, self.x.ptr, 1, HIDDEN, HIDDEN, HIDDEN, eps, stream), "norm")
+            ok(L.q8mi_qgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.x.ptr, HIDDEN,
+                                    self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
+                                    HIDDEN, 1, QDIM, KVDIM, KVDIM, 0, stream), "qfanout4")
+        ok(L.q8mi_qgemv_add(w["o"].ptr, self.attn.ptr, ATTN_OUT, self.h.ptr, 0, HIDDEN, ATTN_OUT, 1, HIDDEN, stream), "qo")
+        if one_launch:
+            ok(L.q8mi_nqgemv_silu_mul(w["gate"].ptr, w["up"].ptr, self.h_in.ptr, self.norm_w.ptr, eps, self.x.ptr,
+                                      self.ffn.ptr, FFN, HIDDEN, 1, stream), "nqsilu_mul")
+        else:
+            ok(L.q8mi_rms_norm(self.h_in.ptr, self.norm_w.ptr, self.x.ptr, 1, HIDDEN, HIDDEN, HIDDEN, eps, stream), "norm")
+            ok(L.q8mi_qgemv_silu_mul(w["gate"].ptr, w["up"].ptr, self.x.ptr, HIDDEN, self.ffn.ptr, FFN, HIDDEN, 1, FFN,
+                                     stream), "qsilu_mul")
+        ok(L.q8mi_qgemv_add(w["down"].ptr, self.ffn.ptr, FFN, self.h.ptr, 0, HIDDEN, FFN, 1, HIDDEN, stream), "qdown")
+
     def run_silu(self, layer, stream=None):
         if self.fused:
             self.ok(self.L.q8mi_qgemv_silu_mul(layer.w["gate"].ptr, layer.w["up"].ptr, self.x.ptr, HIDDEN,
@@ -419,6 +448,12 @@ def main():
             t = time_loop(hip, lambda i: st.run(layers[i % len(layers)]), max(args.steps // 2, 20), 5)
             sweep[f"m{m}"] = {"ms_per_step": round(t, 5), "gbps": round(b / (t * 1e-3) / 1e9, 1)}
         result["gemv_layer_gbps_by_m"] = sweep
+        # the layer's two RMS norms in front of the fan-out and the SwiGLU: inside those launches, or on their own
+        norms = {}
+        for name, one in (("norms_inside_the_gemv_4_launches", True), ("norms_as_2_more_launches", False)):
+            t = time_loop(hip, lambda i: step.run_with_norms(layers[i % len(layers)], one), max(args.steps // 2, 20), 5)
+            norms[name] = {"ms_per_step": round(t, 5), "gbps": round(step_bytes / (t * 1e-3) / 1e9, 1)}
+        result["layer_with_rms_norms_m1"] = norms
     for l in layers[1:]:
         for b in l.w.values():
             b.free()

@@ -12,6 +12,10 @@
 //     (the reference pairs only same-shape neighbours, :11261-11290).
 //   * batch-1 ops on rows of at most 8192 columns run as one launch that quantizes the
 //     activations inside the GEMV; the outputs are the same bits as the two-step form.
+//   * rms_norm sums the squares in a fixed order and takes an IEEE root (the reference's order
+//     follows its block size and its root is rsqrtf); rms_norm_q8_0_matmul_fanout fuses the norm
+//     into the quantizer (batch <= 8) or into the GEMV itself (batch 1) for Q8_0 weights, where
+//     the reference runs rms_norm_batch and q8_0_matmul_fanout one after the other.
 //   * strided batch > 8 (in_stride != cols or out_stride != rows), which the
 //     reference serves with a legacy kernel outside this path, runs as GEMV
 //     slices of eight rows.
@@ -131,6 +135,20 @@ std::unique_ptr<DeviceTensor> HipQ8Backend::tensor_f32(uint64_t count, const cha
 
 std::unique_ptr<DeviceTensor> HipQ8Backend::tensor_bf16(uint64_t count, const char *) {
     return make_tensor(count, 2, DeviceTensorDType::BF16);
+}
+
+std::unique_ptr<DeviceWeight> HipQ8Backend::weight_f32(const float *data, uint64_t count, const char *) {
+    auto w = std::make_unique<HipWeight>();
+    w->rows = 1;
+    w->cols = count;
+    w->format = DeviceWeightFormat::F32;
+    w->bytes = count * 4;
+    if (hipMalloc(reinterpret_cast<void **>(&w->ptr), w->bytes ? w->bytes : 1) != hipSuccess ||
+        hipMemcpy(w->ptr, data, w->bytes, hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return w;
 }
 
 // src/kernels_cuda.cu:1566-1594, 10158-10160: repack on the host, one upload
@@ -389,6 +407,96 @@ DeviceStatus HipQ8Backend::q8_0_matmul_fanout(DeviceTensor *const *outs, const D
             return failed("mmvq_q8_0_fanout4_batch");
     }
     return launch_status("hip q8_0_matmul_fanout");
+}
+
+// ---- RMS norm ------------------------------------------------------------------------------
+// src/kernels_cuda.cu:14748-14779
+DeviceStatus HipQ8Backend::rms_norm(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight, float eps) {
+    return rms_norm_batch(out, x, weight, 1, static_cast<uint32_t>(T(x).count), eps);
+}
+
+// src/kernels_cuda.cu:14781-14816
+DeviceStatus HipQ8Backend::rms_norm_batch(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight,
+                                          uint32_t batch, uint32_t n, float eps) {
+    if (batch == 0) return {};
+    const auto &w = W(weight);
+    if (T(out).is_bf16()) return {false, "hip rms_norm_batch BF16 output is not implemented"};
+    if (T(x).is_bf16()) return {false, "hip rms_norm_batch BF16 input is outside the Q8_0 path"};
+    if (w.format != DeviceWeightFormat::F32 || w.cols < n) return {false, "rms_norm_batch: norm weight is not fp32 [n]"};
+    if (T(x).count < static_cast<uint64_t>(batch) * n || T(out).count < static_cast<uint64_t>(batch) * n)
+        return {false, "rms_norm_batch: tensor smaller than batch * n"};
+    if (q8mi_rms_norm(T(x).f32(), reinterpret_cast<const float *>(w.ptr), T(out).f32(), batch, n, n, n, eps,
+                      stream_) != Q8MI_OK)
+        return failed("rms_norm");
+    return launch_status("hip rms_norm_batch");
+}
+
+// include/qw3/device_backend.hpp:421-444
+DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized, DeviceTensor *const *outs,
+                                                       const DeviceWeight *const *weights, const uint32_t *out_strides,
+                                                       uint32_t fanout, const DeviceTensor &x,
+                                                       const DeviceWeight &norm_weight, uint32_t batch,
+                                                       uint32_t in_stride, float eps) {
+    if (fanout == 0 || batch == 0) return {};
+    const auto &nw = W(norm_weight);
+    const uint32_t cols = in_stride;
+    bool fast = batch <= 8 && cols % 32 == 0 && !T(x).is_bf16() && !T(normalized).is_bf16() &&
+                nw.format == DeviceWeightFormat::F32 && nw.cols == cols &&
+                T(x).count >= static_cast<uint64_t>(batch) * cols &&
+                T(normalized).count >= static_cast<uint64_t>(batch) * cols;
+    for (uint32_t i = 0; i < fanout && fast; ++i) {
+        const auto &w = W(*weights[i]);
+        fast = w.format == DeviceWeightFormat::Q8_0 && w.cols == cols && !T(*outs[i]).is_bf16() &&
+               out_strides[i] >= w.rows && T(*outs[i]).count >= static_cast<uint64_t>(batch) * out_strides[i];
+    }
+    if (!fast) {   // base-class behaviour
+        if (auto st = rms_norm_batch(normalized, x, norm_weight, batch, in_stride, eps); !st.ok) return st;
+        return q8_0_matmul_fanout(outs, weights, out_strides, fanout, normalized, batch, in_stride);
+    }
+    const float *xin = T(x).f32();
+    const float *nwp = reinterpret_cast<const float *>(nw.ptr);
+    float *nrm = T(normalized).f32();
+    auto group = [&](uint32_t i0, const uint8_t *(&wp)[4], float *(&op)[4], uint32_t (&r)[4], uint32_t (&s)[4]) {
+        for (uint32_t k = 0; k < 4; ++k) { wp[k] = nullptr; op[k] = nullptr; r[k] = 0; s[k] = 0; }
+        for (uint32_t i = i0; i < fanout && i < i0 + 4; ++i) {
+            wp[i - i0] = W(*weights[i]).ptr;
+            op[i - i0] = T(*outs[i]).f32();
+            r[i - i0] = static_cast<uint32_t>(W(*weights[i]).rows);
+            s[i - i0] = out_strides[i];
+        }
+    };
+    const uint8_t *wp[4];
+    float *op[4];
+    uint32_t r[4], s[4];
+    uint32_t first = 0;
+    bool quantized = false;
+    if (batch == 1) {   // the first four weights: norm + quantizer inside the GEMV, which also leaves `normalized`
+        group(0, wp, op, r, s);
+        const int rc = q8mi_nqgemv_fanout4(wp[0], wp[1], wp[2], wp[3], xin, nwp, eps, nrm, op[0], op[1], op[2], op[3],
+                                           r[0], r[1], r[2], r[3], cols, 1, stream_);
+        if (rc == Q8MI_OK) first = 4;
+        else if (rc != Q8MI_REJECTED) return failed("nqgemv_fanout4");
+    }
+    if (first == 0) {
+        if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(batch, cols), "q8_1 scratch alloc"); !st.ok) return st;
+        if (q8mi_rms_norm_quantize_q8_1(xin, nwp, nrm, q8_1_.ptr, batch, cols, cols, cols, eps, stream_) != Q8MI_OK)
+            return failed("rms_norm_quantize_q8_1");
+        quantized = true;
+    }
+    for (uint32_t i0 = first; i0 < fanout; i0 += 4) {
+        group(i0, wp, op, r, s);
+        if (!quantized) {   // batch 1, weights beyond the fourth: quantize `normalized` inside the GEMV
+            if (q8mi_qgemv_fanout4(wp[0], wp[1], wp[2], wp[3], nrm, cols, op[0], op[1], op[2], op[3], r[0], r[1], r[2],
+                                   r[3], cols, 1, s[0], s[1], s[2], s[3], stream_) != Q8MI_OK)
+                return failed("qgemv_fanout4");
+            continue;
+        }
+        if (!ported::launch_mmvq_q8_0_fanout4_batch(wp[0], wp[1], wp[2], wp[3], q8_1_.ptr, op[0], op[1], op[2], op[3],
+                                                    r[0], r[1], r[2], r[3], cols, batch, s[0], s[1], s[2], s[3],
+                                                    stream_))
+            return failed("mmvq_q8_0_fanout4_batch");
+    }
+    return launch_status("hip rms_norm_q8_0_matmul_fanout");
 }
 
 // src/kernels_cuda.cu:11919-11957: in-place residual add for batch <= 8, else matmul + add

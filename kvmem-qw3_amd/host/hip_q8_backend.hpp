@@ -11,7 +11,9 @@
 //   q8_0_matmul_add (:529), argmax (:2456), argmax_buffer / argmax_to_buffer /
 //   copy_argmax_buffer_to_host (:2458-2473), argmax_batch (:2477),
 //   argmax_launch / argmax_collect (:2503-2509), begin/end_capture, replay_graph
-//   (:120-122), plus the handful of tensor calls a test needs.
+//   (:120-122), weight_f32 (:214), rms_norm / rms_norm_batch (:624-638) and
+//   rms_norm_q8_0_matmul_fanout with its recurrent / attention twins (:421-523),
+//   plus the handful of tensor calls a test needs.
 // Routing follows the reference's CUDA backend (src/kernels_cuda.cu:10764-12630,
 // 14559-14658) except where noted in the .cpp; one op is new: lm_head_verify.
 //
@@ -83,6 +85,8 @@ public:
     // tensors / weights
     std::unique_ptr<DeviceTensor> tensor_f32(uint64_t count, const char *label);
     std::unique_ptr<DeviceTensor> tensor_bf16(uint64_t count, const char *label);
+    // fp32 vector (norm weights): rows = 1, cols = count (src/kernels_cuda.cu: weight_f32)
+    std::unique_ptr<DeviceWeight> weight_f32(const float *data, uint64_t count, const char *label);
     // `data`: interleaved GGUF Q8_0 blocks (34 B); stored split-plane on the device
     std::unique_ptr<DeviceWeight> weight_q8_0(const void *data, uint64_t rows, uint64_t cols, const char *label);
     DeviceStatus copy_bytes_from_host(DeviceTensor &x, uint64_t byte_offset, const void *host, uint64_t bytes);
@@ -110,6 +114,37 @@ public:
     DeviceStatus q8_0_matmul_silu_mul(DeviceTensor &out, const DeviceWeight &weight_gate,
                                       const DeviceWeight &weight_up, const DeviceTensor &x, uint32_t batch,
                                       uint32_t in_stride, uint32_t out_stride);
+
+    // RMS norm in front of the projections.  rms_norm normalises the whole tensor as one row
+    // (src/kernels_cuda.cu:14748-14779), rms_norm_batch `batch` dense rows of n (:14781-14816).
+    DeviceStatus rms_norm(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight, float eps);
+    DeviceStatus rms_norm_batch(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight, uint32_t batch,
+                                uint32_t n, float eps);
+    // norm, then several projections of the normalised rows (include/qw3/device_backend.hpp:421-444;
+    // the reference's CUDA override fuses FP8 weights only and runs the two steps for Q8_0,
+    // src/kernels_cuda.cu:11615-11658).  Here a batch of one row is one launch (norm and quantizer
+    // inside the fan-out GEMV), up to eight rows are a fused norm + quantizer and one GEMV launch per
+    // four weights; `normalized` receives the fp32 rows either way.
+    DeviceStatus rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized, DeviceTensor *const *outs,
+                                             const DeviceWeight *const *weights, const uint32_t *out_strides,
+                                             uint32_t fanout, const DeviceTensor &x, const DeviceWeight &norm_weight,
+                                             uint32_t batch, uint32_t in_stride, float eps);
+    DeviceStatus rms_norm_q8_0_matmul_recurrent_fanout(DeviceTensor &normalized, DeviceTensor *const *outs,
+                                                       const DeviceWeight *const *weights, const uint32_t *out_strides,
+                                                       uint32_t fanout, const DeviceTensor &x,
+                                                       const DeviceWeight &norm_weight, uint32_t batch,
+                                                       uint32_t in_stride, float eps) {
+        return rms_norm_q8_0_matmul_fanout(normalized, outs, weights, out_strides, fanout, x, norm_weight, batch,
+                                           in_stride, eps);
+    }
+    DeviceStatus rms_norm_q8_0_matmul_attention_fanout(DeviceTensor &normalized, DeviceTensor *const *outs,
+                                                       const DeviceWeight *const *weights, const uint32_t *out_strides,
+                                                       uint32_t fanout, const DeviceTensor &x,
+                                                       const DeviceWeight &norm_weight, uint32_t batch,
+                                                       uint32_t in_stride, float eps) {
+        return rms_norm_q8_0_matmul_fanout(normalized, outs, weights, out_strides, fanout, x, norm_weight, batch,
+                                           in_stride, eps);
+    }
 
     // argmax
     DeviceArgmax argmax(const DeviceTensor &x);

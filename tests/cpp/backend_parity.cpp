@@ -581,6 +581,82 @@ void case_lm_head_verify(qw3::HipQ8Backend &b) {
 
 // A captured decode-style sequence replayed several times with eager work and
 // synchronizations in between; every replay must equal the eager result bit for bit.
+// rms_norm, rms_norm_batch and rms_norm_q8_0_matmul_fanout at batch 1 (one launch), 3 (fused
+// norm + quantizer) and 20 (the two-step base behaviour), with five weights so that a second
+// group of the fan-out runs too.  The normalised rows must be the oracle's bits.
+void case_rms_norm(qw3::HipQ8Backend &b) {
+    const uint32_t cols = 2048;
+    const float eps = 1e-6f;
+    const uint32_t heights[5] = {768, 130, 31, 256, 64};
+    std::vector<HostWeight> hw;
+    std::vector<std::unique_ptr<qw3::DeviceWeight>> dw;
+    for (int i = 0; i < 5; ++i) {
+        hw.push_back(make_weight(heights[i], cols, 300 + i));
+        dw.push_back(b.weight_q8_0(hw.back().gguf.data(), heights[i], cols, "w"));
+    }
+    auto nwv = normal_vec(cols, 310, 0.5f);
+    for (auto &f : nwv) f += 1.0f;
+    auto nw = b.weight_f32(nwv.data(), cols, "norm.weight");
+    std::string d;
+    for (uint32_t batch : {1u, 3u, 20u}) {
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 320 + batch, 3.0f);
+        auto dx = upload_f32(b, x);
+        std::vector<float> nref(x.size());
+        q8o_rms_norm(x.data(), nwv.data(), nref.data(), batch, cols, cols, cols, eps);
+
+        auto plain = b.tensor_f32(x.size(), "plain");
+        bool ok = batch == 1 ? require(b.rms_norm(*plain, *dx, *nw, eps), "rms_norm")
+                             : require(b.rms_norm_batch(*plain, *dx, *nw, batch, cols, eps), "rms_norm_batch");
+        ok = ok && std::memcmp(download_f32(b, *plain).data(), nref.data(), nref.size() * 4) == 0;
+        report(("rms_norm_bits_batch" + std::to_string(batch)).c_str(), ok);
+
+        auto normalized = b.tensor_f32(x.size(), "normalized");
+        std::vector<std::unique_ptr<qw3::DeviceTensor>> outs;
+        qw3::DeviceTensor *op[5];
+        const qw3::DeviceWeight *wp[5];
+        uint32_t strides[5];
+        for (int i = 0; i < 5; ++i) {
+            strides[i] = heights[i] + (batch > 1 ? 8 : 0);
+            outs.push_back(b.tensor_f32(static_cast<size_t>(batch) * strides[i], "o"));
+            op[i] = outs.back().get();
+            wp[i] = dw[i].get();
+        }
+        ok = require(b.rms_norm_q8_0_matmul_fanout(*normalized, op, wp, strides, 5, *dx, *nw, batch, cols, eps), "fanout");
+        ok = ok && std::memcmp(download_f32(b, *normalized).data(), nref.data(), nref.size() * 4) == 0;
+        if (!ok && d.empty()) d = "normalized rows differ from the oracle";
+        for (int i = 0; i < 5 && ok; ++i) {
+            std::vector<float> ref, mag;
+            if (batch <= 8) {
+                oracle_linear(hw[i], nref.data(), batch, cols, strides[i], ref, mag);
+                ok = close_fp32(download_f32(b, *op[i]), ref, mag, batch, heights[i], strides[i], d);
+            } else {   // above 8 rows the matmul route quantizes to D4 blocks where the shape allows
+                auto two = b.tensor_f32(static_cast<size_t>(batch) * strides[i], "two");
+                ok = require(b.q8_0_matmul(*two, *dw[i], *plain, batch, cols, strides[i]), "matmul");
+                const auto a = download_f32(b, *op[i]), c = download_f32(b, *two);
+                for (uint32_t j = 0; j < batch && ok; ++j)
+                    ok = std::memcmp(&a[static_cast<size_t>(j) * strides[i]], &c[static_cast<size_t>(j) * strides[i]],
+                                     heights[i] * 4) == 0;
+                if (!ok) d = "differs from rms_norm_batch + q8_0_matmul";
+            }
+        }
+        report(("rms_norm_q8_0_matmul_fanout_batch" + std::to_string(batch)).c_str(), ok, d);
+    }
+    // the twins forward to the same operator
+    {
+        const auto x = normal_vec(cols, 399, 2.0f);
+        auto dx = upload_f32(b, x);
+        auto n1 = b.tensor_f32(cols, "n1"), n2 = b.tensor_f32(cols, "n2");
+        auto o1 = b.tensor_f32(heights[0], "o1"), o2 = b.tensor_f32(heights[0], "o2");
+        qw3::DeviceTensor *p1[1] = {o1.get()}, *p2[1] = {o2.get()};
+        const qw3::DeviceWeight *wp[1] = {dw[0].get()};
+        const uint32_t st[1] = {heights[0]};
+        bool ok = require(b.rms_norm_q8_0_matmul_attention_fanout(*n1, p1, wp, st, 1, *dx, *nw, 1, cols, eps), "attention") &&
+                  require(b.rms_norm_q8_0_matmul_recurrent_fanout(*n2, p2, wp, st, 1, *dx, *nw, 1, cols, eps), "recurrent");
+        ok = ok && download_f32(b, *o1) == download_f32(b, *o2) && download_f32(b, *n1) == download_f32(b, *n2);
+        report("rms_norm_fanout_twins", ok);
+    }
+}
+
 void case_graph_replay(qw3::HipQ8Backend &b) {
     const uint32_t hidden = 1024, ffn = 3072;
     const HostWeight wg = make_weight(ffn, hidden, 91), wu = make_weight(ffn, hidden, 92), wd = make_weight(hidden, ffn, 93);
@@ -629,7 +705,7 @@ int main(int argc, char **argv) {
     struct Case { const char *name; void (*fn)(qw3::HipQ8Backend &); };
     const Case cases[] = {
         {"closed_form", case_closed_form}, {"matvec", case_matvec_family}, {"matmul", case_matmul},
-        {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"gguf", case_gguf}, {"lm_head", case_lm_head_verify}, {"graph", case_graph_replay},
+        {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"gguf", case_gguf}, {"lm_head", case_lm_head_verify}, {"rms_norm", case_rms_norm}, {"graph", case_graph_replay},
     };
     for (const auto &c : cases) {
         if (!only.empty() && only != c.name) continue;

@@ -8,7 +8,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DRIVER = os.path.join(ROOT, "tests", "cpp", "backend_parity")
 
-CASES = ["closed_form", "matvec", "matmul", "argmax", "get_rows", "gguf", "lm_head", "graph"]
+CASES = ["closed_form", "matvec", "matmul", "argmax", "get_rows", "gguf", "lm_head", "rms_norm", "graph"]
 
 
 @pytest.mark.gpu
