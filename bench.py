@@ -382,6 +382,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
     ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", choices=["gemm", "lm_head"], help="one secondary figure alone (for profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's throughput; run with --gpus 1 "
@@ -394,6 +395,12 @@ def main():
     hip.set_device(0)
     q8mi.lib()
 
+    if args.only == "gemm":
+        print(json.dumps({"gemm_int8": bench_gemm(q8mi, hip, synth, reps=max(args.steps // 20, 3))}))
+        return
+    if args.only == "lm_head":
+        print(json.dumps({"lm_head_fused": bench_lm_head(q8mi, hip, synth)}))
+        return
     counter_calibration(q8mi, hip)
     layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
     step = DecodeStep(q8mi, hip, m=1)
