@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import q8mi
-from gpu_common import NULL, dev, quantize_q8_1
+from gpu_common import NULL, assert_close_fp32, dev, quantize_q8_1
 from q8mi import hip, ok, synth
 
 pytestmark = pytest.mark.gpu
@@ -174,3 +174,52 @@ def test_lm_head_rejections(gpu):
     assert L.q8mi_lm_head_argmax_accept(*args(100, 512, 0)) == q8mi.REJECTED
     assert L.q8mi_lm_head_argmax_accept(*args(100, 512, 9)) == q8mi.REJECTED
     assert L.q8mi_lm_head_argmax_accept(*args(0, 512, 2)) == q8mi.REJECTED
+
+
+# ---- the real LM head: 248 320 tokens x 5120 columns (1.35 GB of weights) ------------------------
+FULL_VOCAB, FULL_COLS = 248320, 5120
+
+
+@pytest.fixture(scope="module")
+def full_head(gpu):
+    w = synth.q8_0_weight(FULL_VOCAB, FULL_COLS, seed=4242)
+    return w, dev(w)
+
+
+@pytest.mark.parametrize("batch", [1, 2, 4, 6, 8])
+def test_lm_head_full_vocabulary(gpu, oracle, full_head, batch):
+    """At the model's size the oracle does not run the whole head in seconds, so: (1) the plain GEMV's
+    logits are held against the oracle on a seeded sample of rows plus every winning row, (2) the
+    oracle's argmax of those logits is the expected token of each verify row, (3) the fused head must
+    return those tokens and the accept length of every forced-match prefix."""
+    L = gpu.lib()
+    w, dw = full_head
+    x = synth.normal(batch, FULL_COLS, seed=700 + batch)
+    dy, y = quantize_q8_1(x)
+    logits_dev = hip.DeviceBuffer(4 * batch * FULL_VOCAB)
+    ok(L.q8mi_gemv(dw.ptr, dy.ptr, logits_dev.ptr, FULL_VOCAB, FULL_COLS, batch, FULL_VOCAB, NULL), "gemv")
+    hip.synchronize()
+    logits = logits_dev.download(np.float32).reshape(batch, FULL_VOCAB)
+    ref_pairs = oracle.argmax_rows_scan(logits, batch, FULL_VOCAB)
+    tokens = ref_pairs["index"]
+    rng = np.random.default_rng(batch)
+    sample = np.unique(np.concatenate([rng.integers(0, FULL_VOCAB, 3000), tokens, [0, FULL_VOCAB - 1]]))
+    sub = np.ascontiguousarray(w[sample])
+    rc, ref = oracle.gemv(sub, y, sample.size, FULL_COLS, batch, threads=8)
+    rc, absum = oracle.gemv_abs(sub, y, sample.size, FULL_COLS, batch)
+    assert_close_fp32(logits[:, sample], ref, absum, "LM-head logits on sampled rows")
+    # top-2 gaps of this seed are far above the fp32 tolerance, so the tokens are unambiguous
+    top2 = np.partition(logits, -2, axis=1)[:, -2:]
+    assert np.all(top2[:, 1] - top2[:, 0] > 1e-4 * np.abs(top2[:, 1]))
+    for prefix in sorted({0, batch // 2, batch - 1}):
+        drafts = rng.integers(0, FULL_VOCAB, batch - 1).astype(np.int32)
+        drafts[:prefix] = tokens[:prefix]
+        if prefix < batch - 1 and drafts[prefix] == tokens[prefix]:
+            drafts[prefix] = (drafts[prefix] + 1) % FULL_VOCAB
+        exp_len, exp_next = oracle.accept(tokens, drafts, eos=2)
+        assert exp_len == prefix
+        pairs, n_acc, nxt, _ = run_lm_head(dw, dy, FULL_VOCAB, FULL_COLS, batch, drafts, 2, on_device=(prefix % 2 == 1))
+        assert np.array_equal(pairs["index"], tokens), "row argmax tokens differ"
+        assert n_acc == exp_len and nxt == exp_next
+        want = logits[np.arange(batch), tokens]
+        assert np.all(np.abs(pairs["value"] - want) <= 1e-5 * np.abs(want) + 1e-6)
