@@ -242,8 +242,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_kernel(
 
 // ---- direct-to-LDS variant (rows whose int8 plane is 16-byte aligned) ----------------------
 // Workgroup tile: 32*RB weight rows x 128 activation rows; RB = 4 is the main tile, RB = 1 a
-// quarter tile used for the rows left over after the last full round of main tiles (and for
-// problems too small to fill the chip with main tiles).
+// quarter tile with the same two stages (what problems too small to fill the chip with main tiles
+// used before the ring-staged tiles below; selectable for comparison).
 // Stage layout (two stages; TR = 32*RB):
 //   weight quants      TR rows x 128 B; 16-byte piece p of row r sits in slot p ^ swz(r), so equal
 //                      pieces of 8 or 16 consecutive rows fall on distinct banks
@@ -459,6 +459,217 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
     }
 }
 
+// ---- medium batches: 32-row tiles behind a ring of LDS stages ---------------------------------
+// A batch of 33..a few hundred rows gives each CU only a few hundred MFMAs per launch: one K-step
+// of a narrow tile is a few hundred cycles of arithmetic, far less than the time its operands
+// take to arrive, so with two stages every K-step costs a memory latency (what the quarter tile
+// above does: ~1 us per step).  Here the tile is 32 weight rows x (32 * CB) activation rows and
+// the K-steps (one 128-element super-block each) run through a ring of NS stages: NS - 1 steps
+// are in flight while one is consumed, loads are awaited by count (vmcnt), oldest first, and one
+// barrier per step publishes it.  Everything travels global -> LDS directly in whole 128-byte
+// lines (per-lane strided loads of the operands were measured 2-3 x slower), the scales included:
+// the fp16 weight scales raw (converted by their readers), the activation scales as one 4-byte
+// transfer per lane that lays the 32 scales of a (group, block) out contiguously.  The pieces of a
+// step are dealt round-robin to the W waves, every wave issuing the same number of loads (the
+// remainder repeats the last piece) so that the wait counts are compile-time constants.
+// The waves split the tile by activation group first (CB groups of 32 rows) and by K second:
+// S = W / CB waves share an output patch, each taking 4 / S of the four blocks of every step; their
+// partial sums are added through LDS at the end as a balanced tree (deterministic).
+template <int CB, int W>
+struct RingTile {
+    static constexpr int kCols = 32 * CB;
+    static constexpr int kShares = W / CB;                             // waves per output patch (K split)
+    static constexpr int kYChunks = (kCols * kRec + 1023) / 1024;     // 1 KB pieces of the activation records
+    static constexpr int kDyItems = CB * 2;                            // 64 lanes fill two 32-float slots
+    static constexpr int kItems = 4 + kYChunks + kDyItems + 1;         // weight pieces, records, scales, weight scales
+    static constexpr int kLoads = (kItems + W - 1) / W;                // load instructions per wave and step
+    static constexpr int kOffYr = 32 * 128;
+    static constexpr int kOffDy = kOffYr + kYChunks * 1024;            // fp32 activation scales, [group][block][32]
+    static constexpr int kOffWsc = kOffDy + CB * 4 * 128;              // raw fp16 weight scales, [row][4]
+    static constexpr int kStage = kOffWsc + 256;
+    static_assert(W % CB == 0 && 4 % kShares == 0, "a patch is shared by 1, 2 or 4 waves");
+};
+
+// 4 bytes per lane, global -> LDS at lds_off + lane * 4.
+__device__ __forceinline__ void dma4(const uint8_t *uniform_base, uint32_t lane_off, uint32_t lds_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :: "s"(lds_off), "v"(lane_off), "s"(uniform_base) : "memory", "m0");
+}
+
+// Waits until at most `steps` K-steps of this wave's loads are still in flight.
+template <int LOADS, int MAX_STEPS>
+__device__ __forceinline__ void wait_ring(uint32_t steps) {
+    static_assert(LOADS * MAX_STEPS <= 63, "vmcnt holds 6 bits");
+    if constexpr (MAX_STEPS > 0) {
+        if (steps >= static_cast<uint32_t>(MAX_STEPS)) {
+            asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LOADS * MAX_STEPS) : "memory");
+            return;
+        }
+        wait_ring<LOADS, MAX_STEPS - 1>(steps);
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+}
+
+template <int CB, int W, int NS>
+__global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles) {
+    using T = RingTile<CB, W>;
+    constexpr uint32_t S = T::kShares;
+    extern __shared__ __align__(16) uint8_t smem[];
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
+    const uint32_t grp = wave % CB, share = wave / CB;   // activation group, K share
+    const uint32_t id = blockIdx.x, xcd = id % 8u, seq = id / 8u;
+    const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
+    if (rt >= row_tiles) return;   // uniform for the workgroup
+    const uint32_t row0 = rt * 32u, col0 = ct * T::kCols;
+    const uint32_t nsb = nb / 4;
+    const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+
+    // The pieces of a step this wave loads: kind and LDS position are wave-uniform, the per-lane
+    // source offsets do not change over the K loop.  Weight rows past the end re-read the last row,
+    // activation rows past the end of the batch the last activation row (never stored).
+    auto clamp_row = [&](uint32_t r) { return row0 + r < rows ? r : rows - 1 - row0; };
+    uint32_t lane_off[T::kLoads];
+#pragma unroll
+    for (int i = 0; i < T::kLoads; ++i) {
+        uint32_t item = wave + W * i;
+        item = item < T::kItems ? item : T::kItems - 1;
+        if (item < 4) {                                   // 8 weight rows x 128 B
+            const uint32_t r = item * 8 + lane / 8;
+            lane_off[i] = clamp_row(r) * static_cast<uint32_t>(row_bytes) + ((lane & 7u) ^ swz(r)) * 16;
+        } else if (item < 4 + T::kYChunks) {              // 1 KB of activation records
+            lane_off[i] = (item - 4) * 1024 + lane * 16;
+        } else if (item < 4 + T::kYChunks + T::kDyItems) {   // the scales of two (group, block) pairs
+            const uint32_t sl = (item - 4 - T::kYChunks) * 2 + lhalf;
+            uint32_t j = col0 + (sl / 4) * 32 + l32;
+            j = j < batch ? j : batch - 1;
+            lane_off[i] = (j - col0) * kRec + (sl % 4) * 4;
+        } else {                                          // fp16 weight scales: 32 rows x 8 B
+            lane_off[i] = clamp_row(lane / 2) * static_cast<uint32_t>(row_bytes) + (lane & 1u) * 4;
+        }
+    }
+    const uint8_t *wd_base0 = uniform_ptr(w + row0 * row_bytes);
+    const uint8_t *y_base0 = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec);
+    const uint64_t y_step = static_cast<uint64_t>(batch) * kRec;
+    const uint64_t y_room0 = static_cast<uint64_t>(nsb) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
+    const uint32_t smem_off = lds_offset_of(smem);
+
+    auto issue = [&](uint32_t step) {
+        const uint32_t stage_off = smem_off + (step % NS) * T::kStage;
+        const uint8_t *wd_base = wd_base0 + static_cast<uint64_t>(step) * 8;
+        const uint8_t *wq_base = wd_base0 + 2 * nb + static_cast<uint64_t>(step) * 128;
+        const uint8_t *y_base = y_base0 + step * y_step;
+        const uint64_t room = y_room0 - step * y_step;
+        const uint32_t y_limit = static_cast<uint32_t>(room < 0xffffffffull ? room : 0xffffffffull);
+#pragma unroll
+        for (int i = 0; i < T::kLoads; ++i) {
+            uint32_t item = wave + W * i;
+            item = item < T::kItems ? item : T::kItems - 1;
+            if (item < 4) {
+                dma16(wq_base, lane_off[i], stage_off + item * 1024);
+            } else if (item < 4 + T::kYChunks) {
+                const uint32_t off = lane_off[i] <= y_limit ? lane_off[i] : y_limit;   // never past the buffer
+                dma16(y_base, off, stage_off + T::kOffYr + (item - 4) * 1024);
+            } else if (item < 4 + T::kYChunks + T::kDyItems) {
+                dma4(y_base, lane_off[i], stage_off + T::kOffDy + (item - 4 - T::kYChunks) * 256);
+            } else {
+                dma4(wd_base, lane_off[i], stage_off + T::kOffWsc);
+            }
+        }
+    };
+
+    v16i seed;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) seed[i] = static_cast<int>(kMagicBits);
+    asm volatile("" : "+v"(seed));
+    float acc[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+
+    const uint32_t ahead = nsb < NS - 1 ? nsb : NS - 1;
+    for (uint32_t s = 0; s < ahead; ++s) issue(s);
+    wait_ring<T::kLoads, NS - 2>(ahead - 1);
+    __syncthreads();
+
+    const uint32_t fl = swz(l32);
+    const uint32_t a_off = T::kOffYr + (grp * 32 + l32) * kRec + 16 + lhalf * 16;
+    const uint32_t dy_off = T::kOffDy + grp * 512 + lhalf * 16;
+    for (uint32_t sb = 0; sb < nsb; ++sb) {
+        if (sb + NS - 1 < nsb) issue(sb + NS - 1);   // into the slot consumed one step ago
+        const uint8_t *cur = smem + (sb % NS) * T::kStage;
+#pragma unroll
+        for (uint32_t t = 0; t < 4 / S; ++t) {
+            const uint32_t sub = share * (4 / S) + t;
+            const v4i a = *reinterpret_cast<const v4i *>(cur + a_off + sub * 32);
+            const v4i b = *reinterpret_cast<const v4i *>(cur + l32 * 128 + (((2 * sub + lhalf) ^ fl) * 16));
+            const float dw = half_bits_to_float(*reinterpret_cast<const uint16_t *>(cur + T::kOffWsc + l32 * 8 + sub * 2));
+            float dy[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 q = *reinterpret_cast<const float4 *>(cur + dy_off + sub * 128 + g * 32);
+                dy[4 * g + 0] = q.x; dy[4 * g + 1] = q.y; dy[4 * g + 2] = q.z; dy[4 * g + 3] = q.w;
+            }
+            const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, seed, 0, 0, 0);
+            const float cw = -kMagic * dw;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = fmaf(fmaf(as_f32(r[v]), dw, cw), dy[v], acc[v]);
+        }
+        if (sb + 1 < nsb) {
+            const uint32_t later = nsb - 2 - sb;   // steps issued beyond the next one
+            wait_ring<T::kLoads, NS - 2>(later < NS - 2 ? later : NS - 2);
+        }
+        __syncthreads();
+    }
+
+    // D[i][n]: n = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (activation row of the group)
+    const uint32_t r_out = row0 + l32;
+    auto store = [&](int v, float value) {
+        const uint32_t j = col0 + grp * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
+        if (r_out < rows && j < batch) dst[static_cast<uint64_t>(j) * stride_dst + r_out] = value;
+    };
+    if constexpr (S == 1) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) store(v, acc[v]);
+    } else {
+        // every load has landed and every wave is past its last read of the stages: reuse them
+        float *part = reinterpret_cast<float *>(smem);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) part[(wave * 16 + v) * kWave + lane] = acc[v];
+        __syncthreads();
+        constexpr int kMine = 16 / S;   // outputs of the patch this wave finishes
+#pragma unroll
+        for (int k = 0; k < kMine; ++k) {
+            const int v = share * kMine + k;
+            auto p = [&](uint32_t s) { return part[((s * CB + grp) * 16 + v) * kWave + lane]; };
+            float total;
+            if constexpr (S == 2) total = p(0) + p(1);
+            else total = (p(0) + p(1)) + (p(2) + p(3));
+            store(v, total);
+        }
+    }
+}
+
+// ring depths and waves per workgroup of the medium-batch kernel (compile-time; see the sweep in the design notes)
+#ifndef Q8MI_RING1
+#define Q8MI_RING1 6
+#endif
+#ifndef Q8MI_RING2
+#define Q8MI_RING2 4
+#endif
+#ifndef Q8MI_RING4
+#define Q8MI_RING4 3
+#endif
+#ifndef Q8MI_RINGW2
+#define Q8MI_RINGW2 8
+#endif
+#ifndef Q8MI_RINGW4
+#define Q8MI_RINGW4 8
+#endif
+
 template <bool CHECK, bool A16>
 int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb,
                    uint32_t batch, uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid,
@@ -518,29 +729,63 @@ int launch_dma_rows(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
 // Tile choice.  Workgroups are scheduled dynamically and a lone workgroup on a CU runs nearly
 // twice as fast as two sharing its VALUs, so a partly filled last round of main tiles costs
 // little: problems with at least 0.4 main tiles per resident slot (two per CU) use main tiles
-// throughout; smaller ones use quarter tiles, which put four times as many workgroups on the chip
-// (measured crossover on MI355X: between 160 and 256 main tiles).
-// Q8MI_GEMM_TILE (1 or 4, read only when the process runs with Q8MI_TUNE=1) overrides the choice.
+// throughout (measured crossover on MI355X: between 160 and 256 main tiles); smaller ones use the
+// ring-staged 32-row tiles.
+// Q8MI_GEMM_TILE (4 = main, 1 = two-stage quarter tiles; read only when the process runs with
+// Q8MI_TUNE=1) overrides the choice.
+template <int CB, int W, int NS>
+int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
+                uint32_t stride, hipStream_t stream) {
+    using T = RingTile<CB, W>;
+    constexpr int lds = NS * T::kStage;
+    static_assert(lds >= W * 16 * kWave * 4, "the stages are reused for the partial sums of the waves");
+    static bool granted = false;
+    if (!granted) {
+        if (lds > 64 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", lds);
+        }
+        granted = true;
+    }
+    const uint32_t row_tiles = (rows + 31u) / 32u;
+    const uint32_t col_tiles = (batch + T::kCols - 1) / T::kCols;
+    const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
+    if (grid64 > 0x7fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    gemm_d4_ring_kernel<CB, W, NS><<<static_cast<uint32_t>(grid64), kWave * W, lds, stream>>>(
+        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
+    return check_launch("gemm");
+}
+
 int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
                     uint32_t stride, hipStream_t stream) {
     const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
     const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
     const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
     const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
-    int tile = tiles * 5 >= slots * 2 ? 4 : 1;
+    int tile = tiles * 5 >= slots * 2 ? 4 : 0;
     static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
     if (live) {
-        if (const char *e = getenv("Q8MI_GEMM_TILE")) tile = atoi(e) == 1 ? 1 : 4;
+        if (const char *e = getenv("Q8MI_GEMM_TILE")) tile = atoi(e);
     }
-    return tile == 4 ? launch_dma_rows<4>(w, y, dst, rows, nb, batch, stride, stream)
-                     : launch_dma_rows<1>(w, y, dst, rows, nb, batch, stride, stream);
+    if (tile == 4) return launch_dma_rows<4>(w, y, dst, rows, nb, batch, stride, stream);
+    if (tile == 1) return launch_dma_rows<1>(w, y, dst, rows, nb, batch, stride, stream);   // two-stage quarter tiles
+    // too few main tiles to fill the chip: 32-row tiles behind a ring of stages, as wide as the batch needs
+    if (batch <= 32) return launch_ring<1, 4, Q8MI_RING1>(w, y, dst, rows, nb, batch, stride, stream);
+    if (batch <= 64) return launch_ring<2, Q8MI_RINGW2, Q8MI_RING2>(w, y, dst, rows, nb, batch, stride, stream);
+    // at most one tile per CU: sixteen waves (four K shares per group) instead of eight
+    const uint64_t ring_tiles = static_cast<uint64_t>((rows + 31u) / 32u) * ((batch + 127u) / 128u);
+    if (ring_tiles <= static_cast<uint32_t>(device_cu_count()))
+        return launch_ring<4, 16, Q8MI_RING4>(w, y, dst, rows, nb, batch, stride, stream);
+    return launch_ring<4, Q8MI_RINGW4, Q8MI_RING4>(w, y, dst, rows, nb, batch, stride, stream);
 }
 
 int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,
                    uint32_t batch, uint32_t stride, hipStream_t stream) {
     // small batches: the weight-streaming matrix-core GEMV, which reads the weights at HBM speed
-    // instead of padding the batch to a 128-wide tile (it declines what tiles serve better)
-    if (batch <= 32 && (cols / kQK) % 8 == 0) {
+    // instead of padding the batch to a 32-wide tile (it declines what the ring tiles serve better)
+    if (batch <= 16 && (cols / kQK) % 8 == 0) {
         const int rc = gemv_mfma_d4(w, y, dst, rows, cols, batch, stride, stream);
         if (rc != Q8MI_REJECTED) return rc;
     }

@@ -580,10 +580,12 @@ GemvTuning gemv_tuning() {
 }
 
 // D4-quantized activations through the matrix-core GEMV: what the GEMM entry points use for
-// batches too small for an MFMA tile.  As many activation rows per launch as fit LDS (at most 16);
-// a batch is cut into that many rows at a time, each slice streaming the weights once, for as many
-// passes as measured faster than tiles (two of 16 rows, four of fewer).  Q8MI_REJECTED otherwise
-// (the caller then uses tiles).
+// batches too small for an MFMA tile.  As many activation rows per launch as fit LDS (at most 16:
+// 16 at 5120 columns, 4 at 17408); served while one pass over the weights covers the batch, or two
+// passes of the short slices (measured against the 32-row ring tiles of the GEMM: 14.7..17.2 us
+// against 19 us at 5120 x 5120 and 9..16 rows, but 26..32 us in two passes at 17..32 rows;
+// 49 against 58 us at 5120 x 17408 and 8 rows).  Q8MI_REJECTED otherwise (the caller then uses
+// tiles).
 int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, uint32_t cols, uint32_t batch,
                  uint32_t stride_dst_row, hipStream_t stream) {
     const uint32_t nb = cols / kQK;
@@ -593,7 +595,7 @@ int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, 
     for (uint32_t m = 16; m >= 4; m -= 4) {
         if (mfma_x_lds_bytes(nb, m, m / 4, false) + 16u * 1024u <= kLdsLimit - 256) { fit = m; break; }
     }
-    if (fit == 0 || batch > (fit >= 16 ? 2u : 4u) * fit)
+    if (fit == 0 || batch > (fit >= 16 ? fit : 2 * fit))   // rows of 17408 columns: two passes of four rows still win
         return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): batch %u at %u columns is served by tiles", batch, cols);
     const auto *y = static_cast<const uint8_t *>(y_d4);
     for (uint32_t j0 = 0; j0 < batch; j0 += fit) {

@@ -199,7 +199,8 @@ def test_gemm_ragged_and_medium(gpu, oracle, rows, batch, cols):
 @pytest.mark.parametrize("batch", [1, 3, 4, 7, 8, 9, 12, 13, 16, 17, 29, 32])
 def test_gemm_small_batches_stream_the_weights(gpu, oracle, rows, cols, batch):
     """Batches of up to 16 rows on D4 activations are served by the weight-streaming matrix-core
-    GEMV (when the activations fit LDS): same contract as the tile kernel."""
+    GEMV (when the activations fit LDS), 17..32 by the narrowest ring tile: same contract as the
+    tile kernel."""
     if rows == 5120 and batch not in (4, 9, 16, 29):
         pytest.skip("big shape: three batches only")
     w = synth.q8_0_weight(rows, cols, seed=rows * 5 + cols)
@@ -271,3 +272,30 @@ def test_gemm_rejections(gpu):
     assert L.q8mi_gemm(b.ptr, b.ptr, b.ptr, 128, 128, 0, 128, NULL) == q8mi.REJECTED
     assert L.q8mi_gemm_medium(b.ptr, b.ptr, b.ptr, 128, 160, 4, 128, NULL) == q8mi.REJECTED
     assert L.q8mi_gemm_medium(b.ptr, b.ptr, b.ptr, 128, 128, 65, 128, NULL) == q8mi.REJECTED
+
+
+@pytest.mark.parametrize("rows,cols", [(1000, 256), (333, 1024), (5120, 5120), (640, 17408), (160, 2304)])
+@pytest.mark.parametrize("batch", [33, 48, 64, 65, 100, 128, 200])
+def test_gemm_medium_batches(gpu, oracle, rows, cols, batch):
+    """Batches too small to fill the chip with 128 x 128 tiles run 32-row tiles behind a ring of
+    LDS stages, 32, 64 or 128 activation rows wide, the narrow ones with K split over the waves:
+    rows and batch ragged against every tile width, K shorter and much longer than the ring."""
+    if rows == 5120 and batch not in (33, 64, 128):
+        pytest.skip("big shape: three batches only")
+    w = synth.q8_0_weight(rows, cols, seed=rows * 3 + cols)
+    x = synth.normal(batch, cols, seed=batch * 17 + cols)
+    x[batch // 2, :128] = 0.0
+    dw = dev(w)
+    dy, y = quantize_d4(x)
+    rc, ref = oracle.gemm_d4(w, y, rows, cols, batch, threads=8)
+    rr, jj = np.meshgrid(np.arange(rows, dtype=np.uint32), np.arange(batch, dtype=np.uint32))
+    rc, _, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr.reshape(-1), jj.reshape(-1))
+    stride = rows + 7
+    got = run_gemm(dw, dy, rows, cols, batch, stride=stride)
+    assert_close_fp32(got[:, :rows], ref, absum, f"gemm medium batch {batch}")
+    assert np.all(got[:, rows:].view(np.uint32) == 0xffffffff), "stores must stay inside the rows"
+    again = run_gemm(dw, dy, rows, cols, batch, stride=stride)
+    assert np.array_equal(again.view(np.uint32), got.view(np.uint32)), "deterministic"
+    if batch <= 64:
+        got_m = run_gemm(dw, dy, rows, cols, batch, medium=True)
+        assert np.array_equal(got_m.view(np.uint32), got[:, :rows].view(np.uint32))
