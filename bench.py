@@ -324,6 +324,30 @@ def bench_gemm(q8mi, hip, synth, reps=10):
     return out
 
 
+def bench_gemm_medium(q8mi, hip, synth, reps=30):
+    """Batches between the GEMV's and the prefill tile's (continuous-batching sizes) on the three
+    layer shapes: D4 activations through q8mi_gemm, microseconds per call over rotating weight copies."""
+    L, ok = q8mi.lib(), q8mi.ok
+    out = {}
+    for rows, cols in ((HIDDEN, HIDDEN), (FFN, HIDDEN), (HIDDEN, FFN)):
+        ws = [hip.to_device(synth.q8_0_weight(rows, cols, seed=s + 31)) for s in range(3)]
+        per = {}
+        for m in (16, 32, 64, 128):
+            x = hip.to_device(synth.normal(m, cols, seed=m))
+            y = hip.DeviceBuffer(L.q8mi_q8_1_d4_scratch_bytes(m, cols))
+            dst = hip.DeviceBuffer(4 * m * rows)
+            ok(L.q8mi_quantize_q8_1_d4(x.ptr, y.ptr, m, cols, cols, None), "quantize_d4")
+            t = time_loop(hip, lambda i: ok(L.q8mi_gemm(ws[i % 3].ptr, y.ptr, dst.ptr, rows, cols, m, rows, None), "gemm"),
+                          reps, 3)
+            per[f"m{m}"] = round(t * 1e3, 1)
+            for b in (x, y, dst):
+                b.free()
+        out[f"k{cols}_n{rows}_us"] = per
+        for b in ws:
+            b.free()
+    return out
+
+
 def bench_lm_head(q8mi, hip, synth, reps=10):
     """Fused LM head (5120 x 248320) + argmax + accept at M = 1, 2, 4, 6, 8."""
     L, ok = q8mi.lib(), q8mi.ok
@@ -377,8 +401,10 @@ def counter_calibration(q8mi, hip, n=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=10)
+    # a step is ~80 us: the defaults time 0.16 s after 40 ms of warm-up (the first milliseconds after
+    # the host-side set-up run at a lower clock)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
     ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -396,7 +422,8 @@ def main():
     q8mi.lib()
 
     if args.only == "gemm":
-        print(json.dumps({"gemm_int8": bench_gemm(q8mi, hip, synth, reps=max(args.steps // 20, 3))}))
+        print(json.dumps({"gemm_int8": bench_gemm(q8mi, hip, synth, reps=10),
+                          "gemm_medium_batches": bench_gemm_medium(q8mi, hip, synth)}))
         return
     if args.only == "lm_head":
         print(json.dumps({"lm_head_fused": bench_lm_head(q8mi, hip, synth)}))
@@ -472,6 +499,7 @@ def main():
         for v in result["gemm_int8"].values():
             v["frac_of_rescale_ceiling"] = round(v["tops"] / ceil["mfma_with_rescale_tops"], 4)
         result["gemm_int8"]["measured_ceilings"] = ceil
+        result["gemm_medium_batches"] = bench_gemm_medium(q8mi, hip, synth)
         result["lm_head_fused"] = bench_lm_head(q8mi, hip, synth)
     if not (args.quick or args.no_cpu):
         result["cpu_baseline"] = cpu_baseline()
