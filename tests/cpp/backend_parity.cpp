@@ -685,6 +685,43 @@ void case_graph_replay(qw3::HipQ8Backend &b) {
     }
     report("graph_replay_x4", ok, d);
 
+    // the fused norm + fan-out (one launch) and a medium-batch matmul (ring-staged tiles), captured
+    // together after one eager run and replayed with eager work in between
+    {
+        const uint32_t mb = 40;
+        auto nwv = normal_vec(hidden, 97, 0.3f);
+        for (auto &f : nwv) f += 1.0f;
+        auto nw = b.weight_f32(nwv.data(), hidden, "norm.weight");
+        auto normalized = b.tensor_f32(hidden, "normalized");
+        auto fo = b.tensor_f32(ffn, "fo");
+        qw3::DeviceTensor *outs[1] = {fo.get()};
+        const qw3::DeviceWeight *ws[1] = {dg.get()};
+        const uint32_t strides[1] = {ffn};
+        auto xm = upload_f32(b, normal_vec(static_cast<size_t>(mb) * hidden, 98));
+        auto om = b.tensor_f32(static_cast<size_t>(mb) * ffn, "om");
+        auto step2 = [&]() {
+            return b.rms_norm_q8_0_matmul_fanout(*normalized, outs, ws, strides, 1, *x, *nw, 1, hidden, 1e-6f).ok &&
+                   b.q8_0_matmul(*om, *du, *xm, mb, hidden, ffn).ok;
+        };
+        bool ok2 = step2() && require(b.synchronize(), "sync");
+        const auto e1 = download_f32(b, *fo), e2 = download_f32(b, *om);
+        ok2 = ok2 && b.begin_capture() && step2();
+        ok2 = require(b.end_capture(), "end_capture") && ok2;
+        std::string d2;
+        for (int rep = 0; rep < 3 && ok2; ++rep) {
+            ok2 = require(b.zero_tensor(*fo), "zero") && require(b.zero_tensor(*om), "zero") &&
+                  require(b.replay_graph(), "replay") && require(b.synchronize(), "sync");
+            const auto g1 = download_f32(b, *fo), g2 = download_f32(b, *om);
+            if (std::memcmp(g1.data(), e1.data(), g1.size() * 4) != 0 || std::memcmp(g2.data(), e2.data(), g2.size() * 4) != 0) {
+                ok2 = false;
+                d2 = "replay " + std::to_string(rep) + " differs";
+            }
+            auto tmp = b.tensor_f32(ffn, "tmp");
+            ok2 = ok2 && b.q8_0_matvec(*tmp, *dg, *x).ok && require(b.synchronize(), "sync");
+        }
+        report("graph_replay_norm_fanout_and_medium_matmul", ok2, d2);
+    }
+
     // growth of a scratch buffer is refused while capturing
     const HostWeight wbig = make_weight(64, 8192, 95);
     auto dbig = b.weight_q8_0(wbig.gguf.data(), 64, 8192, "big");
