@@ -152,7 +152,10 @@ int q8mi_rms_norm_quantize_q8_1(const float *x, const float *weight, float *norm
  * outputs are the bits of q8mi_rms_norm followed by the matching q8mi_qgemv* call.
  * Outputs are dense (one row).  Q8MI_REJECTED (nothing launched; use
  * q8mi_rms_norm_quantize_q8_1 and the GEMV) when batch != 1, cols is above 6144 or
- * not a multiple of 256, or x / weight / normalized are not 16-byte aligned. */
+ * not a multiple of 256, x / weight / normalized are not 16-byte aligned, or
+ * normalized == x (every workgroup reads x while one writes the normalised row, so
+ * the two must not overlap; q8mi_rms_norm and q8mi_rms_norm_quantize_q8_1 may work
+ * in place). */
 int q8mi_nqgemv(const uint8_t *weight, const float *x, const float *norm_weight, float eps, float *normalized,
                 void *dst, int dst_is_bf16, uint32_t rows, uint32_t cols, uint32_t batch, void *stream);
 int q8mi_nqgemv_silu_mul(const uint8_t *weight_gate, const uint8_t *weight_up, const float *x,

@@ -764,15 +764,18 @@ extern "C" int q8mi_gemv_two(const uint8_t *w0, const uint8_t *w1, const void *y
 }
 
 // ---- entry points that RMS-normalise and quantize one activation row inside the GEMV ----------
-static int norm_gate(const char *what, const float *x, const float *norm_weight, uint32_t batch) {
+static int norm_gate(const char *what, const float *x, const float *norm_weight, const float *normalized,
+                     uint32_t batch) {
     if (x == nullptr || norm_weight == nullptr) return fail(Q8MI_REJECTED, "%s: null pointer", what);
     if (batch != 1) return fail(Q8MI_REJECTED, "%s: batch %u (one row only)", what, batch);
+    // every workgroup reads x while workgroup 0 writes the normalised row
+    if (normalized == x) return fail(Q8MI_REJECTED, "%s: the normalised row must not overwrite x", what);
     return Q8MI_OK;
 }
 
 extern "C" int q8mi_nqgemv(const uint8_t *w, const float *x, const float *norm_weight, float eps, float *normalized,
                            void *dst, int dst_is_bf16, uint32_t rows, uint32_t cols, uint32_t batch, void *stream) {
-    if (int rc = norm_gate("nqgemv", x, norm_weight, batch)) return rc;
+    if (int rc = norm_gate("nqgemv", x, norm_weight, normalized, batch)) return rc;
     return run_single("nqgemv", dst_is_bf16 ? kStoreBF16 : kStoreF32, w, XSource{nullptr, x, cols, norm_weight, eps, normalized},
                       dst, rows, cols, batch, rows, stream);
 }
@@ -780,7 +783,7 @@ extern "C" int q8mi_nqgemv(const uint8_t *w, const float *x, const float *norm_w
 extern "C" int q8mi_nqgemv_silu_mul(const uint8_t *wg, const uint8_t *wu, const float *x, const float *norm_weight,
                                     float eps, float *normalized, float *dst, uint32_t rows, uint32_t cols,
                                     uint32_t batch, void *stream) {
-    if (int rc = norm_gate("nqgemv_silu_mul", x, norm_weight, batch)) return rc;
+    if (int rc = norm_gate("nqgemv_silu_mul", x, norm_weight, normalized, batch)) return rc;
     return run_silu_mul(wg, wu, XSource{nullptr, x, cols, norm_weight, eps, normalized}, dst, rows, cols, batch, rows,
                         stream);
 }
@@ -789,7 +792,7 @@ extern "C" int q8mi_nqgemv_fanout4(const uint8_t *w0, const uint8_t *w1, const u
                                    const float *x, const float *norm_weight, float eps, float *normalized, float *d0,
                                    float *d1, float *d2, float *d3, uint32_t rows0, uint32_t rows1, uint32_t rows2,
                                    uint32_t rows3, uint32_t cols, uint32_t batch, void *stream) {
-    if (int rc = norm_gate("nqgemv_fanout4", x, norm_weight, batch)) return rc;
+    if (int rc = norm_gate("nqgemv_fanout4", x, norm_weight, normalized, batch)) return rc;
     return run_fanout4(w0, w1, w2, w3, XSource{nullptr, x, cols, norm_weight, eps, normalized}, d0, d1, d2, d3, rows0,
                        rows1, rows2, rows3, cols, batch, rows0, rows1, rows2, rows3, stream);
 }

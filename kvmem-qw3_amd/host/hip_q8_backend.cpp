@@ -470,7 +470,8 @@ DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized,
     uint32_t r[4], s[4];
     uint32_t first = 0;
     bool quantized = false;
-    if (batch == 1) {   // the first four weights: norm + quantizer inside the GEMV, which also leaves `normalized`
+    if (batch == 1 && nrm != xin) {   // the first four weights: norm + quantizer inside the GEMV, which also leaves
+                                      // `normalized` (not in place: every workgroup reads x)
         group(0, wp, op, r, s);
         const int rc = q8mi_nqgemv_fanout4(wp[0], wp[1], wp[2], wp[3], xin, nwp, eps, nrm, op[0], op[1], op[2], op[3],
                                            r[0], r[1], r[2], r[3], cols, 1, stream_);

@@ -201,3 +201,23 @@ def test_nqgemv_rejections(gpu):
     assert L.q8mi_nqgemv(*args(5120, 1, x.at(4))) == q8mi.REJECTED    # vector loads need alignment
     assert L.q8mi_nqgemv(*args(5100, 1, x.ptr)) == q8mi.REJECTED      # cols % 32
     assert L.q8mi_nqgemv(*args(1056, 1, x.ptr)) == q8mi.REJECTED      # cols % 256 (weight planes off 16 bytes)
+    assert L.q8mi_nqgemv(w.ptr, x.ptr, x.at(32768), EPS, x.ptr, out.ptr, 0, 64, 5120, 1, NULL) == q8mi.REJECTED  # in place
+
+
+def test_rms_norm_in_place(gpu, oracle):
+    """The stand-alone norm (with or without the quantizer) may overwrite its input, long rows included."""
+    L = gpu.lib()
+    for n in (5120, 17408):
+        x, w = rows_of(n, 3, seed=n + 1)
+        ref = oracle.rms_norm(x, w, EPS)
+        rc, ref_y = oracle.quantize_q8_1(ref)
+        dx, dw = dev(x), dev(w)
+        ok(L.q8mi_rms_norm(dx.ptr, dw.ptr, dx.ptr, 3, n, n, n, EPS, NULL), "rms_norm in place")
+        hip.synchronize()
+        assert np.array_equal(dx.download(np.uint32), u32(ref).reshape(-1))
+        dx = dev(x)
+        y = hip.DeviceBuffer(L.q8mi_q8_1_scratch_bytes(3, n))
+        ok(L.q8mi_rms_norm_quantize_q8_1(dx.ptr, dw.ptr, dx.ptr, y.ptr, 3, n, n, n, EPS, NULL), "in place")
+        hip.synchronize()
+        assert np.array_equal(dx.download(np.uint32), u32(ref).reshape(-1))
+        assert np.array_equal(y.download(np.uint8), ref_y)
