@@ -221,3 +221,34 @@ def test_rms_norm_in_place(gpu, oracle):
         hip.synchronize()
         assert np.array_equal(dx.download(np.uint32), u32(ref).reshape(-1))
         assert np.array_equal(y.download(np.uint8), ref_y)
+
+
+def test_rms_norm_non_finite_rows(gpu, oracle):
+    """A NaN or an infinity in a row makes its scale NaN or zero; whatever comes out must be the
+    oracle's bits (normalised values compared as bit patterns, NaNs as NaNs) and its Q8_1 bytes."""
+    L = gpu.lib()
+    n = 1024
+    x, w = rows_of(n, 4, seed=5)
+    x[0, 17] = np.nan
+    x[1, 500] = np.inf
+    x[2, :] = 0.0                      # a zero row: scale = 1/sqrt(eps), outputs zero
+    x[3, 3] = -np.inf
+    ref = oracle.rms_norm(x, w, EPS)
+    rc, ref_y = oracle.quantize_q8_1(ref)
+    dx, dw = dev(x), dev(w)
+    nrm = hip.DeviceBuffer(4 * 4 * n)
+    y = hip.DeviceBuffer(L.q8mi_q8_1_scratch_bytes(4, n))
+    ok(L.q8mi_rms_norm_quantize_q8_1(dx.ptr, dw.ptr, nrm.ptr, y.ptr, 4, n, n, n, EPS, NULL), "rms_norm_quantize")
+    hip.synchronize()
+    got = nrm.download(np.float32).reshape(4, n)
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    keep = ~np.isnan(ref)
+    assert np.array_equal(got[keep].view(np.uint32), ref[keep].view(np.uint32))
+    assert np.all(got[2] == 0.0)
+    # quants and the scale halfword of every block; the sum halfword of a NaN block may differ in payload only
+    gy = y.download(np.uint8).reshape(-1, 36)
+    ry = ref_y.reshape(-1, 36)
+    assert np.array_equal(gy[:, 4:], ry[:, 4:])
+    gd, rd = gy[:, :4].copy().view(np.float16), ry[:, :4].copy().view(np.float16)
+    assert np.array_equal(np.isnan(gd), np.isnan(rd))
+    assert np.array_equal(gd[~np.isnan(rd)], rd[~np.isnan(rd)])
