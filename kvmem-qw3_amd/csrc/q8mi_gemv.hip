@@ -196,7 +196,7 @@ __device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, flo
 // ---- matrix-core variant for batch 3..32 (see q8mi_gemv_mfma_core.hpp) --------------------------
 // Unit u covers rows 4u .. 4u+3 of the concatenated row space; for SwiGLU gate rows 2u, 2u+1
 // (fragment rows 0, 1) and the matching up rows (fragment rows 2, 3).
-template <int MG, int THREADS, bool SILU, bool HS, bool D4>
+template <int MG, int THREADS, bool SILU, bool HS, bool D4, int DEPTH>
 __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, uint32_t batch,
                                                             uint32_t park_floats) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
 #ifdef Q8MI_TRACE
     const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
 #endif
-    mfma_stream<MG, THREADS, HS, D4>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
+    mfma_stream<MG, THREADS, HS, D4, DEPTH>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
 #ifdef Q8MI_TRACE
     const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
 #endif
@@ -430,12 +430,14 @@ int launch_m(const GemvParams &p, hipStream_t stream) {
     return p.mode == kSiluMul ? launch_ms<M, true>(p, stream) : launch_ms<M, false>(p, stream);
 }
 
+constexpr uint64_t kMfmaShallowMaxRows = 65536;
+
 // One workgroup of 512 threads per CU: its eight waves split the items of its units evenly, so a
 // matrix only needs as many 4-row units as there are CUs to keep the chip busy.
-template <int MG, bool SILU, bool HS, bool D4 = false>
-int launch_mfma(GemvParams p, uint32_t batch, hipStream_t stream) {
+template <int MG, bool SILU, bool HS, bool D4, int DEPTH>
+int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     constexpr int THREADS = 512;
-    auto kern = gemv_mfma_kernel<MG, THREADS, SILU, HS, D4>;
+    auto kern = gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH>;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
     p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG, HS);
@@ -462,6 +464,16 @@ int launch_mfma(GemvParams p, uint32_t batch, hipStream_t stream) {
 #endif
     kern<<<grid, THREADS, lds, stream>>>(p, batch, park_floats);
     return check_launch("gemv_mfma");
+}
+
+// Items a wave keeps in flight: one for layer-sized matrices (2 % faster at M = 4..8), two for long
+// streams such as a vocabulary (where one is much slower) and for the D4 route.
+template <int MG, bool SILU, bool HS, bool D4 = false>
+int launch_mfma(const GemvParams &p, uint32_t batch, hipStream_t stream) {
+    const uint64_t weight_rows = SILU ? 2ull * p.total_rows : p.total_rows;
+    if (!D4 && weight_rows <= kMfmaShallowMaxRows)
+        return launch_mfma_depth<MG, SILU, HS, D4, kMfmaGemvDepth>(p, batch, stream);
+    return launch_mfma_depth<MG, SILU, HS, D4, kMfmaDepth>(p, batch, stream);
 }
 
 // Activations that fit LDS in the matrix-core layout (with room for the parked sums).

@@ -75,6 +75,10 @@ inline uint32_t mfma_park_floats_per_unit(uint32_t mg) { return 4 * kMfmaUnitRow
 #define Q8MI_MFMA_DEPTH 2
 #endif
 constexpr int kMfmaDepth = Q8MI_MFMA_DEPTH;
+#ifndef Q8MI_MFMA_GEMV_DEPTH
+#define Q8MI_MFMA_GEMV_DEPTH 1
+#endif
+constexpr int kMfmaGemvDepth = Q8MI_MFMA_GEMV_DEPTH;   // the layer-sized GEMVs (Q8_1 activations)
 
 struct MfmaItem {
     v2i q[8];   // per step: bytes 8 t .. 8 t + 7 of the step's 128 bytes of row L / 16 (memory order),
@@ -223,7 +227,9 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *y,
 //                          meaningful in the lanes with lane / 16 == (lane % 16) / 4; must not touch
 //                          global memory
 // Must be called by every wave of the workgroup (contains the staging barrier).
-template <int MG, int THREADS, bool HS, bool D4, class RowPtr, class Park>
+// DEPTH: items a wave keeps in flight.  Two for the long LM-head stream and the D4 route; one for
+// the layer-sized GEMVs (measured 2 % faster there at M = 4..8, and much slower on the vocabulary).
+template <int MG, int THREADS, bool HS, bool D4, int DEPTH = kMfmaDepth, class RowPtr, class Park>
 __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uint32_t nb, uint32_t batch,
                                             uint32_t d4_batch_total, const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
                                             Park park) {
@@ -245,7 +251,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
     MfmaStage<MG, THREADS, HS> xstage;
     if constexpr (!D4) xstage.issue(y, nb, batch);
     asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
-    MfmaItem items[kMfmaDepth];
+    MfmaItem items[DEPTH];
     uint32_t ik = i0 / nitems, istep = i0 % nitems, ileft = n_items;
     const uint8_t *irow = row_ptr(useq.unit(ik));
     // Lane L loads slot (L % 16) ^ swz of row L / 16, swz = 2 for rows 2 and 3: the operand shuffle
@@ -272,7 +278,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
         }
     };
 #pragma unroll
-    for (int d = 0; d < kMfmaDepth; ++d) issue(items[d]);
+    for (int d = 0; d < DEPTH; ++d) issue(items[d]);
     asm volatile("" ::: "memory");   // keeps the loads above from being moved below the staging barrier
     if constexpr (D4) mfma_stage_x_d4<MG, THREADS>(smem, y, nb, batch, d4_batch_total);
     else xstage.finish(smem, y, nb, batch);
@@ -405,15 +411,15 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
     // last item the refills re-read it, so the loop stays branch-free and the load counters
     // exact); then the items of a last, partial round, without refills.
     uint32_t t = 0;
-    for (; t + kMfmaDepth <= n_items; t += kMfmaDepth) {
+    for (; t + DEPTH <= n_items; t += DEPTH) {
 #pragma unroll
-        for (int d = 0; d < kMfmaDepth; ++d) {
+        for (int d = 0; d < DEPTH; ++d) {
             consume(items[d], t + d + 1);
             issue(items[d]);
         }
     }
 #pragma unroll
-    for (int d = 0; d < kMfmaDepth - 1; ++d)
+    for (int d = 0; d < DEPTH - 1; ++d)
         if (t + d < n_items) consume(items[d], t + d + 1);
 }
 
