@@ -266,7 +266,9 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             // steps past the row's end re-read step 0; compute gives them a zero scale
-            it.q[s] = *reinterpret_cast<const v2i *>(qp + (static_cast<uint32_t>(s) < vsteps ? s * 128 : 0));
+            // read once per launch: streaming cache hint, as in the dot-product core
+            it.q[s] = __builtin_nontemporal_load(
+                reinterpret_cast<const v2i *>(qp + (static_cast<uint32_t>(s) < vsteps ? s * 128 : 0)));
         }
         if (ileft > 1) {          // otherwise keep re-reading the last real item
             --ileft;

@@ -112,7 +112,9 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const v4i *__restrict__
     const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
 #endif
     for (; i + 3 * stride < n16; i += 4 * stride) {
-        const v4i v0 = p[i], v1 = p[i + stride], v2 = p[i + 2 * stride], v3 = p[i + 3 * stride];
+        // streaming ("nt") loads, as the GEMV's weight loads
+        const v4i v0 = __builtin_nontemporal_load(p + i), v1 = __builtin_nontemporal_load(p + i + stride),
+                  v2 = __builtin_nontemporal_load(p + i + 2 * stride), v3 = __builtin_nontemporal_load(p + i + 3 * stride);
         a.x ^= v0.x ^ v1.x ^ v2.x ^ v3.x;
         a.y ^= v0.y ^ v1.y ^ v2.y ^ v3.y;
         a.z ^= v0.z ^ v1.z ^ v2.z ^ v3.z;
