@@ -344,19 +344,30 @@ __device__ __forceinline__ void stage_scales(uint8_t *stage, const Scales &sc, u
 template <bool CHECK, int RB>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
         const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
-        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles) {
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles,
+        uint32_t split_from) {
     using T = DmaTile<RB>;
     extern __shared__ __align__(16) uint8_t smem[];
     const uint32_t tid = threadIdx.x, lane = tid % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
+    // Tiles from split_from on are computed by two workgroups, one per half of K, which add their
+    // sums into a zeroed dst (see launch_dma): the tiles of a last, partly filled round.
+    uint32_t id = blockIdx.x, k_half = 0;
+    const bool split = id >= split_from;
+    if (split) {
+        k_half = (id - split_from) & 1u;
+        id = split_from + ((id - split_from) >> 1);
+    }
     // consecutive workgroup ids land on different XCDs: give every XCD whole row tiles and walk
     // the column tiles of a row tile back to back, so its weights stay in that XCD's L2
-    const uint32_t id = blockIdx.x, xcd = id % 8u, seq = id / 8u;
+    const uint32_t xcd = id % 8u, seq = id / 8u;
     const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
     if (rt >= row_tiles) return;   // uniform for the workgroup
     const uint32_t row0 = rt * T::kRows, col0 = ct * kTileCols;
     const uint32_t nsb = nb / 4;
+    const uint32_t sb0 = (split && k_half) ? nsb / 2 : 0u;
+    const uint32_t sb1 = (split && !k_half) ? nsb / 2 : nsb;
 
     v16i seed;
 #pragma unroll
@@ -383,12 +394,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
         lo.sc = gr * static_cast<uint32_t>(row_bytes);
         lo.ysc = (tid & 127u) * kRec;
     }
-    const uint8_t *wd_base = uniform_ptr(w + row0 * row_bytes);   // scale plane of the tile's first row
-    const uint8_t *wq_base = wd_base + 2 * nb;                     // its quant plane
-    const uint8_t *y_base = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec);
     const uint64_t y_step = static_cast<uint64_t>(batch) * kRec;
+    const uint8_t *wd_base = uniform_ptr(w + row0 * row_bytes + sb0 * 8u);   // scale plane of the tile's first row
+    const uint8_t *wq_base = wd_base + 2 * nb - sb0 * 8u + sb0 * 128u;       // its quant plane
+    const uint8_t *y_base = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec + sb0 * y_step);
     // last 16-byte offset from y_base that is still inside the activation buffer (used when CHECK)
-    uint64_t y_room = static_cast<uint64_t>(nsb) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
+    uint64_t y_room = static_cast<uint64_t>(nsb - sb0) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
     auto limit32 = [](uint64_t v) { return static_cast<uint32_t>(v < 0xffffffffull ? v : 0xffffffffull); };
     const uint32_t smem_off = lds_offset_of(smem);
 
@@ -403,10 +414,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
     const uint32_t b_row = l32 * 128;
     asm volatile("" : "+v"(seed));   // keep the seed in registers instead of rebuilding it per block
 
-    for (uint32_t sb = 0; sb < nsb; ++sb) {
-        const uint32_t cur_sel = (sb & 1u) * T::kStage, nxt_sel = T::kStage - cur_sel;
+    for (uint32_t sb = sb0; sb < sb1; ++sb) {
+        const uint32_t cur_sel = ((sb - sb0) & 1u) * T::kStage, nxt_sel = T::kStage - cur_sel;
         const uint8_t *cur = smem + cur_sel;
-        const bool more = sb + 1 < nsb;
+        const bool more = sb + 1 < sb1;
         if (more) {
             wq_base += 128; wd_base += 8; y_base += y_step; y_room -= y_step;
             stage_issue<CHECK, RB>(smem_off + nxt_sel, sc, lo, wq_base, wd_base, y_base, limit32(y_room), wave);
@@ -448,6 +459,20 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
         __syncthreads();
     }
     // D[i][n]: n = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (activation row)
+    if (split) {
+        // two addends onto zero: the sum does not depend on which half arrives first
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const uint32_t r = row0 + rb * 32 + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t j = col0 + wave * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
+                if (!CHECK || (r < rows && j < batch))
+                    unsafeAtomicAdd(&dst[static_cast<uint64_t>(j) * stride_dst + r], acc[rb][v]);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
         const uint32_t r = row0 + rb * 32 + l32;
@@ -456,6 +481,24 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
             const uint32_t j = col0 + wave * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
             if (!CHECK || (r < rows && j < batch)) dst[static_cast<uint64_t>(j) * stride_dst + r] = acc[rb][v];
         }
+    }
+}
+
+// Zeroes the dst patches of the tiles from split_from on (one workgroup per tile), which the two
+// K halves of gemm_d4_dma_kernel then add into.  A kernel rather than a memset so that a caller
+// can capture the launch into a graph.
+template <int RB>
+__global__ __launch_bounds__(kGemmThreads) void gemm_zero_split_tiles_kernel(
+        float *__restrict__ dst, uint32_t rows, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles,
+        uint32_t col_tiles, uint32_t split_from) {
+    using T = DmaTile<RB>;
+    const uint32_t id = split_from + blockIdx.x, xcd = id % 8u, seq = id / 8u;
+    const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
+    if (rt >= row_tiles) return;
+    const uint32_t row0 = rt * T::kRows, col0 = ct * kTileCols;
+    for (uint32_t i = threadIdx.x; i < T::kRows * kTileCols; i += kGemmThreads) {
+        const uint32_t r = row0 + i % T::kRows, j = col0 + i / T::kRows;
+        if (r < rows && j < batch) dst[static_cast<uint64_t>(j) * stride_dst + r] = 0.0f;
     }
 }
 
@@ -698,7 +741,16 @@ int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows
     return check_launch("gemm");
 }
 
-// Workgroups of each tile shape that one CU holds at a time (queried once per instantiation).
+// Q8MI_GEMM_SPLIT=0 (read only when the process runs with Q8MI_TUNE=1) switches the K split of
+// the last round off, for comparison.
+bool gemm_split_enabled() {
+    static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
+    if (live) {
+        if (const char *e = getenv("Q8MI_GEMM_SPLIT")) return atoi(e) != 0;
+    }
+    return true;
+}
+
 template <bool CHECK, int RB>
 int launch_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
                uint32_t stride, hipStream_t stream) {
@@ -715,10 +767,26 @@ int launch_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, ui
     }
     const uint32_t row_tiles = (rows + T::kRows - 1) / T::kRows;
     const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
-    const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
-    if (grid64 > 0x7fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
+    if (grid64 > 0x7ffffff0ull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    // A last round that fills at most half of the chip's slots (two workgroups per CU) leaves the
+    // other CUs idle for most of a tile's time: those tiles are cut in two along K and both halves
+    // add into a zeroed dst.  Measured on MI355X at M=2048: K=17408, N=5120 (640 tiles on 512 slots)
+    // and K=5120, N=17408 (2176 tiles).  Only main tiles on whole groups of eight row tiles (every
+    // id is a tile then) and at least four super-blocks of K.
+    uint32_t split_from = 0xffffffffu;
+    if (gemm_split_enabled() && RB == 4 && row_tiles % 8 == 0 && nb / 4 >= 4) {
+        const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
+        const uint64_t left = grid64 % slots;
+        if (grid64 >= slots && left != 0 && left * 2 <= slots) {
+            split_from = static_cast<uint32_t>(grid64 - left);
+            gemm_zero_split_tiles_kernel<RB><<<static_cast<uint32_t>(left), kGemmThreads, 0, stream>>>(
+                dst, rows, batch, stride, row_tiles, col_tiles, split_from);
+            grid64 += left;
+        }
+    }
     gemm_d4_dma_kernel<CHECK, RB><<<static_cast<uint32_t>(grid64), kGemmThreads, T::kLds, stream>>>(
-        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
+        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles, split_from);
     return check_launch("gemm");
 }
 

@@ -75,11 +75,13 @@ def test_gemm_reference_shapes(gpu, oracle, rows, batch, cols):
 
 
 @pytest.mark.parametrize("rows,batch,cols", [(4096, 2048, 256), (4480, 2050, 512), (9000, 1024, 256),
-                                             (17408, 2048, 128)])
+                                             (17408, 2048, 128), (5120, 2048, 512), (5120, 2000, 640),
+                                             (17408, 2048, 512)])
 def test_gemm_large_tilings(gpu, oracle, rows, batch, cols):
-    """Shapes with at least one full round of main tiles on the chip: main tiles only, and main
-    tiles + quarter tiles for the leftover rows (ragged in rows and batch), with a padded
-    output stride."""
+    """Shapes with at least one full round of main tiles on the chip: main tiles only, ragged in
+    rows and batch, with a padded output stride; the last three leave a last round of 128 tiles on
+    a 256-CU chip, which are computed as two halves of K added into a zeroed output (one with an
+    odd number of 128-column super-blocks and a ragged batch)."""
     w = synth.q8_0_weight(rows, cols, seed=rows + 3 * cols)
     x = synth.normal(batch, cols, seed=batch + 5 * cols)
     dw = dev(w)
@@ -102,6 +104,17 @@ def test_gemm_large_tilings(gpu, oracle, rows, batch, cols):
         rr = np.arange(rows, dtype=np.uint32)
         rc, ref_c, absum_c = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr, np.full(rows, j, np.uint32))
         assert_close_fp32(got[j, :rows], ref_c, absum_c, f"gemm column {j}")
+
+
+def test_gemm_split_last_round_is_deterministic(gpu):
+    """The tiles of a partly filled last round are summed from two halves of K by two workgroups
+    in whichever order they finish: two addends onto zero, so repeated calls agree bit for bit."""
+    rows, batch, cols = 5120, 2048, 1024
+    dw = dev(synth.q8_0_weight(rows, cols, seed=5))
+    dy, _ = quantize_d4(synth.normal(batch, cols, seed=6))
+    first = run_gemm(dw, dy, rows, cols, batch)
+    for _ in range(3):
+        assert np.array_equal(run_gemm(dw, dy, rows, cols, batch).view(np.uint32), first.view(np.uint32))
 
 
 # the layer's projections: QKV, O, gate/up (one shape), down
