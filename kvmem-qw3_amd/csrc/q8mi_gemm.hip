@@ -30,6 +30,7 @@
 // is then the correctly rounded d_w*S (12582912*d_w is exact: d_w has 11
 // significant bits), and acc = fma(g, d_y, acc): two FMAs per (output, block).
 #include <cstdio>
+#include <atomic>
 #include <cstdlib>
 
 #include "q8mi_device.hpp"
@@ -722,7 +723,7 @@ int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows
                    uint32_t batch, uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid,
                    hipStream_t stream) {
     // more than 64 KiB of dynamic LDS has to be granted per kernel, once per process
-    static bool granted = false;
+    static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
     if (!granted) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_kernel<CHECK, A16>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess) {
@@ -755,7 +756,7 @@ template <bool CHECK, int RB>
 int launch_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
                uint32_t stride, hipStream_t stream) {
     using T = DmaTile<RB>;
-    static bool granted = false;
+    static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
     if (!granted) {
         if (T::kLds > 64 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_dma_kernel<CHECK, RB>),
@@ -811,7 +812,7 @@ int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, u
     using T = RingTile<CB, W>;
     constexpr int lds = NS * T::kStage;
     static_assert(lds >= W * 16 * kWave * 4, "the stages are reused for the partial sums of the waves");
-    static bool granted = false;
+    static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
     if (!granted) {
         if (lds > 64 * 1024 &&
             hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS>),
