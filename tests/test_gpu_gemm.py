@@ -117,6 +117,27 @@ def test_gemm_split_last_round_is_deterministic(gpu):
         assert np.array_equal(run_gemm(dw, dy, rows, cols, batch).view(np.uint32), first.view(np.uint32))
 
 
+def test_gemm_split_last_round_replays_in_a_graph(gpu):
+    """The two-kernel call (zeroing kernel + GEMM with a K-split last round) captured into a HIP
+    graph: every replay, onto an output poisoned in between, gives the eager call's bits."""
+    rows, batch, cols = 5120, 2048, 512
+    dw = dev(synth.q8_0_weight(rows, cols, seed=15))
+    dy, _ = quantize_d4(synth.normal(batch, cols, seed=16))
+    eager = run_gemm(dw, dy, rows, cols, batch)
+    out = hip.DeviceBuffer(4 * batch * rows).fill(0xff)
+    stream = hip.Stream()
+    g = hip.Graph(stream)
+    with g:
+        ok(q8mi.lib().q8mi_gemm(dw.ptr, dy.ptr, out.ptr, rows, cols, batch, rows, stream.handle), "gemm")
+    for replay in range(3):
+        g.launch()
+        stream.synchronize()
+        got = out.download(np.float32).reshape(batch, rows)
+        assert np.array_equal(got.view(np.uint32), eager.view(np.uint32)), f"replay {replay}"
+        out.fill(0x7f)          # eager work between the replays
+        hip.synchronize()
+
+
 # the layer's projections: QKV, O, gate/up (one shape), down
 @pytest.mark.parametrize("rows,cols", [(5120, 5120), (8192, 5120), (5120, 6144), (17408, 5120), (5120, 17408)])
 def test_gemm_heavy_tail_batch_8192(gpu, oracle, rows, cols):
