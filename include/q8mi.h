@@ -179,10 +179,12 @@ int q8mi_quantize_q8_1_d4(const float *x, void *y_d4, uint32_t batch, uint32_t c
  * rows >= 128 && cols % 128 == 0 -> y is D4 (144-B super-blocks); otherwise y is
  * Q8_1 (36-B blocks).  Rejects cols % 32 != 0, rows == 0, batch == 0.
  * dst must be ordinary (coarse-grained) device memory: when the 128 x 128 tiles
- * leave a last round that fills at most half of the chip, those tiles are
+ * leave a last round that fills at most half of the chip, or when a batch of
+ * up to 32 rows gives at most one 32-row tile per CU, those outputs are
  * zeroed by a small kernel and then summed from two halves of K with hardware
  * fp32 atomic adds (two addends onto zero, so results repeat bit for bit); the
- * call then enqueues two kernels instead of one. */
+ * call then enqueues two kernels instead of one.  The same holds for
+ * q8mi_gemm_medium. */
 int q8mi_gemm(const uint8_t *weight, const void *y, float *dst, uint32_t rows, uint32_t cols,
               uint32_t batch, uint32_t stride_dst_row, void *stream);
 /* replaces launch_mmq_q8_0_medium, src/mmq_q8.cu:2512-2548: y is always D4.

@@ -555,10 +555,11 @@ __device__ __forceinline__ void wait_ring(uint32_t steps) {
     }
 }
 
-template <int CB, int W, int NS>
+template <int CB, int W, int NS, bool KSPLIT>
 __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
         const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
         uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles) {
+    constexpr bool ksplit = KSPLIT;
     using T = RingTile<CB, W>;
     constexpr uint32_t S = T::kShares;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -566,11 +567,16 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
     const uint32_t grp = wave % CB, share = wave / CB;   // activation group, K share
-    const uint32_t id = blockIdx.x, xcd = id % 8u, seq = id / 8u;
+    // ksplit: every tile is computed by two workgroups, one per half of K, which add their sums
+    // into a zeroed dst (see launch_ring)
+    const uint32_t id = ksplit ? blockIdx.x >> 1 : blockIdx.x, k_half = ksplit ? blockIdx.x & 1u : 0u;
+    const uint32_t xcd = id % 8u, seq = id / 8u;
     const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
     if (rt >= row_tiles) return;   // uniform for the workgroup
     const uint32_t row0 = rt * 32u, col0 = ct * T::kCols;
-    const uint32_t nsb = nb / 4;
+    const uint32_t nsb_all = nb / 4;
+    const uint32_t sb0 = (ksplit && k_half) ? nsb_all / 2 : 0u;                   // first super-block of this workgroup
+    const uint32_t nsb = ((ksplit && !k_half) ? nsb_all / 2 : nsb_all) - sb0;     // and how many it covers
     const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
 
     // The pieces of a step this wave loads: kind and LDS position are wave-uniform, the per-lane
@@ -599,15 +605,16 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     const uint8_t *wd_base0 = uniform_ptr(w + row0 * row_bytes);
     const uint8_t *y_base0 = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec);
     const uint64_t y_step = static_cast<uint64_t>(batch) * kRec;
-    const uint64_t y_room0 = static_cast<uint64_t>(nsb) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
+    const uint64_t y_room0 = static_cast<uint64_t>(nsb_all) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
     const uint32_t smem_off = lds_offset_of(smem);
 
-    auto issue = [&](uint32_t step) {
+    auto issue = [&](uint32_t step) {   // step counts from this workgroup's first super-block
         const uint32_t stage_off = smem_off + (step % NS) * T::kStage;
-        const uint8_t *wd_base = wd_base0 + static_cast<uint64_t>(step) * 8;
-        const uint8_t *wq_base = wd_base0 + 2 * nb + static_cast<uint64_t>(step) * 128;
-        const uint8_t *y_base = y_base0 + step * y_step;
-        const uint64_t room = y_room0 - step * y_step;
+        const uint32_t gstep = sb0 + step;
+        const uint8_t *wd_base = wd_base0 + static_cast<uint64_t>(gstep) * 8;
+        const uint8_t *wq_base = wd_base0 + 2 * nb + static_cast<uint64_t>(gstep) * 128;
+        const uint8_t *y_base = y_base0 + gstep * y_step;
+        const uint64_t room = y_room0 - gstep * y_step;
         const uint32_t y_limit = static_cast<uint32_t>(room < 0xffffffffull ? room : 0xffffffffull);
 #pragma unroll
         for (int i = 0; i < T::kLoads; ++i) {
@@ -673,7 +680,11 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     const uint32_t r_out = row0 + l32;
     auto store = [&](int v, float value) {
         const uint32_t j = col0 + grp * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
-        if (r_out < rows && j < batch) dst[static_cast<uint64_t>(j) * stride_dst + r_out] = value;
+        if (r_out < rows && j < batch) {
+            float *out = &dst[static_cast<uint64_t>(j) * stride_dst + r_out];
+            if constexpr (KSPLIT) unsafeAtomicAdd(out, value);   // two addends onto zero: order-independent
+            else *out = value;
+        }
     };
     if constexpr (S == 1) {
 #pragma unroll
@@ -695,6 +706,13 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
             store(v, total);
         }
     }
+}
+
+// Zeroes dst[j][0 .. rows) for j < batch: the start value of a launch whose workgroups add into dst.
+// A kernel rather than a memset so that a caller can capture the call into a graph.
+__global__ __launch_bounds__(256) void gemm_zero_dst_kernel(float *__restrict__ dst, uint32_t rows, uint32_t stride_dst) {
+    float *row = dst + static_cast<uint64_t>(blockIdx.y) * stride_dst;
+    for (uint32_t r = blockIdx.x * 1024u + threadIdx.x; r < rows && r < (blockIdx.x + 1u) * 1024u; r += 256u) row[r] = 0.0f;
 }
 
 // Ring depths and waves per workgroup of the medium-batch kernel (compile-time).  Measured on
@@ -806,29 +824,52 @@ int launch_dma_rows(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
 // ring-staged 32-row tiles.
 // Q8MI_GEMM_TILE (4 = main, 1 = two-stage quarter tiles; read only when the process runs with
 // Q8MI_TUNE=1) overrides the choice.
-template <int CB, int W, int NS>
-int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
-                uint32_t stride, hipStream_t stream) {
+template <int CB, int W, int NS, bool KSPLIT>
+int launch_ring_inst(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
+                     uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid, hipStream_t stream) {
     using T = RingTile<CB, W>;
     constexpr int lds = NS * T::kStage;
     static_assert(lds >= W * 16 * kWave * 4, "the stages are reused for the partial sums of the waves");
     static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
     if (!granted) {
         if (lds > 64 * 1024 &&
-            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS>),
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS, KSPLIT>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
             (void)hipGetLastError();
             return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", lds);
         }
         granted = true;
     }
+    gemm_d4_ring_kernel<CB, W, NS, KSPLIT><<<grid, kWave * W, lds, stream>>>(
+        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
+    return check_launch("gemm");
+}
+
+template <int CB, int W, int NS>
+int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
+                uint32_t stride, hipStream_t stream) {
+    using T = RingTile<CB, W>;
     const uint32_t row_tiles = (rows + 31u) / 32u;
     const uint32_t col_tiles = (batch + T::kCols - 1) / T::kCols;
     const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
-    if (grid64 > 0x7fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
-    gemm_d4_ring_kernel<CB, W, NS><<<static_cast<uint32_t>(grid64), kWave * W, lds, stream>>>(
-        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
-    return check_launch("gemm");
+    if (grid64 > 0x3fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    // With at most one tile per CU the launch lasts as long as one workgroup's chain of K steps
+    // (a step is bound by its serial latency, not by bandwidth or arithmetic): two workgroups per
+    // tile, one per half of K, halve that chain; they add into a dst zeroed by one more small
+    // kernel.  Two addends onto zero, so results repeat bit for bit.  Only the narrowest tile
+    // (up to 32 activation rows, four waves): measured on MI355X 19.2 -> 15.5 us at 5120 x 5120 and
+    // 58.6 -> 44.6 us at K = 17408, batch 32; the wider tiles already split K over their waves
+    // and gain nothing (64 rows) or lose (128 rows, sixteen waves: 29 -> 35 us).
+    if constexpr (CB == 1) {
+        if (gemm_split_enabled() && static_cast<uint64_t>(row_tiles) * col_tiles <= static_cast<uint32_t>(device_cu_count()) &&
+            nb / 4 >= 8 && batch <= 65535u) {
+            gemm_zero_dst_kernel<<<dim3((rows + 1023u) / 1024u, batch), 256, 0, stream>>>(dst, rows, stride);
+            return launch_ring_inst<CB, W, NS, true>(w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles,
+                                                     static_cast<uint32_t>(grid64 * 2), stream);
+        }
+    }
+    return launch_ring_inst<CB, W, NS, false>(w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles,
+                                              static_cast<uint32_t>(grid64), stream);
 }
 
 int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
