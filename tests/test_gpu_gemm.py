@@ -117,6 +117,24 @@ def test_gemm_split_last_round_is_deterministic(gpu):
         assert np.array_equal(run_gemm(dw, dy, rows, cols, batch).view(np.uint32), first.view(np.uint32))
 
 
+def test_gemm_narrow_tiles_split_along_k_are_deterministic(gpu, oracle):
+    """Up to 32 activation rows on at most one 32-row tile per CU: two workgroups per tile add their
+    halves of K into a zeroed output.  Repeated calls agree bit for bit, a poisoned output is fully
+    rewritten, the padding of a wider output stride is left alone, and the sums match the oracle."""
+    rows, batch, cols = 5120, 29, 5120
+    w = synth.q8_0_weight(rows, cols, seed=25)
+    dw = dev(w)
+    dy, y = quantize_d4(synth.normal(batch, cols, seed=26))
+    first = run_gemm(dw, dy, rows, cols, batch, stride=rows + 8)
+    assert np.all(first[:, rows:].view(np.uint32) == 0xffffffff)
+    for _ in range(3):
+        again = run_gemm(dw, dy, rows, cols, batch, stride=rows + 8)
+        assert np.array_equal(again.view(np.uint32), first.view(np.uint32))
+    rr, jj = np.meshgrid(np.arange(0, rows, 37, dtype=np.uint32), np.arange(batch, dtype=np.uint32))
+    rc, ref_s, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr.reshape(-1), jj.reshape(-1))
+    assert_close_fp32(first[jj.reshape(-1), rr.reshape(-1)], ref_s, absum, "narrow tiles, K split")
+
+
 def test_gemm_split_last_round_replays_in_a_graph(gpu):
     """The two-kernel call (zeroing kernel + GEMM with a K-split last round) captured into a HIP
     graph: every replay, onto an output poisoned in between, gives the eager call's bits."""
