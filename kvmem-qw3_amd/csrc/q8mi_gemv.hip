@@ -609,6 +609,11 @@ int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, 
     }
     if (fit == 0 || batch > (fit >= 16 ? fit : 2 * fit))   // rows of 17408 columns: two passes of four rows still win
         return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): batch %u at %u columns is served by tiles", batch, cols);
+    // ... unless the GEMM's 32-row tiles come at most one per CU: those are then cut in two along K
+    // (launch_ring) and beat two passes (measured at 17408 columns and 5..8 rows: 43 against 46..48 us
+    // on 5120 weight rows, 49 against 65..67 us on 8192)
+    if (batch > fit && (rows + 31u) / 32u <= static_cast<uint32_t>(device_cu_count()) && nb / 4 >= 8)
+        return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): batch %u at %u columns is served by split tiles", batch, cols);
     const auto *y = static_cast<const uint8_t *>(y_d4);
     for (uint32_t j0 = 0; j0 < batch; j0 += fit) {
         const uint32_t m = batch - j0 < fit ? batch - j0 : fit;
