@@ -30,6 +30,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "kvmem-qw3_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))      # q8mi_support: input generators and ceiling probes
 
 HBM_PEAK_GBPS = 8000.0        # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0       # MI355X published dense int8 MFMA rate (TOP/s)
@@ -62,7 +63,7 @@ class DecodeStep:
     """Buffers + the launch sequence of one layer's decode GEMVs for batch m."""
 
     def __init__(self, q8mi, hip, m, seed=1):
-        from q8mi import synth
+        import q8mi_support as synth
         self.L = q8mi.lib()
         self.ok = q8mi.ok
         self.m = m
@@ -169,6 +170,30 @@ def time_loop(hip, fn, steps, warmup):
     return e0.elapsed_ms(e1) / steps
 
 
+def time_loop_settled(hip, fn, steps, warmup, settle_ms=40.0, min_ms=100.0):
+    """The headline timing, robust against small --steps / --warmup: `warmup` untimed steps, then
+    further untimed rounds until settle_ms of device time have passed since the host-side set-up
+    (the first ~20 ms after it run a few per cent slow), then timed rounds of `steps` steps each
+    until at least min_ms of device time has been timed.  Returns (ms per step, steps timed)."""
+    done = 0
+    for i in range(warmup):
+        fn(done + i)
+    done += warmup
+    hip.synchronize()
+    round_ms = time_loop(hip, lambda i: fn(done + i), steps, 0) * steps     # untimed in effect: sizes the rest
+    done += steps
+    settled = round_ms
+    while settled < settle_ms:
+        settled += time_loop(hip, lambda i: fn(done + i), steps, 0) * steps
+        done += steps
+    total_ms, timed = 0.0, 0
+    while timed == 0 or total_ms < min_ms:
+        total_ms += time_loop(hip, lambda i: fn(done + i), steps, 0) * steps
+        done += steps
+        timed += steps
+    return total_ms / timed, timed
+
+
 def time_graph_replays(hip, record, steps, warmup):
     """Device time per replay of the launches `record(stream)` makes, captured once as a HIP graph
     on a stream of its own (events recorded on that stream)."""
@@ -210,7 +235,7 @@ def cpu_baseline(seconds=12.0):
     (5120x5120, M=1), timed on this host: once on one core, once row-parallel."""
     sys.path.insert(0, ROOT)
     from oracle import q8_oracle as o
-    from q8mi import synth
+    import q8mi_support as synth
     rows = cols = HIDDEN
     w = synth.q8_0_weight(rows, cols, seed=12345)
     x = synth.normal(1, cols, seed=54321)
@@ -241,7 +266,7 @@ def cpu_gemm_sample(rows=2048, m=2048, cols=HIDDEN):
     row-parallel on the host cores: a bounded sample of the prefill GEMM's CPU rate."""
     sys.path.insert(0, ROOT)
     from oracle import q8_oracle as o
-    from q8mi import synth
+    import q8mi_support as synth
     w = synth.q8_0_weight(rows, cols, seed=99)
     x = synth.normal(m, cols, seed=98)
     rc, y = o.quantize_q8_1_d4(x)
@@ -274,25 +299,29 @@ def bench_config0(q8mi, hip, synth, copies=48, reps=480):
             "resident_us": round(t_res * 1e3, 3), "resident_gbps": round(nbytes / (t_res * 1e-3) / 1e9, 1)}
 
 
-def bench_read_probe(q8mi, hip, nbytes=1 << 30, reps=20):
+def bench_read_probe(synth, hip, nbytes=1 << 30, reps=20):
     """Measured ceiling of a plain streaming read (every lane 16 bytes per load, grid-stride)."""
     buf, sink = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(64)
-    fn = lambda i: q8mi.ok(q8mi.lib().q8mi_probe_read(buf.ptr, nbytes, 2, sink.ptr, None), "probe_read")
+    fn = lambda i: synth.ok(synth.lib().q8sup_probe_read(buf.ptr, nbytes, 2, sink.ptr, None), "probe_read")
     t = time_loop(hip, fn, reps, 3)
     buf.free()
     sink.free()
     return round(nbytes / (t * 1e-3) / 1e9, 1)
 
 
-def bench_mfma_ceilings(q8mi, hip, iters=5000):
-    """Measured issue-rate ceilings of the matrix unit: int8 MFMAs alone, and with the scalar fp32
-    FMAs that rescaling their results costs (2 per int32 sum; packed fp32 math is not available)."""
-    L = q8mi.lib()
-    sink = hip.DeviceBuffer(L.q8mi_probe_mfma_sink_bytes())
+def bench_mfma_ceilings(synth, hip, iters=5000):
+    """Measured issue-rate ceilings of the matrix unit (register-only loops, two workgroups per CU):
+    int8 MFMAs alone; with the 2 scalar fp32 FMAs per int32 sum that rescaling costs (packed fp32 math
+    is not available), independent and fed by the MFMA results as in the kernel; and the arithmetic
+    with 1 FMA per sum (block sums as fp32 from the fp16 matrix unit, scale products from the fp32
+    matrix unit), in int8-equivalent TOP/s."""
+    L = synth.lib()
+    sink = hip.DeviceBuffer(L.q8sup_probe_mfma_sink_bytes())
     ops = C.c_uint64(0)
     out = {}
-    for name, flag in (("mfma_only_tops", 0), ("mfma_with_rescale_tops", 1)):
-        fn = lambda i: q8mi.ok(L.q8mi_probe_mfma(flag, iters, sink.ptr, C.byref(ops), None), "probe_mfma")
+    for name, mode in (("mfma_only_tops", 0), ("mfma_with_rescale_tops", 1), ("mfma_with_dependent_rescale_tops", 3),
+                       ("f16_mfma_one_fma_per_sum_tops", 2)):
+        fn = lambda i: synth.ok(L.q8sup_probe_mfma(mode, iters, sink.ptr, C.byref(ops), None), "probe_mfma")
         t = time_loop(hip, fn, 3, 1)
         out[name] = round(ops.value / (t * 1e-3) / 1e12, 1)
     sink.free()
@@ -389,12 +418,12 @@ def measured_traffic():
     return None
 
 
-def counter_calibration(q8mi, hip, n=3):
+def counter_calibration(synth, hip, n=3):
     """A few launches of a plain copy kernel of known size (reads and writes COPY_BYTES
     each): the reference point that memory-traffic counters of a profiled run are scaled by."""
     src, dst = hip.DeviceBuffer(COPY_BYTES), hip.DeviceBuffer(COPY_BYTES)
     for _ in range(n):
-        q8mi.ok(q8mi.lib().q8mi_probe_copy(src.ptr, dst.ptr, COPY_BYTES, None), "probe_copy")
+        synth.ok(synth.lib().q8sup_probe_copy(src.ptr, dst.ptr, COPY_BYTES, None), "probe_copy")
     hip.synchronize()
     src.free()
     dst.free()
@@ -403,10 +432,10 @@ def counter_calibration(q8mi, hip, n=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # a step is ~80 us: the defaults time 0.16 s after 40 ms of warm-up (the first milliseconds after
-    # the host-side set-up run at a lower clock)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=500)
+    # a step is ~80 us; whatever --steps and --warmup say, at least 40 ms run untimed first and at
+    # least 100 ms are timed (rounds of --steps steps), see time_loop_settled
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
     ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -417,7 +446,8 @@ def main():
                  "(the path would shard by weight rows: each GPU keeps rows/N of every weight)")
 
     import q8mi
-    from q8mi import hip, synth
+    from q8mi import hip
+    import q8mi_support as synth
     if hip.device_count() < 1:
         sys.exit("bench.py: no HIP device visible")
     hip.set_device(0)
@@ -430,15 +460,15 @@ def main():
     if args.only == "lm_head":
         print(json.dumps({"lm_head_fused": bench_lm_head(q8mi, hip, synth)}))
         return
-    counter_calibration(q8mi, hip)
+    counter_calibration(synth, hip)
     layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
     step = DecodeStep(q8mi, hip, m=1)
     step_bytes = step.algorithmic_bytes(layers[0].bytes)
 
-    # headline: K timed steps over rotating weight copies
-    ms_stream = time_loop(hip, lambda i: step.run(layers[i % len(layers)]), args.steps, args.warmup)
+    # headline: rounds of K timed steps over rotating weight copies, at least 100 ms of device time
+    ms_stream, steps_timed = time_loop_settled(hip, lambda i: step.run(layers[i % len(layers)]), args.steps, args.warmup)
     value = step_bytes / (ms_stream * 1e-3) / 1e9
-    ms_resident = time_loop(hip, lambda i: step.run(layers[0]), args.steps, args.warmup)
+    ms_resident, _ = time_loop_settled(hip, lambda i: step.run(layers[0]), args.steps, 0, settle_ms=0.0, min_ms=50.0)
 
     # dominant kernel: the fused gate/up SwiGLU GEMV (52 % of the step's bytes)
     n_each = min(max(args.steps, 50), 400)
@@ -451,6 +481,7 @@ def main():
     result = {
         "metric": "Q8_0 GEMV HBM GB/s at M=1 (decode GEMV set of one 27B-style layer)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "steps_timed": steps_timed, "device": hip.device_name(),
         "ms_per_step": round(ms_stream, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 x int8 -> int32 dots, fp32 accumulate", "data": "synthetic",
         "config": {"workload": "BASELINE config 1: decode GEMV set of one layer, M=1 "
@@ -497,12 +528,19 @@ def main():
             b.free()
     if not args.quick:
         result["config0_gemv_m1"] = bench_config0(q8mi, hip, synth)
-        result["hbm_read_probe_gbps"] = bench_read_probe(q8mi, hip)
+        result["hbm_read_probe_gbps"] = bench_read_probe(synth, hip)
         result["gemm_int8"] = bench_gemm(q8mi, hip, synth)
-        ceil = bench_mfma_ceilings(q8mi, hip)
+        ceil = bench_mfma_ceilings(synth, hip)
         for v in result["gemm_int8"].values():
             v["frac_of_rescale_ceiling"] = round(v["tops"] / ceil["mfma_with_rescale_tops"], 4)
         result["gemm_int8"]["measured_ceilings"] = ceil
+        # the second half of the dual metric in the shape of `roofline`: prefill GEMM at M=2048, gate/up shape
+        g = result["gemm_int8"]["m2048_k5120_n17408"]
+        result["roofline_gemm"] = {"bound": "mfma", "achieved": g["tops"], "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                   "frac": g["frac_of_int8_peak"], "traffic": None,
+                                   "kernel": "gemm_d4_dma_kernel<false, 4> (128 x 128 tiles, M=2048, K=5120, N=17408)",
+                                   "ops_per_launch": 2 * 2048 * FFN * HIDDEN, "launch_ms": g["gemm_ms"],
+                                   "frac_of_measured_rescale_ceiling": g["frac_of_rescale_ceiling"]}
         result["gemm_medium_batches"] = bench_gemm_medium(q8mi, hip, synth)
         result["lm_head_fused"] = bench_lm_head(q8mi, hip, synth)
     if not (args.quick or args.no_cpu):
@@ -510,10 +548,6 @@ def main():
         result["cpu_baseline"]["gemm_int8"] = cpu_gemm_sample()
     else:
         result["cpu_baseline"] = None
-    try:
-        result["device"] = hip.device_name()
-    except Exception:
-        pass
     print(json.dumps(result))
 
 

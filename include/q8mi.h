@@ -196,14 +196,12 @@ int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *dst, uint32
  * src/kernels_cuda.cu:14523-14530: out[i] = bf16(in[i]), round to nearest even. */
 int q8mi_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, void *stream);
 
-/* Checker hook (no counterpart in the reference): writes the int32 block dots
- * S[row][j][kb] = sum_t q_w*q_x for n sampled (row, j, kb) triples, computed on
- * the GPU with the same int8 dot instruction the kernels use.  y_layout:
- * 0 = Q8_1, 1 = D4.  sample arrays and out are device pointers. */
-int q8mi_block_dots(const uint8_t *weight, const void *y, int y_layout, uint32_t rows,
-                    uint32_t cols, uint32_t batch, const uint32_t *sample_row,
-                    const uint32_t *sample_j, const uint32_t *sample_kb, uint32_t n, int32_t *out,
-                    void *stream);
+/* replaces add_kernel / add_bf16_kernel, src/kernels_cuda.cu:1644-1677, as launched by add and
+ * add_n (:14818-14862): out[i] = a[i] + b[i] for i < n, fp32, or (is_bf16) three bf16 arrays with
+ * out[i] = bf16(f32(a[i]) + f32(b[i])) rounded to nearest even.  out may be a or b.  The second
+ * half of the reference's batched q8_0_matmul_add (include/qw3/device_backend.hpp:529-540:
+ * q8_0_matmul into a temporary, then add). */
+int q8mi_add(void *out, const void *a, const void *b, uint64_t n, int is_bf16, void *stream);
 
 /* ---- dequantizing row gather (embedding lookup) ---------------------------- */
 /* out[i] = fp32(d[i / 32]) * q[i] of one row, fp32 or (out_is_bf16) bf16 rounded
@@ -273,44 +271,6 @@ int q8mi_repack_q8_0_split_host(const void *gguf_blocks, uint64_t rows, uint64_t
 /* Same repack done on the GPU (both pointers device memory; in != out). */
 int q8mi_repack_q8_0_split(const void *gguf_blocks, uint64_t rows, uint64_t cols, void *split_out,
                            void *stream);
-
-/* ---- measurement helper --------------------------------------------------- */
-/* Plain streaming read of `bytes` device bytes (16-byte loads, grid-stride,
- * wgs_per_cu workgroups of 256 per CU): the practical HBM read ceiling that
- * the GEMV's achieved bandwidth is compared with.  No counterpart in the
- * reference.  sink: one device uint32 (never written in practice). */
-int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per_cu, uint32_t *sink,
-                    void *stream);
-/* Plain device-to-device copy of `bytes` bytes by a kernel (reads `bytes`,
- * writes `bytes`): the known-size launch that hardware memory-traffic counters
- * are calibrated against.  No counterpart in the reference. */
-int q8mi_probe_copy(const void *src, void *dst, uint64_t bytes, void *stream);
-/* Matrix-unit ceilings the GEMM is compared with: two workgroups of four waves
- * per CU, every wave running `iters` rounds of four independent
- * v_mfma_i32_32x32x32_i8 (what one wave issues per 32-block of a 128 x 128 GEMM
- * tile) plus, when with_rescale is nonzero, the 128 scalar fp32 FMAs that
- * rescaling those four results costs with packed fp32 math unavailable.
- * *ops_out (host) receives the int8 operations launched,
- * 2 * 32 * 32 * 32 * 4 * iters per wave; the caller times the launch.  No
- * counterpart in the reference.  sink: 2 * CUs * 256 device int32. */
-int q8mi_probe_mfma(int with_rescale, uint32_t iters, int32_t *sink, uint64_t *ops_out, void *stream);
-size_t q8mi_probe_mfma_sink_bytes(void);
-
-/* ---- synthetic inputs (host side, for benches and tests) ----------------- */
-/* Counter-based generator: element i of stream `seed` depends only on
- * (seed, i), so any thread split gives the same bytes.
- *   kind 0: N(0,1) * scale
- *   kind 1: Student-t(nu=3)/sqrt(3) * scale, with every column whose hash
- *           (seed, col) falls in the lowest `outlier_ppm` millionths multiplied
- *           by outlier_gain (BASELINE config 4: 1000 ppm, gain 20).
- * out: host fp32 [rows][cols]. */
-int q8mi_synth_f32(float *out, uint64_t rows, uint64_t cols, uint64_t seed, int kind, float scale,
-                   uint32_t outlier_ppm, float outlier_gain, int threads);
-/* N(0, sigma^2) weights quantized to Q8_0 (tests/mmq_parity.cu:54-80 rule:
- * d = amax/127 stored fp16, q = clamp(lrintf(w * (1/d)), +-127)) and written
- * straight into split-plane rows.  out: host, rows*cols/32*34 bytes. */
-int q8mi_synth_q8_0_weight(uint8_t *split_out, uint64_t rows, uint64_t cols, uint64_t seed,
-                           float sigma, int threads);
 
 #ifdef __cplusplus
 }

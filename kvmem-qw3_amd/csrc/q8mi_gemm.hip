@@ -29,9 +29,7 @@
 // F = 12582912 + S exactly (|S| <= 516128 < 2^22).  g = fma(F, d_w, -12582912*d_w)
 // is then the correctly rounded d_w*S (12582912*d_w is exact: d_w has 11
 // significant bits), and acc = fma(g, d_y, acc): two FMAs per (output, block).
-#include <cstdio>
 #include <atomic>
-#include <cstdlib>
 
 #include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
@@ -720,21 +718,8 @@ __global__ __launch_bounds__(256) void gemm_zero_dst_kernel(float *__restrict__ 
 // path of a step binds), eight waves beat four by 1.4 x at 64 activation rows, sixteen beat eight
 // at 128 rows only while there is at most one tile per CU; two super-blocks per step (half as
 // many barriers, two independent chains per wave) were 1.2-1.3 x slower at the same LDS budget.
-#ifndef Q8MI_RING1
-#define Q8MI_RING1 6
-#endif
-#ifndef Q8MI_RING2
-#define Q8MI_RING2 4
-#endif
-#ifndef Q8MI_RING4
-#define Q8MI_RING4 3
-#endif
-#ifndef Q8MI_RINGW2
-#define Q8MI_RINGW2 8
-#endif
-#ifndef Q8MI_RINGW4
-#define Q8MI_RINGW4 8
-#endif
+constexpr int kRing1 = 6, kRing2 = 4, kRing4 = 3;   // ring depth of the 32-, 64- and 128-row-wide tile
+constexpr int kRingWaves2 = 8, kRingWaves4 = 8;    // waves per workgroup of the 64- and 128-wide tile
 
 template <bool CHECK, bool A16>
 int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb,
@@ -749,25 +734,10 @@ int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows
             return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", kLdsBytes);
         }
         granted = true;
-#ifdef Q8MI_TRACE
-        int occ = -1;
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, gemm_d4_kernel<CHECK, A16>, kGemmThreads, kLdsBytes);
-        fprintf(stderr, "gemm_d4_kernel<%d,%d>: %d workgroups per CU\n", int(CHECK), int(A16), occ);
-#endif
     }
     gemm_d4_kernel<CHECK, A16><<<grid, kGemmThreads, kLdsBytes, stream>>>(
         w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
     return check_launch("gemm");
-}
-
-// Q8MI_GEMM_SPLIT=0 (read only when the process runs with Q8MI_TUNE=1) switches the K split of
-// the last round off, for comparison.
-bool gemm_split_enabled() {
-    static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
-    if (live) {
-        if (const char *e = getenv("Q8MI_GEMM_SPLIT")) return atoi(e) != 0;
-    }
-    return true;
 }
 
 template <bool CHECK, int RB>
@@ -794,7 +764,7 @@ int launch_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, ui
     // and K=5120, N=17408 (2176 tiles).  Only main tiles on whole groups of eight row tiles (every
     // id is a tile then) and at least four super-blocks of K.
     uint32_t split_from = 0xffffffffu;
-    if (gemm_split_enabled() && RB == 4 && row_tiles % 8 == 0 && nb / 4 >= 4) {
+    if (RB == 4 && row_tiles % 8 == 0 && nb / 4 >= 4) {
         const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
         const uint64_t left = grid64 % slots;
         if (grid64 >= slots && left != 0 && left * 2 <= slots) {
@@ -822,8 +792,6 @@ int launch_dma_rows(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
 // little: problems with at least 0.4 main tiles per resident slot (two per CU) use main tiles
 // throughout (measured crossover on MI355X: between 160 and 256 main tiles); smaller ones use the
 // ring-staged 32-row tiles.
-// Q8MI_GEMM_TILE (4 = main, 1 = two-stage quarter tiles; read only when the process runs with
-// Q8MI_TUNE=1) overrides the choice.
 template <int CB, int W, int NS, bool KSPLIT>
 int launch_ring_inst(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
                      uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid, hipStream_t stream) {
@@ -861,7 +829,7 @@ int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, u
     // 58.6 -> 44.6 us at K = 17408, batch 32; the wider tiles already split K over their waves
     // and gain nothing (64 rows) or lose (128 rows, sixteen waves: 29 -> 35 us).
     if constexpr (CB == 1) {
-        if (gemm_split_enabled() && static_cast<uint64_t>(row_tiles) * col_tiles <= static_cast<uint32_t>(device_cu_count()) &&
+        if (static_cast<uint64_t>(row_tiles) * col_tiles <= static_cast<uint32_t>(device_cu_count()) &&
             nb / 4 >= 8 && batch <= 65535u) {
             gemm_zero_dst_kernel<<<dim3((rows + 1023u) / 1024u, batch), 256, 0, stream>>>(dst, rows, stride);
             return launch_ring_inst<CB, W, NS, true>(w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles,
@@ -878,21 +846,15 @@ int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
     const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
     const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
     const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
-    int tile = tiles * 5 >= slots * 2 ? 4 : 0;
-    static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
-    if (live) {
-        if (const char *e = getenv("Q8MI_GEMM_TILE")) tile = atoi(e);
-    }
-    if (tile == 4) return launch_dma_rows<4>(w, y, dst, rows, nb, batch, stride, stream);
-    if (tile == 1) return launch_dma_rows<1>(w, y, dst, rows, nb, batch, stride, stream);   // two-stage quarter tiles
+    if (tiles * 5 >= slots * 2) return launch_dma_rows<4>(w, y, dst, rows, nb, batch, stride, stream);
     // too few main tiles to fill the chip: 32-row tiles behind a ring of stages, as wide as the batch needs
-    if (batch <= 32) return launch_ring<1, 4, Q8MI_RING1>(w, y, dst, rows, nb, batch, stride, stream);
-    if (batch <= 64) return launch_ring<2, Q8MI_RINGW2, Q8MI_RING2>(w, y, dst, rows, nb, batch, stride, stream);
+    if (batch <= 32) return launch_ring<1, 4, kRing1>(w, y, dst, rows, nb, batch, stride, stream);
+    if (batch <= 64) return launch_ring<2, kRingWaves2, kRing2>(w, y, dst, rows, nb, batch, stride, stream);
     // at most one tile per CU: sixteen waves (four K shares per group) instead of eight
     const uint64_t ring_tiles = static_cast<uint64_t>((rows + 31u) / 32u) * ((batch + 127u) / 128u);
     if (ring_tiles <= static_cast<uint32_t>(device_cu_count()))
-        return launch_ring<4, 16, Q8MI_RING4>(w, y, dst, rows, nb, batch, stride, stream);
-    return launch_ring<4, Q8MI_RINGW4, Q8MI_RING4>(w, y, dst, rows, nb, batch, stride, stream);
+        return launch_ring<4, 16, kRing4>(w, y, dst, rows, nb, batch, stride, stream);
+    return launch_ring<4, kRingWaves4, kRing4>(w, y, dst, rows, nb, batch, stride, stream);
 }
 
 int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,

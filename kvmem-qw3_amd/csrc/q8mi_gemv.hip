@@ -10,8 +10,6 @@
 // once per unit, so they are a runtime switch; SwiGLU changes which rows a unit
 // streams and is a template parameter (its launches also show up under their own
 // kernel name in a profile).
-#include <stdlib.h>
-
 #include "q8mi_gemv_core.hpp"
 #include "q8mi_gemv_mfma_core.hpp"
 
@@ -43,9 +41,6 @@ struct GemvParams {
     uint32_t x_bytes;     // LDS bytes of the staged activations (0 when they are read from global)
     int mode;
     int interleave;
-#ifdef Q8MI_TRACE
-    unsigned long long *trace;   // [grid][4] timestamps (tuning builds only)
-#endif
 };
 
 // Which of the (up to four) concatenated weights a row belongs to.
@@ -91,9 +86,6 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t nsteps = (p.nb * 2 + 127) / 128;
     const uint64_t row_bytes = static_cast<uint64_t>(p.nb) * 34;
-#ifdef Q8MI_TRACE
-    const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
-#endif
     const UnitSeq useq = group_units(p.units, blockIdx.x, gridDim.x, p.interleave);
     const uint32_t ucount = useq.count;
     const uint32_t n_items = ucount * nsteps;
@@ -129,17 +121,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
     // written before the staging barrier
     const XIn in{p.y, p.xf, p.x_stride, p.norm_w, p.eps, p.normalized, park_base};
     gemv_stream<M, R, THREADS, XMODE>(smem, in, p.nb, useq, i0, i1, rows_of, park);
-#ifdef Q8MI_TRACE
-    const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
-#endif
     __syncthreads();
-#ifdef Q8MI_TRACE
-    if (p.trace && threadIdx.x == 0) {
-        p.trace[blockIdx.x * 4 + 0] = t_begin;
-        p.trace[blockIdx.x * 4 + 1] = t_stream;
-        p.trace[blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
-    }
-#endif
 
     // combine + write-out: entry e = (unit ordinal k, activation row m, slot r)
     auto total_of = [&](uint32_t k, uint32_t mr) {
@@ -174,9 +156,6 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
             store_out(p.mode, ref.dst, static_cast<uint64_t>(m) * ref.stride + ref.local, total_of(k, mr));
         }
     }
-#ifdef Q8MI_TRACE
-    if (p.trace && threadIdx.x == 0) p.trace[blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
-#endif
 }
 
 __device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, float v) {
@@ -240,21 +219,8 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
             }
         }
     };
-#ifdef Q8MI_TRACE
-    const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
-#endif
     mfma_stream<MG, THREADS, HS, D4, DEPTH>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
-#ifdef Q8MI_TRACE
-    const unsigned long long t_stream = __builtin_amdgcn_s_memrealtime();
-#endif
     __syncthreads();
-#ifdef Q8MI_TRACE
-    if (p.trace && threadIdx.x == 0) {
-        p.trace[blockIdx.x * 4 + 0] = t_begin;
-        p.trace[blockIdx.x * 4 + 1] = t_stream;
-        p.trace[blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
-    }
-#endif
 
     // unit ranges of the waves, worked out once (wave w touched unit ordinals kf[w] .. kl[w])
     __shared__ uint32_t s_kf[kWaves], s_kl[kWaves];
@@ -296,9 +262,6 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
             store_out(p.mode, ref.dst, static_cast<uint64_t>(m) * ref.stride + ref.local, total_of(k, rr, m));
         }
     }
-#ifdef Q8MI_TRACE
-    if (p.trace && threadIdx.x == 0) p.trace[blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
-#endif
 }
 
 // Fallback for rows whose planes are not 16-byte aligned (cols/32 not a
@@ -349,40 +312,21 @@ __global__ __launch_bounds__(256) void gemv_unaligned_kernel(const GemvParams p,
     }
 }
 
-// One launch of a given instantiation: geometry is cached per (instantiation, LDS size).
+// One launch of a given instantiation.
 template <int M, int THREADS, int XMODE, bool SILU>
 int launch_inst(GemvParams p, uint32_t x_bytes, hipStream_t stream) {
     auto kern = gemv_kernel<M, THREADS, XMODE, SILU>;
+    static KernelGeometry geometry;
     constexpr uint32_t R = RowsPerUnit<M>::value;
     p.x_bytes = x_bytes;
     p.units = SILU ? (p.total_rows + R / 2 - 1) / (R / 2) : (p.total_rows + R - 1) / R;
     const uint32_t lds = x_bytes + (THREADS / kWave) * kParkFloats * 4;
-    static thread_local uint32_t cached_lds = 0xffffffffu;
-    static thread_local int cached_occ = 0;
-    if (cached_lds != lds) {
-        if (lds > 64u * 1024u &&
-            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(lds)) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
-        }
-        int occ = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, THREADS, lds) != hipSuccess || occ < 1) {
-            (void)hipGetLastError();
-            occ = 1;
-        }
-        cached_occ = occ;
-        cached_lds = lds;
-    }
+    if (lds > kLdsLimit || !geometry.grant(reinterpret_cast<const void *>(kern), kLdsLimit))
+        return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
+    uint32_t per_cu = geometry.workgroups_per_cu(kern, THREADS, lds);
+    if (per_cu > kGemvWgsPerCu) per_cu = kGemvWgsPerCu;
+    p.interleave = kGemvInterleave;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
-    const GemvTuning tune = gemv_tuning();
-    uint32_t per_cu = static_cast<uint32_t>(cached_occ);
-    if (tune.wgs_per_cu > 0 && static_cast<uint32_t>(tune.wgs_per_cu) < per_cu) per_cu = tune.wgs_per_cu;
-    p.interleave = tune.interleave;
-#ifdef Q8MI_TRACE
-    p.trace = nullptr;
-    if (const char *e = getenv("Q8MI_TRACE_PTR")) p.trace = reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 0));
-#endif
     const uint32_t grid = pick_grid(p.units, (p.nb * 2 + 127) / 128, M, THREADS / kWave, cus, per_cu);
     kern<<<grid, THREADS, lds, stream>>>(p);
     return check_launch("gemv");
@@ -392,7 +336,6 @@ template <int M, bool SILU>
 int launch_ms(const GemvParams &p, hipStream_t stream) {
     const uint32_t xb = x_lds_bytes(p.nb, M);
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
-    const int forced = gemv_tuning().threads;
     if (p.norm_w != nullptr) {   // fused norm + quantizer: one row, held in registers between the two passes
         if constexpr (M == 1) {
             const uint32_t cols = p.nb * kQK;
@@ -411,15 +354,13 @@ int launch_ms(const GemvParams &p, hipStream_t stream) {
         if (M > 2) return fail(Q8MI_REJECTED, "qgemv: batch %d above 2 (quantize once and use the GEMV instead)", M);
         // rows above 8192 columns: one 1024-thread workgroup per CU quantizes them once per CU instead of twice
         const bool long_rows = p.nb * kQK > 8192u && xb + park_1024 <= kLdsLimit;
-        if (xb + park_256 <= 76u * 1024u && forced != 1024 && !long_rows)
+        if (xb + park_256 <= 76u * 1024u && !long_rows)
             return launch_inst<M, 256, kXF32, SILU>(p, xb, stream);
         if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXF32, SILU>(p, xb, stream);
         return fail(Q8MI_REJECTED, "qgemv: %u activation rows of %u columns do not fit LDS", M, p.nb * 32);
     }
     // the LDS staging loads 16 bytes at a time: activations on a 4-byte boundary are read by the lanes
     if (reinterpret_cast<uintptr_t>(p.y) % 16 != 0) return launch_inst<M, 256, kXGlobal, SILU>(p, 0, stream);
-    if (forced == 256 && xb + park_256 <= kLdsLimit) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);
-    if (forced == 1024 && xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds, SILU>(p, xb, stream);
     if (xb + park_256 <= 76u * 1024u) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);   // two per CU fit
     if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXLds, SILU>(p, xb, stream);
     return launch_inst<M, 256, kXGlobal, SILU>(p, 0, stream);
@@ -441,7 +382,7 @@ int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
     p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG, HS);
-    p.interleave = gemv_tuning().interleave;
+    p.interleave = kGemvInterleave;
     const uint32_t grid = p.units < cus ? p.units : cus;
     const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
     const uint32_t per_group = (p.units + grid - 1) / grid;
@@ -449,19 +390,9 @@ int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     const uint32_t lds = p.x_bytes + (THREADS / kWave) * park_floats * 4;
     constexpr uint32_t kDynLimit = kLdsLimit - 256;   // the kernel also has a few static LDS words
     if (lds > kDynLimit) return fail(Q8MI_REJECTED, "gemv (matrix-core variant): %u bytes of LDS needed", lds);
-    static thread_local uint32_t granted = 0;
-    if (lds > 64u * 1024u && lds > granted) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(kDynLimit)) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
-        }
-        granted = kDynLimit;
-    }
-#ifdef Q8MI_TRACE
-    p.trace = nullptr;
-    if (const char *e = getenv("Q8MI_TRACE_PTR")) p.trace = reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 0));
-#endif
+    static KernelGeometry geometry;
+    if (!geometry.grant(reinterpret_cast<const void *>(kern), kDynLimit))
+        return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
     kern<<<grid, THREADS, lds, stream>>>(p, batch, park_floats);
     return check_launch("gemv_mfma");
 }
@@ -507,7 +438,7 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         return check_launch("gemv_unaligned");
     }
     if (p.xf == nullptr && reinterpret_cast<uintptr_t>(p.y) % 16 == 0 &&
-        batch >= static_cast<uint32_t>(gemv_tuning().mfma_from) &&
+        batch >= kMfmaFromBatch &&
         (mfma_fits(p.nb, batch, false) || mfma_fits(p.nb, batch, true))) {
         const int rc = launch_mfma_any(p, batch, stream);
         if (rc != Q8MI_REJECTED) return rc;   // a unit list whose parked sums do not fit: dot-product variant
@@ -574,22 +505,6 @@ int run_single(const char *what, int mode, const uint8_t *w, const XSource &y, v
 }
 
 }  // namespace
-
-// Shipped configuration: two workgroups per CU, interleaved units (best of the sweeps);
-// the matrix-core variant from batch kMfmaFromBatch on.
-constexpr int kMfmaFromBatch = 3;
-GemvTuning gemv_tuning() {
-    static const bool live = [] { const char *e = getenv("Q8MI_TUNE"); return e && e[0] == '1'; }();
-    auto read = [] {
-        GemvTuning t{2, 1, 0, kMfmaFromBatch};
-        if (const char *e = getenv("Q8MI_GEMV_WGS_PER_CU")) t.wgs_per_cu = atoi(e);
-        if (const char *e = getenv("Q8MI_GEMV_INTERLEAVE")) t.interleave = atoi(e);
-        if (const char *e = getenv("Q8MI_GEMV_THREADS")) t.threads = atoi(e);
-        if (const char *e = getenv("Q8MI_GEMV_MFMA_FROM")) t.mfma_from = atoi(e);
-        return t;
-    };
-    return live ? read() : GemvTuning{2, 1, 0, kMfmaFromBatch};
-}
 
 // D4-quantized activations through the matrix-core GEMV: what the GEMM entry points use for
 // batches too small for an MFMA tile.  As many activation rows per launch as fit LDS (at most 16:

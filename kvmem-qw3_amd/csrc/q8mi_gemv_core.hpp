@@ -25,6 +25,9 @@
 // lanes read them from global memory (served by L2).
 #pragma once
 
+#include <atomic>
+#include <mutex>
+
 #include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
 #include "q8mi_quantize_core.hpp"
@@ -538,16 +541,55 @@ __host__ __device__ inline uint32_t max_units_touched(uint32_t group_units_max, 
 }
 
 // ---- host side: launch geometry -------------------------------------------
-// Launch-geometry knobs.  Defaults are the shipped configuration; when the
-// process starts with Q8MI_TUNE=1 they are re-read from the environment on every
-// launch (used by tuning sweeps only).
-struct GemvTuning {
-    int wgs_per_cu;    // 0 = as many as fit (occupancy)
-    int interleave;    // unit assignment, see group_units
-    int threads;       // 0 = by LDS footprint, else 256 or 1024
-    int mfma_from;     // smallest batch served by the matrix-core variant
+// Measured best on MI355X: two workgroups per CU, units dealt round-robin to the workgroups
+// (neighbouring workgroups read neighbouring rows), the matrix-core variant from batch 3 on.
+constexpr uint32_t kGemvWgsPerCu = 2;
+constexpr int kGemvInterleave = 1;        // unit assignment, see group_units
+constexpr uint32_t kMfmaFromBatch = 3;    // smallest batch served by the matrix-core variant
+
+// Per kernel instantiation (one static instance each): the dynamic LDS limit is raised once, to
+// the most any launch of this kernel may ask for and never lowered again, so launches from
+// several host threads cannot undercut one another; workgroups per CU are looked up once per
+// distinct LDS size and kept in a small process-wide table.
+class KernelGeometry {
+public:
+    // false when the runtime refuses the LDS grant
+    bool grant(const void *kernel, uint32_t max_dynamic_lds) {
+        if (granted_.load(std::memory_order_acquire)) return true;
+        std::lock_guard<std::mutex> lock(mu_);
+        if (granted_.load(std::memory_order_relaxed)) return true;
+        if (max_dynamic_lds > 64u * 1024u &&
+            hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(max_dynamic_lds)) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        granted_.store(true, std::memory_order_release);
+        return true;
+    }
+    template <class Kernel>
+    uint32_t workgroups_per_cu(Kernel kernel, int threads, uint32_t lds) {
+        std::lock_guard<std::mutex> lock(mu_);
+        for (uint32_t i = 0; i < n_; ++i)
+            if (lds_[i] == lds) return occ_[i];
+        int occ = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, threads, lds) != hipSuccess || occ < 1) {
+            (void)hipGetLastError();
+            occ = 1;
+        }
+        if (n_ < kSlots) {
+            lds_[n_] = lds;
+            occ_[n_] = static_cast<uint32_t>(occ);
+            ++n_;
+        }
+        return static_cast<uint32_t>(occ);
+    }
+
+private:
+    static constexpr uint32_t kSlots = 32;
+    std::mutex mu_;
+    std::atomic<bool> granted_{false};
+    uint32_t lds_[kSlots] = {}, occ_[kSlots] = {}, n_ = 0;
 };
-GemvTuning gemv_tuning();
 
 // Parked units per wave for batch M.
 inline uint32_t park_capacity(uint32_t m) { return kParkFloats / (m * (m >= 4 ? 4u : 2u)); }

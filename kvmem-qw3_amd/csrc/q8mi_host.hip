@@ -1,13 +1,8 @@
 // Host-side pieces of the library: error text, device queries, the weight
-// repack (host and device), the block-dot checker hook and the synthetic input
-// generator.
-#include <math.h>
+// repack (host and device) and the small elementwise kernels.
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
-
-#include <thread>
-#include <vector>
 
 #include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
@@ -66,32 +61,6 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint16_t *__restrict_
     for (int t = 0; t < 16; ++t) q[t] = src[1 + t];
 }
 
-// ---- checker hook: int32 block dots on the GPU -------------------------------
-__global__ __launch_bounds__(256) void block_dots_kernel(const uint8_t *__restrict__ w,
-                                                         const uint8_t *__restrict__ y, int layout,
-                                                         uint32_t nb, uint32_t batch,
-                                                         const uint32_t *__restrict__ sr,
-                                                         const uint32_t *__restrict__ sj,
-                                                         const uint32_t *__restrict__ sk, uint32_t n,
-                                                         int32_t *__restrict__ out) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    const uint32_t row = sr[i], j = sj[i], kb = sk[i];
-    const uint16_t *wq = reinterpret_cast<const uint16_t *>(w + static_cast<uint64_t>(row) * nb * 34 + 2 * nb +
-                                                            static_cast<uint64_t>(kb) * 32);
-    const uint8_t *xq8 = layout == 0
-        ? y + (static_cast<uint64_t>(j) * nb + kb) * kQ81Bytes + 4
-        : y + (static_cast<uint64_t>(kb / 4) * batch + j) * kD4Bytes + 16 + (kb % 4) * 32;
-    const int *xq = reinterpret_cast<const int *>(xq8);
-    int s = 0;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        const int a = static_cast<int>(wq[2 * t]) | (static_cast<int>(wq[2 * t + 1]) << 16);
-        s = __builtin_amdgcn_sdot4(a, xq[t], s, false);
-    }
-    out[i] = s;
-}
-
 // ---- fp32 -> bf16 (round to nearest even), for bf16 activations downstream ----
 __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float *__restrict__ in,
                                                           uint16_t *__restrict__ out, uint64_t n) {
@@ -99,118 +68,45 @@ __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float *__restric
     if (i < n) out[i] = float_to_bf16_bits(in[i]);
 }
 
-// ---- measurement helper: plain streaming read ---------------------------------
-// Every lane reads 16 bytes per trip, the grid covers the buffer with a
-// grid-stride loop; the xor of everything read goes to sink[0] only if it is a
-// value that cannot occur, so the loads cannot be optimised away.
-__global__ __launch_bounds__(256) void probe_read_kernel(const v4i *__restrict__ p, uint64_t n16,
-                                                         uint32_t *__restrict__ sink) {
-    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256;
-    uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
-    v4i a = {0, 0, 0, 0};
-#ifdef Q8MI_TRACE
-    const unsigned long long t_begin = __builtin_amdgcn_s_memrealtime();
-#endif
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        // streaming ("nt") loads, as the GEMV's weight loads
-        const v4i v0 = __builtin_nontemporal_load(p + i), v1 = __builtin_nontemporal_load(p + i + stride),
-                  v2 = __builtin_nontemporal_load(p + i + 2 * stride), v3 = __builtin_nontemporal_load(p + i + 3 * stride);
-        a.x ^= v0.x ^ v1.x ^ v2.x ^ v3.x;
-        a.y ^= v0.y ^ v1.y ^ v2.y ^ v3.y;
-        a.z ^= v0.z ^ v1.z ^ v2.z ^ v3.z;
-        a.w ^= v0.w ^ v1.w ^ v2.w ^ v3.w;
-    }
-    for (; i < n16; i += stride) {
-        const v4i v = p[i];
-        a.x ^= v.x; a.y ^= v.y; a.z ^= v.z; a.w ^= v.w;
-    }
-    if ((a.x ^ a.y ^ a.z ^ a.w) == 0x5a17c0de && (a.x & a.y) == 0x0badf00d) sink[0] = 1;
-#ifdef Q8MI_TRACE
-    // tuning build: the caller's sink holds 16 bytes per workgroup after its first 16
-    if (threadIdx.x == 0) {
-        unsigned long long *t = reinterpret_cast<unsigned long long *>(sink) + 2 + 2 * blockIdx.x;
-        t[0] = t_begin;
-        t[1] = __builtin_amdgcn_s_memrealtime() + (a.x == 0x7fffffff ? 1 : 0);
-    }
-#endif
-}
-
-// Plain copy, 16 bytes per lane per trip: a kernel whose HBM reads and writes are
-// both exactly `bytes`, used to calibrate memory-traffic counters.
-__global__ __launch_bounds__(256) void probe_copy_kernel(const v4i *__restrict__ src, v4i *__restrict__ dst,
-                                                         uint64_t n16) {
-    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256;
-    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
-}
-
-// ---- measurement helper: matrix-unit ceilings -----------------------------------
-// Four independent int8 MFMAs per round, optionally with NV independent scalar FMAs:
-// nothing else (no loads, no LDS), so the time is the issue rate of the two pipes.
-template <int NV>
-__global__ __launch_bounds__(256) void probe_mfma_kernel(int *__restrict__ out, uint32_t iters, float a, float b) {
-    v4i va = {static_cast<int>(threadIdx.x), 1, 2, 3}, vb = {4, 5, 6, static_cast<int>(threadIdx.x)};
-    v16i c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
-    float x[8];
+// ---- elementwise add: out = a + b (fp32), or bf16(f32(a) + f32(b)) rounded to nearest even ----
+// Four (fp32) or eight (bf16) elements per thread when the three pointers are 16-byte aligned.
+template <bool BF16>
+__global__ __launch_bounds__(256) void add_kernel(void *__restrict__ out_v, const void *a_v, const void *b_v, uint64_t n,
+                                                  bool vec) {
+    constexpr uint32_t kPer = BF16 ? 8 : 4;
+    const uint64_t i0 = (static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x) * kPer;
+    if (i0 >= n) return;
+    if constexpr (BF16) {
+        uint16_t *out = static_cast<uint16_t *>(out_v);
+        const uint16_t *a = static_cast<const uint16_t *>(a_v), *b = static_cast<const uint16_t *>(b_v);
+        if (vec && i0 + kPer <= n) {
+            const uint4 av = *reinterpret_cast<const uint4 *>(a + i0), bv = *reinterpret_cast<const uint4 *>(b + i0);
+            const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+            uint32_t r[4];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) x[k] = static_cast<float>(threadIdx.x + k);
-    for (uint32_t i = 0; i < iters; ++i) {
-        c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c0, 0, 0, 0);
-        c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c1, 0, 0, 0);
-        c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c2, 0, 0, 0);
-        c3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, c3, 0, 0, 0);
-#pragma unroll
-        for (int k = 0; k < NV; ++k) x[k % 8] = fmaf(x[k % 8], a, b);
+            for (int k = 0; k < 4; ++k) {
+                const float lo = bf16_bits_to_float(static_cast<uint16_t>(aw[k] & 0xffffu)) +
+                                 bf16_bits_to_float(static_cast<uint16_t>(bw[k] & 0xffffu));
+                const float hi = bf16_bits_to_float(static_cast<uint16_t>(aw[k] >> 16)) +
+                                 bf16_bits_to_float(static_cast<uint16_t>(bw[k] >> 16));
+                r[k] = static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
+            }
+            *reinterpret_cast<uint4 *>(out + i0) = make_uint4(r[0], r[1], r[2], r[3]);
+        } else {
+            for (uint64_t i = i0; i < n && i < i0 + kPer; ++i)
+                out[i] = float_to_bf16_bits(bf16_bits_to_float(a[i]) + bf16_bits_to_float(b[i]));
+        }
+    } else {
+        float *out = static_cast<float *>(out_v);
+        const float *a = static_cast<const float *>(a_v), *b = static_cast<const float *>(b_v);
+        if (vec && i0 + kPer <= n) {
+            const float4 av = *reinterpret_cast<const float4 *>(a + i0), bv = *reinterpret_cast<const float4 *>(b + i0);
+            *reinterpret_cast<float4 *>(out + i0) = make_float4(av.x + bv.x, av.y + bv.y, av.z + bv.z, av.w + bv.w);
+        } else {
+            for (uint64_t i = i0; i < n && i < i0 + kPer; ++i) out[i] = a[i] + b[i];
+        }
     }
-    int s = 0;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) s += c0[v] + c1[v] + c2[v] + c3[v];
-    float f = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) f += x[k];
-    out[blockIdx.x * 256 + threadIdx.x] = s + static_cast<int>(f);
 }
-
-// ---- synthetic inputs --------------------------------------------------------
-inline uint64_t splitmix64(uint64_t z) {
-    z += 0x9E3779B97F4A7C15ull;
-    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-    return z ^ (z >> 31);
-}
-
-inline uint64_t draw(uint64_t seed, uint64_t stream, uint64_t i) {
-    return splitmix64(splitmix64(seed * 0xD1342543DE82EF95ull + stream) + i);
-}
-
-// uniform in (0, 1): 53 random bits, never 0
-inline double unit(uint64_t bits) { return (static_cast<double>(bits >> 11) + 0.5) * (1.0 / 9007199254740992.0); }
-
-// standard normal from two independent draws (Box-Muller, cosine branch)
-inline double normal(uint64_t seed, uint64_t stream, uint64_t i) {
-    const double u1 = unit(draw(seed, stream, 2 * i));
-    const double u2 = unit(draw(seed, stream, 2 * i + 1));
-    return sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2);
-}
-
-template <typename F>
-void parallel_rows(uint64_t rows, int threads, F fn) {
-    if (threads < 1) threads = 1;
-    if (static_cast<uint64_t>(threads) > rows) threads = rows ? static_cast<int>(rows) : 1;
-    if (threads == 1) {
-        fn(0, rows);
-        return;
-    }
-    std::vector<std::thread> pool;
-    const uint64_t chunk = (rows + threads - 1) / threads;
-    for (int t = 0; t < threads; ++t) {
-        const uint64_t lo = chunk * t, hi = lo + chunk < rows ? lo + chunk : rows;
-        if (lo >= hi) break;
-        pool.emplace_back([=] { fn(lo, hi); });
-    }
-    for (auto &th : pool) th.join();
-}
-
-inline uint16_t f32_to_f16_host(float f) { return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); }
 
 }  // namespace
 }  // namespace q8mi
@@ -253,21 +149,6 @@ extern "C" int q8mi_repack_q8_0_split(const void *gguf_blocks, uint64_t rows, ui
     return check_launch("repack");
 }
 
-extern "C" int q8mi_block_dots(const uint8_t *weight, const void *y, int y_layout, uint32_t rows,
-                               uint32_t cols, uint32_t batch, const uint32_t *sample_row,
-                               const uint32_t *sample_j, const uint32_t *sample_kb, uint32_t n,
-                               int32_t *out, void *stream) {
-    (void)rows;
-    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "block_dots: cols %u not a multiple of 32", cols);
-    if (y_layout != 0 && y_layout != 1) return fail(Q8MI_REJECTED, "block_dots: unknown layout %d", y_layout);
-    if (y_layout == 1 && cols % 128 != 0) return fail(Q8MI_REJECTED, "block_dots: D4 needs cols %% 128 == 0");
-    if (n == 0) return Q8MI_OK;
-    block_dots_kernel<<<(n + 255) / 256, 256, 0, as_stream(stream)>>>(
-        weight, static_cast<const uint8_t *>(y), y_layout, cols / kQK, batch, sample_row, sample_j,
-        sample_kb, n, out);
-    return check_launch("block_dots");
-}
-
 extern "C" int q8mi_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, void *stream) {
     if (n == 0) return Q8MI_OK;
     const uint64_t grid = (n + 255) / 256;
@@ -276,91 +157,16 @@ extern "C" int q8mi_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, void
     return check_launch("f32_to_bf16");
 }
 
-extern "C" int q8mi_probe_read(const void *buf, uint64_t bytes, uint32_t wgs_per_cu, uint32_t *sink,
-                               void *stream) {
-    if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(buf) % 16 != 0)
-        return fail(Q8MI_REJECTED, "probe_read: buffer must be 16-byte aligned and sized");
-    if (wgs_per_cu == 0 || wgs_per_cu > 64) return fail(Q8MI_REJECTED, "probe_read: wgs_per_cu outside 1..64");
-    const uint32_t grid = static_cast<uint32_t>(device_cu_count()) * wgs_per_cu;
-    probe_read_kernel<<<grid, 256, 0, as_stream(stream)>>>(static_cast<const v4i *>(buf), bytes / 16, sink);
-    return check_launch("probe_read");
-}
-
-extern "C" int q8mi_probe_copy(const void *src, void *dst, uint64_t bytes, void *stream) {
-    if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0)
-        return fail(Q8MI_REJECTED, "probe_copy: buffers must be 16-byte aligned and sized");
-    const uint32_t grid = static_cast<uint32_t>(device_cu_count()) * 8;
-    probe_copy_kernel<<<grid, 256, 0, as_stream(stream)>>>(static_cast<const v4i *>(src), static_cast<v4i *>(dst),
-                                                           bytes / 16);
-    return check_launch("probe_copy");
-}
-
-extern "C" size_t q8mi_probe_mfma_sink_bytes(void) {
-    return static_cast<size_t>(device_cu_count()) * 2 * 256 * sizeof(int32_t);
-}
-
-extern "C" int q8mi_probe_mfma(int with_rescale, uint32_t iters, int32_t *sink, uint64_t *ops_out, void *stream) {
-    if (sink == nullptr || iters == 0) return fail(Q8MI_REJECTED, "probe_mfma: null sink or zero rounds");
-    const uint32_t grid = static_cast<uint32_t>(device_cu_count()) * 2;
-    if (with_rescale)
-        probe_mfma_kernel<128><<<grid, 256, 0, as_stream(stream)>>>(sink, iters, 1.0001f, 0.5f);
+extern "C" int q8mi_add(void *out, const void *a, const void *b, uint64_t n, int is_bf16, void *stream) {
+    if (n == 0) return Q8MI_OK;
+    if (out == nullptr || a == nullptr || b == nullptr) return fail(Q8MI_REJECTED, "add: null pointer");
+    const uint64_t per = is_bf16 ? 8 : 4;
+    const uint64_t grid = ((n + per - 1) / per + 255) / 256;
+    if (grid > 0x7fffffffull) return fail(Q8MI_REJECTED, "add: too many elements for one launch");
+    const bool vec = (reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16 == 0;
+    if (is_bf16)
+        add_kernel<true><<<static_cast<uint32_t>(grid), 256, 0, as_stream(stream)>>>(out, a, b, n, vec);
     else
-        probe_mfma_kernel<0><<<grid, 256, 0, as_stream(stream)>>>(sink, iters, 1.0001f, 0.5f);
-    if (ops_out) *ops_out = static_cast<uint64_t>(grid) * 4 * iters * 4 * 2ull * 32 * 32 * 32;
-    return check_launch("probe_mfma");
-}
-
-extern "C" int q8mi_synth_f32(float *out, uint64_t rows, uint64_t cols, uint64_t seed, int kind,
-                              float scale, uint32_t outlier_ppm, float outlier_gain, int threads) {
-    if (kind != 0 && kind != 1) return fail(Q8MI_REJECTED, "synth_f32: unknown kind %d", kind);
-    parallel_rows(rows, threads, [=](uint64_t lo, uint64_t hi) {
-        for (uint64_t r = lo; r < hi; ++r) {
-            for (uint64_t c = 0; c < cols; ++c) {
-                const uint64_t i = r * cols + c;
-                double v;
-                if (kind == 0) {
-                    v = normal(seed, 0, i);
-                } else {
-                    // Student-t(3) = Z / sqrt(chi2_3 / 3); unit variance after / sqrt(3)
-                    const double z = normal(seed, 0, i);
-                    const double a = normal(seed, 1, i), b = normal(seed, 2, i), d = normal(seed, 3, i);
-                    const double chi2 = a * a + b * b + d * d;
-                    v = z / sqrt(chi2 / 3.0) / 1.7320508075688772;
-                    if (outlier_ppm != 0 && draw(seed, 4, c) % 1000000ull < outlier_ppm) v *= outlier_gain;
-                }
-                out[i] = static_cast<float>(v * scale);
-            }
-        }
-    });
-    return Q8MI_OK;
-}
-
-extern "C" int q8mi_synth_q8_0_weight(uint8_t *split_out, uint64_t rows, uint64_t cols, uint64_t seed,
-                                      float sigma, int threads) {
-    if (cols % kQK != 0) return fail(Q8MI_REJECTED, "synth_q8_0_weight: cols %llu not a multiple of 32", (unsigned long long)cols);
-    const uint64_t nb = cols / kQK;
-    parallel_rows(rows, threads, [=](uint64_t lo, uint64_t hi) {
-        float blk[kQK];
-        for (uint64_t r = lo; r < hi; ++r) {
-            uint8_t *d_plane = split_out + r * nb * 34;
-            int8_t *q_plane = reinterpret_cast<int8_t *>(d_plane + 2 * nb);
-            for (uint64_t kb = 0; kb < nb; ++kb) {
-                float amax = 0.0f;
-                for (int t = 0; t < kQK; ++t) {
-                    blk[t] = static_cast<float>(normal(seed, 0, r * cols + kb * kQK + t) * sigma);
-                    amax = fmaxf(amax, fabsf(blk[t]));
-                }
-                const float d = amax / 127.0f;
-                const float d_inv = d == 0.0f ? 0.0f : 1.0f / d;
-                const uint16_t hd = f32_to_f16_host(d);
-                memcpy(d_plane + 2 * kb, &hd, 2);
-                for (int t = 0; t < kQK; ++t) {
-                    long q = lrintf(blk[t] * d_inv);
-                    q = q < -127 ? -127 : (q > 127 ? 127 : q);
-                    q_plane[kb * kQK + t] = static_cast<int8_t>(q);
-                }
-            }
-        }
-    });
-    return Q8MI_OK;
+        add_kernel<false><<<static_cast<uint32_t>(grid), 256, 0, as_stream(stream)>>>(out, a, b, n, vec);
+    return check_launch("add");
 }

@@ -325,35 +325,21 @@ int launch_inst(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t nb, 
                 hipStream_t stream) {
     auto kern = lm_head_kernel<M, THREADS, XMODE>;
     const uint32_t lds = x_bytes + (THREADS / kWave) * kParkFloats * 4;
-    static thread_local uint32_t cached_lds = 0xffffffffu;
-    static thread_local int cached_occ = 0;
-    if (cached_lds != lds) {
-        if (lds > 64u * 1024u &&
-            hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(lds)) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8MI_LAUNCH_ERROR, "lm_head: cannot reserve %u bytes of LDS", lds);
-        }
-        int occ = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, THREADS, lds) != hipSuccess || occ < 1) {
-            (void)hipGetLastError();
-            occ = 1;
-        }
-        cached_occ = occ;
-        cached_lds = lds;
-    }
+    static KernelGeometry geometry;
+    constexpr uint32_t kDynLimit = kLdsLimit - THREADS * 8;   // static LDS: the argmax tree
+    if (lds > kDynLimit || !geometry.grant(reinterpret_cast<const void *>(kern), kDynLimit))
+        return fail(Q8MI_LAUNCH_ERROR, "lm_head: cannot reserve %u bytes of LDS", lds);
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     const uint32_t units = (rows + RowsPerUnit<M>::value - 1) / RowsPerUnit<M>::value;
-    const GemvTuning tune = gemv_tuning();
-    uint32_t max_per_cu = static_cast<uint32_t>(cached_occ);
-    if (tune.wgs_per_cu > 0 && static_cast<uint32_t>(tune.wgs_per_cu) < max_per_cu) max_per_cu = tune.wgs_per_cu;
+    uint32_t max_per_cu = geometry.workgroups_per_cu(kern, THREADS, lds);
+    if (max_per_cu > kGemvWgsPerCu) max_per_cu = kGemvWgsPerCu;
     while (max_per_cu > 1 && cus * max_per_cu > kMaxPartials) --max_per_cu;   // one partial per workgroup
     const uint32_t grid = pick_grid(units, (nb * 2 + 127) / 128, M, THREADS / kWave, cus, max_per_cu);
     if (grid > kMaxPartials)
         return fail(Q8MI_REJECTED, "lm_head: %u rows need %u workgroups, more than the %u partials", rows, grid,
                     kMaxPartials);
     *grid_out = grid;
-    kern<<<grid, THREADS, lds, stream>>>(w, y, rows, nb, partial, logits, stride_logits, tune.interleave, x_bytes);
+    kern<<<grid, THREADS, lds, stream>>>(w, y, rows, nb, partial, logits, stride_logits, kGemvInterleave, x_bytes);
     return check_launch("lm_head");
 }
 
@@ -373,18 +359,12 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
     if (grid > kMaxPartials) grid = kMaxPartials;
     const uint32_t lds = x_bytes + (THREADS / kWave) * 2 * mfma_park_floats_per_unit(MG) * 4;
     if (lds > kDynLimit) return fail(Q8MI_REJECTED, "lm_head (matrix-core variant): the activations do not fit LDS");
-    static thread_local bool granted = false;
-    if (lds > 64u * 1024u && !granted) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(kDynLimit)) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8MI_LAUNCH_ERROR, "lm_head: cannot reserve %u bytes of LDS", lds);
-        }
-        granted = true;
-    }
+    static KernelGeometry geometry;
+    if (!geometry.grant(reinterpret_cast<const void *>(kern), kDynLimit))
+        return fail(Q8MI_LAUNCH_ERROR, "lm_head: cannot reserve %u bytes of LDS", lds);
     *grid_out = grid;
     kern<<<grid, THREADS, lds, stream>>>(w, y, rows, nb, batch, partial, logits, stride_logits,
-                                         gemv_tuning().interleave, x_bytes);
+                                         kGemvInterleave, x_bytes);
     return check_launch("lm_head");
 }
 
@@ -394,7 +374,7 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
 // faster up to 6 rows (measured: 237..257 us against 245..265 us at 4..6 rows, 296 against 265 at 8).
 bool lm_head_uses_mfma(uint32_t rows, uint32_t nb, uint32_t batch) {
     const uint32_t mg = (batch + 3) / 4;
-    if (batch < static_cast<uint32_t>(gemv_tuning().mfma_from)) return false;
+    if (batch < kMfmaFromBatch) return false;
     if (mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u > kLdsLimit - 256) return false;
     return rows <= 65536u || batch >= 7;
 }
@@ -405,13 +385,8 @@ int launch_lm_head(const uint8_t *w, const uint8_t *y, uint32_t rows, uint32_t n
     const uint32_t xb = x_lds_bytes(nb, M);
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
     const uint32_t tree_256 = 256 * 8, tree_1024 = 1024 * 8;   // static LDS of the argmax tree
-    const int forced = gemv_tuning().threads;
     if (reinterpret_cast<uintptr_t>(y) % 16 != 0)   // the LDS staging loads 16 bytes at a time
         return launch_inst<M, 256, kXGlobal>(w, y, rows, nb, 0, partial, logits, stride_logits, grid_out, stream);
-    if (forced == 256 && xb + park_256 + tree_256 <= kLdsLimit)
-        return launch_inst<M, 256, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
-    if (forced == 1024 && xb + park_1024 + tree_1024 <= kLdsLimit)
-        return launch_inst<M, 1024, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
     if (xb + park_256 + tree_256 <= 76u * 1024u)
         return launch_inst<M, 256, kXLds>(w, y, rows, nb, xb, partial, logits, stride_logits, grid_out, stream);
     if (xb + park_1024 + tree_1024 <= kLdsLimit)
@@ -431,24 +406,12 @@ extern "C" size_t q8mi_lm_head_scratch_bytes(uint32_t rows, uint32_t cols, uint3
     return static_cast<size_t>(batch) * kMaxPartials * sizeof(q8mi_argmax_pair);
 }
 
-extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, uint32_t rows,
-                                          uint32_t cols, uint32_t batch, const int32_t *drafts,
-                                          int drafts_on_device, int32_t eos, q8mi_argmax_pair *row_out,
-                                          int32_t *accept_out, float *logits, uint32_t stride_logits,
-                                          void *scratch, void *stream) {
-    if (cols % kQK != 0 || cols == 0)
-        return fail(Q8MI_REJECTED, "lm_head: cols %u not a positive multiple of 32", cols);
-    if ((cols / kQK) % 8 != 0)
-        return fail(Q8MI_REJECTED, "lm_head: cols %u not a multiple of 256 (unaligned planes)", cols);
-    if (batch == 0 || batch > Q8MI_MAX_GEMV_BATCH)
-        return fail(Q8MI_REJECTED, "lm_head: batch %u outside 1..8", batch);
-    if (rows == 0 || rows > 0x7fffffffu) return fail(Q8MI_REJECTED, "lm_head: rows %u out of range", rows);
-    if (batch > 1 && drafts == nullptr) return fail(Q8MI_REJECTED, "lm_head: drafts missing");
-    if (reinterpret_cast<uintptr_t>(weight) % 16 != 0)
-        return fail(Q8MI_REJECTED, "lm_head: weight pointer not 16-byte aligned");
+static int lm_head_run(const uint8_t *weight, const void *y, uint32_t rows, uint32_t cols, uint32_t batch,
+                       const int32_t *drafts, int drafts_on_device, int32_t eos, q8mi_argmax_pair *row_out,
+                       int32_t *accept_out, float *logits, uint32_t stride_logits, q8mi_argmax_pair *partial,
+                       void *stream) {
     const uint32_t nb = cols / kQK;
     uint32_t grid = 0;
-    auto *partial = static_cast<q8mi_argmax_pair *>(scratch);
     const auto *yb = static_cast<const uint8_t *>(y);
     hipStream_t s = as_stream(stream);
     int rc = Q8MI_REJECTED;
@@ -480,4 +443,28 @@ extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, 
     }
     lm_head_finalize_kernel<<<1, kMaxPartials, 0, s>>>(partial, grid, batch, dv, ddev, eos, row_out, accept_out);
     return check_launch("lm_head finalize");
+}
+
+static int lm_head_gate(const uint8_t *weight, uint32_t rows, uint32_t cols, uint32_t batch, const int32_t *drafts) {
+    if (cols % kQK != 0 || cols == 0)
+        return fail(Q8MI_REJECTED, "lm_head: cols %u not a positive multiple of 32", cols);
+    if ((cols / kQK) % 8 != 0)
+        return fail(Q8MI_REJECTED, "lm_head: cols %u not a multiple of 256 (unaligned planes)", cols);
+    if (batch == 0 || batch > Q8MI_MAX_GEMV_BATCH)
+        return fail(Q8MI_REJECTED, "lm_head: batch %u outside 1..8", batch);
+    if (rows == 0 || rows > 0x7fffffffu) return fail(Q8MI_REJECTED, "lm_head: rows %u out of range", rows);
+    if (batch > 1 && drafts == nullptr) return fail(Q8MI_REJECTED, "lm_head: drafts missing");
+    if (reinterpret_cast<uintptr_t>(weight) % 16 != 0)
+        return fail(Q8MI_REJECTED, "lm_head: weight pointer not 16-byte aligned");
+    return Q8MI_OK;
+}
+
+extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, uint32_t rows,
+                                          uint32_t cols, uint32_t batch, const int32_t *drafts,
+                                          int drafts_on_device, int32_t eos, q8mi_argmax_pair *row_out,
+                                          int32_t *accept_out, float *logits, uint32_t stride_logits,
+                                          void *scratch_arg, void *stream) {
+    if (int rc = lm_head_gate(weight, rows, cols, batch, drafts)) return rc;
+    return lm_head_run(weight, y, rows, cols, batch, drafts, drafts_on_device, eos, row_out, accept_out, logits,
+                       stride_logits, static_cast<q8mi_argmax_pair *>(scratch_arg), stream);
 }

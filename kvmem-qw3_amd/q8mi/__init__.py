@@ -47,7 +47,7 @@ SIGNATURES = {
     "q8mi_gemm": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_gemm_medium": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_f32_to_bf16": (_int, [_vp, _vp, _u64, _vp]),
-    "q8mi_block_dots": (_int, [_u8p, _vp, _int, _u32, _u32, _u32, _vp, _vp, _vp, _u32, _vp, _vp]),
+    "q8mi_add": (_int, [_vp, _vp, _vp, _u64, _int, _vp]),
     "q8mi_get_row": (_int, [_u8p, _u64, _u64, _u64, _vp, _int, _vp]),
     "q8mi_get_row_from_argmax": (_int, [_u8p, _vp, _u32, _u64, _u64, _vp, _vp]),
     "q8mi_get_rows": (_int, [_u8p, _vp, _u32, _u64, _u64, _vp, _int, _vp]),
@@ -60,9 +60,6 @@ SIGNATURES = {
                                           _u32, _vp, _vp]),
     "q8mi_repack_q8_0_split_host": (_int, [_vp, _u64, _u64, _vp]),
     "q8mi_repack_q8_0_split": (_int, [_vp, _u64, _u64, _vp, _vp]),
-    "q8mi_probe_read": (_int, [_vp, _u64, _u32, _vp, _vp]),
-    "q8mi_probe_mfma": (_int, [_int, _u32, _vp, C.POINTER(C.c_uint64), _vp]),
-    "q8mi_probe_mfma_sink_bytes": (C.c_size_t, []),
     "q8mi_qgemv": (_int, [_vp, _vp, _u32, _vp, _int, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_qgemv_add": (_int, [_vp, _vp, _u32, _vp, _int, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_qgemv_silu_mul": (_int, [_vp, _vp, _vp, _u32, _vp, _u32, _u32, _u32, _u32, _vp]),
@@ -74,9 +71,6 @@ SIGNATURES = {
     "q8mi_nqgemv_silu_mul": (_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _u32, _u32, _u32, _vp]),
     "q8mi_nqgemv_fanout4": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,
                                    _u32, _u32, _u32, _vp]),
-    "q8mi_probe_copy": (_int, [_vp, _vp, _u64, _vp]),
-    "q8mi_synth_f32": (_int, [_vp, _u64, _u64, _u64, _int, C.c_float, _u32, C.c_float, _int]),
-    "q8mi_synth_q8_0_weight": (_int, [_vp, _u64, _u64, _u64, C.c_float, _int]),
 }
 
 _lib = None

@@ -60,10 +60,23 @@ def synchronize():
 
 
 def device_name():
-    # hipDeviceGetName(char*, int, hipDevice_t)
-    buf = C.create_string_buffer(256)
-    check(rt().hipDeviceGetName(buf, C.c_int(256), C.c_int(0)), "hipDeviceGetName")
-    return buf.value.decode()
+    """Marketing name of device 0, with its architecture name when the runtime reports one
+    (hipGetDeviceProperties: `name` is the first field of the struct, `gcnArchName` a later one that
+    is found by its "gfx" prefix, so no struct layout is assumed)."""
+    buf = C.create_string_buffer(8192)
+    fn = getattr(rt(), "hipGetDevicePropertiesR0600", None) or rt().hipGetDeviceProperties
+    name, arch = "", ""
+    if fn(buf, C.c_int(0)) == 0:
+        raw = buf.raw
+        name = raw[:256].split(b"\0", 1)[0].decode(errors="replace")
+        at = raw.find(b"gfx", 256)
+        if at >= 0:
+            arch = raw[at:at + 64].split(b"\0", 1)[0].decode(errors="replace")
+    if not name:
+        short = C.create_string_buffer(256)
+        if rt().hipDeviceGetName(short, C.c_int(256), C.c_int(0)) == 0:
+            name = short.value.decode(errors="replace")
+    return " ".join(x for x in (name, arch) if x) or "unknown HIP device"
 
 
 class DeviceBuffer:

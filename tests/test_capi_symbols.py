@@ -31,11 +31,26 @@ def test_library_exports_every_declared_symbol():
     assert lib.q8mi_abi_version() == 1
 
 
+def test_instruments_live_in_their_own_library():
+    """Input generators, the block-dot checker and the ceiling probes are not part of the product:
+    libq8mi.so exports none of them, libq8mi_support.so exports exactly what its header declares."""
+    import q8mi_support
+    out = subprocess.run(["nm", "-D", "--defined-only", q8mi.LIB_PATH], capture_output=True, text=True).stdout
+    assert not re.findall(r" T \w*(?:probe|synth|block_dots)\w*", out)
+    text = open(os.path.join(ROOT, "tests", "q8mi_support", "q8mi_support.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(q8sup_[a-z0-9_]+)\s*\(", text)))
+    assert declared == sorted(q8mi_support.SIGNATURES)
+    q8mi_support.lib()
+    out = subprocess.run(["nm", "-D", "--defined-only", q8mi_support.LIB_PATH], capture_output=True, text=True).stdout
+    assert set(re.findall(r" T (q8sup_[a-z0-9_]+)", out)) == set(declared)
+
+
 def test_host_side_entry_points_without_gpu(oracle):
     """Size helpers, the host repack and the synthetic generator run on the CPU."""
     import ctypes as C
     import numpy as np
-    from q8mi import synth
+    import q8mi_support as synth
     L = q8mi.lib()
     assert L.q8mi_q8_1_scratch_bytes(8, 17408) == 8 * 544 * 36
     assert L.q8mi_q8_1_d4_scratch_bytes(2048, 5120) == 2048 * 40 * 144

@@ -86,6 +86,7 @@ def test_oracle_argmax_and_accept(oracle, fx):
 @pytest.mark.gpu
 def test_gpu_formats_and_dots(gpu, fx):
     from gpu_common import NULL, dev, quantize_d4, quantize_q8_1
+    import q8mi_support as synth
     from q8mi import hip, ok
     L = gpu.lib()
     split = np.empty_like(fx["w_split"])
@@ -105,7 +106,7 @@ def test_gpu_formats_and_dots(gpu, fx):
     sr, sj, sk = (dev(a.reshape(-1).astype(np.uint32)) for a in (rr, jj, kk))
     for layout, ybuf, skey in ((0, dy, "dots_q8_1"), (1, dy4, "dots_d4")):
         out = hip.DeviceBuffer(4 * n)
-        ok(L.q8mi_block_dots(dsplit.ptr, ybuf.ptr, layout, ROWS, COLS, BATCH, sr.ptr, sj.ptr, sk.ptr, n, out.ptr,
+        ok(synth.lib().q8sup_block_dots(dsplit.ptr, ybuf.ptr, layout, ROWS, COLS, BATCH, sr.ptr, sj.ptr, sk.ptr, n, out.ptr,
                              NULL), "block_dots")
         hip.synchronize()
         assert np.array_equal(out.download(np.int32, n).reshape(BATCH, ROWS, -1), fx[skey])

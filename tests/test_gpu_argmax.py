@@ -6,7 +6,8 @@ import pytest
 
 import q8mi
 from gpu_common import NULL, assert_close_fp32, dev, quantize_q8_1
-from q8mi import hip, ok, synth
+from q8mi import hip, ok
+import q8mi_support as synth
 
 pytestmark = pytest.mark.gpu
 

@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 from gpu_common import quantize_d4, quantize_q8_1
-from q8mi import synth
+import q8mi_support as synth
 
 pytestmark = pytest.mark.gpu
 
