@@ -13,6 +13,22 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionfinish(session, exitstatus):
+    """GPU runs leave what the fp32 comparisons measured (largest relative error per check family
+    and how many outputs needed the sum|t_kb| term of the bound) beside the run's other output."""
+    try:
+        import gpu_common
+    except Exception:
+        return
+    if not gpu_common.TOLERANCE_STATS:
+        return
+    import json
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "tolerance_stats.json"), "w") as f:
+        json.dump(gpu_common.TOLERANCE_STATS, f, indent=1, sort_keys=True)
+
+
 @pytest.fixture(scope="session")
 def oracle():
     """The CPU oracle (built on demand from oracle/q8_oracle.c)."""

@@ -1,13 +1,14 @@
 """GPU parity at the model's own shapes: the decode GEMV set of one layer exactly as bench.py times
 it (QKV fan-out 5120 -> 6144 + 1024 + 1024, O 6144 -> 5120 with residual, gate/up 5120 -> 17408 SwiGLU,
-down 17408 -> 5120 with residual), at M = 1 (quantizer inside the launches), 2, 4 and 8, against the
+down 17408 -> 5120 with residual), at M = 1 (quantizer inside the launches), 2, 4, 6 and 8, against the
 CPU oracle."""
 import numpy as np
 import pytest
 
 import bench
 from gpu_common import assert_close_fp32
-from q8mi import hip, synth
+import q8mi_support as synth
+from q8mi import hip
 
 pytestmark = pytest.mark.gpu
 
@@ -23,7 +24,7 @@ def layer(gpu):
     return dev_layer, host
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 8])
+@pytest.mark.parametrize("m", [1, 2, 4, 6, 8])
 def test_decode_layer_at_model_shapes(gpu, oracle, layer, m):
     dev_layer, host = layer
     step = bench.DecodeStep(gpu, hip, m, seed=40 + m)

@@ -4,7 +4,8 @@ import pytest
 
 import q8mi
 from gpu_common import NULL, assert_close_fp32, dev, quantize_d4, quantize_q8_1
-from q8mi import hip, ok, synth
+from q8mi import hip, ok
+import q8mi_support as synth
 
 pytestmark = pytest.mark.gpu
 
@@ -25,7 +26,7 @@ def d4_block_dots(oracle, dw, w, dy, y, rows, cols, batch, seed, n=2048):
     sk = rng.integers(0, cols // 32, n, dtype=np.uint32)
     out = hip.DeviceBuffer(4 * n)
     a, b, c = dev(sr), dev(sj), dev(sk)
-    ok(q8mi.lib().q8mi_block_dots(dw.ptr, dy.ptr, 1, rows, cols, batch, a.ptr, b.ptr, c.ptr, n, out.ptr, NULL),
+    ok(synth.lib().q8sup_block_dots(dw.ptr, dy.ptr, 1, rows, cols, batch, a.ptr, b.ptr, c.ptr, n, out.ptr, NULL),
        "block_dots")
     hip.synchronize()
     got = out.download(np.int32)
@@ -253,8 +254,6 @@ def test_gemm_small_batches_stream_the_weights(gpu, oracle, rows, cols, batch):
     """Batches of up to 16 rows on D4 activations are served by the weight-streaming matrix-core
     GEMV (when the activations fit LDS), 17..32 by the narrowest ring tile: same contract as the
     tile kernel."""
-    if rows == 5120 and batch not in (4, 9, 16, 29):
-        pytest.skip("big shape: three batches only")
     w = synth.q8_0_weight(rows, cols, seed=rows * 5 + cols)
     x = synth.normal(batch, cols, seed=batch * 3 + cols)
     dw = dev(w)
@@ -332,8 +331,6 @@ def test_gemm_medium_batches(gpu, oracle, rows, cols, batch):
     """Batches too small to fill the chip with 128 x 128 tiles run 32-row tiles behind a ring of
     LDS stages, 32, 64 or 128 activation rows wide, the narrow ones with K split over the waves:
     rows and batch ragged against every tile width, K shorter and much longer than the ring."""
-    if rows == 5120 and batch not in (33, 64, 128):
-        pytest.skip("big shape: three batches only")
     w = synth.q8_0_weight(rows, cols, seed=rows * 3 + cols)
     x = synth.normal(batch, cols, seed=batch * 17 + cols)
     x[batch // 2, :128] = 0.0
