@@ -500,6 +500,25 @@ DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized,
     return launch_status("hip rms_norm_q8_0_matmul_fanout");
 }
 
+// src/kernels_cuda.cu:14818-14862: elementwise out = a + b over the first `count` elements; the
+// three tensors are all fp32 or all bf16
+DeviceStatus HipQ8Backend::add(DeviceTensor &out, const DeviceTensor &a, const DeviceTensor &b) {
+    return add_n(out, a, b, out.count);
+}
+
+DeviceStatus HipQ8Backend::add_n(DeviceTensor &out, const DeviceTensor &a, const DeviceTensor &b, uint64_t count) {
+    auto &o = T(out);
+    const auto &aa = T(a), &bb = T(b);
+    if (count > o.count || count > aa.count || count > bb.count) return {false, "hip add_n count exceeds tensor size"};
+    if (o.is_bf16() || aa.is_bf16() || bb.is_bf16()) {
+        if (!o.is_bf16()) return {false, "hip add_n BF16 input with FP32 output"};
+        if (!aa.is_bf16()) return {false, "hip add_n BF16 output with FP32 lhs"};
+        if (!bb.is_bf16()) return {false, "hip add_n BF16 output with FP32 rhs"};
+    }
+    if (q8mi_add(o.ptr, aa.ptr, bb.ptr, count, o.is_bf16() ? 1 : 0, stream_) != Q8MI_OK) return failed("add");
+    return launch_status("hip add");
+}
+
 // src/kernels_cuda.cu:11919-11957: in-place residual add for batch <= 8, else matmul + add
 DeviceStatus HipQ8Backend::q8_0_matmul_add(DeviceTensor &out, const DeviceTensor &residual, DeviceTensor &matmul_tmp,
                                            const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
@@ -511,9 +530,9 @@ DeviceStatus HipQ8Backend::q8_0_matmul_add(DeviceTensor &out, const DeviceTensor
                       batch >= 1 && batch <= 8 && in_stride == cols &&
                       o.count >= static_cast<uint64_t>(batch) * out_stride;
     if (!fast) {
-        (void)matmul_tmp;
-        return {false, "q8_0_matmul_add: only the in-place batch <= 8 form is on this path "
-                       "(the caller's two-step fallback covers the rest)"};
+        // include/qw3/device_backend.hpp:529-540: the matmul into the temporary, then out = residual + tmp
+        if (auto st = q8_0_matmul(matmul_tmp, weight, x, batch, in_stride, out_stride); !st.ok) return st;
+        return add(out, residual, matmul_tmp);
     }
     if (auto st = quantize_q8_1(T(x).f32(), batch, cols, in_stride); !st.ok) return st;
     const bool ok = o.is_bf16()

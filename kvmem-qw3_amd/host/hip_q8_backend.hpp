@@ -108,6 +108,10 @@ public:
     DeviceStatus q8_0_matmul_fanout(DeviceTensor *const *outs, const DeviceWeight *const *weights,
                                     const uint32_t *out_strides, uint32_t n, const DeviceTensor &x, uint32_t batch,
                                     uint32_t in_stride);
+    // elementwise out = a + b (include/qw3/device_backend.hpp:639-646): what the batched
+    // q8_0_matmul_add ends with when its fused in-place form does not apply
+    DeviceStatus add(DeviceTensor &out, const DeviceTensor &a, const DeviceTensor &b);
+    DeviceStatus add_n(DeviceTensor &out, const DeviceTensor &a, const DeviceTensor &b, uint64_t count);
     DeviceStatus q8_0_matmul_add(DeviceTensor &out, const DeviceTensor &residual, DeviceTensor &matmul_tmp,
                                  const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
                                  uint32_t in_stride, uint32_t out_stride);
@@ -168,8 +172,7 @@ public:
 
     // Format-neutral forwards with the reference's default bodies
     // (include/qw3/device_backend.hpp:541-607): the executor calls these; for Q8_0
-    // weights they are the q8_0_* operators.  linear_matmul_add is left to the base
-    // class there (it needs the backend's elementwise add, which is outside this path).
+    // weights they are the q8_0_* operators.
     DeviceStatus linear_get_row(DeviceTensor &out, const DeviceWeight &weight, uint64_t row) {
         return q8_0_get_row(out, weight, row);
     }
@@ -180,6 +183,13 @@ public:
     DeviceStatus linear_get_rows_batch(DeviceTensor &out, const DeviceWeight &weight, const uint64_t *rows,
                                        uint32_t batch) {
         return q8_0_get_rows_batch(out, weight, rows, batch);
+    }
+    // include/qw3/device_backend.hpp:609-622: linear_matmul into the temporary, then add
+    DeviceStatus linear_matmul_add(DeviceTensor &out, const DeviceTensor &residual, DeviceTensor &matmul_tmp,
+                                   const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
+                                   uint32_t in_stride, uint32_t out_stride) {
+        if (auto st = q8_0_matmul(matmul_tmp, weight, x, batch, in_stride, out_stride); !st.ok) return st;
+        return add(out, residual, matmul_tmp);
     }
     DeviceStatus linear_matvec(DeviceTensor &out, const DeviceWeight &weight, const DeviceTensor &x) {
         return q8_0_matvec(out, weight, x);

@@ -368,12 +368,83 @@ void case_matmul(qw3::HipQ8Backend &b) {
         ok = ok && close_fp32(download_f32(b, *acc), ref, mag, nb, wa.rows, wa.rows, d);
         report("matmul_add_inplace_batch3", ok, d);
 
-        // forms the backend declines, as the reference does, so that the caller's fallback runs
+        // out of place at batch 3 (no fused form): matmul into the temporary, then out = residual + tmp
+        {
+            auto other = b.tensor_f32(static_cast<size_t>(nb) * wa.rows, "other");
+            auto tmp3 = b.tensor_f32(static_cast<size_t>(nb) * wa.rows, "tmp3");
+            auto res = upload_f32(b, base);
+            ok = require(b.q8_0_matmul_add(*other, *res, *tmp3, *da, *dx, nb, cols, wa.rows), "matmul_add out of place");
+            oracle_linear(wa, x.data(), nb, cols, wa.rows, ref, mag);
+            for (size_t i = 0; i < ref.size(); ++i) { ref[i] = base[i] + ref[i]; mag[i] += std::fabs(base[i]); }
+            ok = ok && close_fp32(download_f32(b, *other), ref, mag, nb, wa.rows, wa.rows, d);
+            ok = ok && download_f32(b, *res) == base;    // the residual is left alone
+            report("matmul_add_out_of_place_batch3", ok, d);
+        }
+        // forms the backend declines, as the reference does
         auto other = b.tensor_f32(static_cast<size_t>(nb) * wa.rows, "other");
-        ok = !b.q8_0_matmul_add(*other, *acc, *tmp, *da, *dx, nb, cols, wa.rows).ok;
-        ok = ok && !b.q8_0_matmul_silu_mul(*other, *da, *da, *dx, nb, cols, wa.rows).ok;
+        ok = !b.q8_0_matmul_silu_mul(*other, *da, *da, *dx, nb, cols, wa.rows).ok;
         ok = ok && b.weight_q8_0(wa.gguf.data(), 4, 40, "bad") == nullptr;
+        ok = ok && !b.add_n(*other, *other, *other, other->count + 1).ok;
         report("declined_forms", ok);
+    }
+}
+
+// Batched q8_0_matmul_add beyond the fused in-place form (src/kernels_cuda.cu:11919-11957 falls back to
+// include/qw3/device_backend.hpp:529-540: q8_0_matmul into matmul_tmp, then add): batch 9, 64 and 2048,
+// in place (out == residual) and out of place, fp32; and bf16 tensors at batch 64.
+void case_matmul_add_batched(qw3::HipQ8Backend &b) {
+    std::string d;
+    const uint32_t rows = 384, cols = 1024;
+    const HostWeight w = make_weight(rows, cols, 141);
+    auto dw = b.weight_q8_0(w.gguf.data(), rows, cols, "w");
+    for (uint32_t batch : {9u, 64u, 2048u}) {
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 142 + batch);
+        const auto base = normal_vec(static_cast<size_t>(batch) * rows, 143 + batch);
+        auto dx = upload_f32(b, x);
+        std::vector<float> prod, lin, mag;
+        oracle_gemm_d4(w, x.data(), batch, prod);                  // what q8_0_matmul leaves in the temporary
+        oracle_linear(w, x.data(), batch, cols, rows, lin, mag);   // magnitudes only
+        std::vector<float> want(prod.size());
+        for (size_t i = 0; i < prod.size(); ++i) { want[i] = base[i] + prod[i]; mag[i] += std::fabs(base[i]); }
+        for (int in_place = 0; in_place < 2; ++in_place) {
+            auto res = upload_f32(b, base);
+            auto tmp = b.tensor_f32(static_cast<size_t>(batch) * rows, "tmp");
+            auto other = b.tensor_f32(static_cast<size_t>(batch) * rows, "out");
+            qw3::DeviceTensor &out = in_place ? *res : *other;
+            bool ok = require(b.q8_0_matmul_add(out, *res, *tmp, *dw, *dx, batch, cols, rows), "matmul_add batched");
+            ok = ok && close_fp32(download_f32(b, out), want, mag, batch, rows, rows, d);
+            if (!in_place) ok = ok && download_f32(b, *res) == base;
+            report(("matmul_add_batch" + std::to_string(batch) + (in_place ? "_in_place" : "_out_of_place")).c_str(), ok, d);
+        }
+    }
+    // bf16 tensors: the temporary is the product rounded to bf16, the sum is rounded again
+    {
+        const uint32_t batch = 64;
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 151);
+        auto dx = upload_f32(b, x);
+        std::vector<float> prod;
+        oracle_gemm_d4(w, x.data(), batch, prod);
+        const auto basef = normal_vec(static_cast<size_t>(batch) * rows, 152);
+        std::vector<uint16_t> base(basef.size());
+        for (size_t i = 0; i < base.size(); ++i) base[i] = q8o_f32_to_bf16(basef[i]);
+        auto res = b.tensor_bf16(base.size(), "res"), tmp = b.tensor_bf16(base.size(), "tmp"), out = b.tensor_bf16(base.size(), "out");
+        bool ok = res && tmp && out && require(b.copy_bytes_from_host(*res, 0, base.data(), base.size() * 2), "upload bf16");
+        ok = ok && require(b.q8_0_matmul_add(*out, *res, *tmp, *dw, *dx, batch, cols, rows), "matmul_add bf16");
+        std::vector<uint16_t> got(base.size()), mid(base.size());
+        ok = ok && require(b.copy_bytes_to_host(*out, got.data(), 0, got.size() * 2), "download bf16");
+        ok = ok && require(b.copy_bytes_to_host(*tmp, mid.data(), 0, mid.size() * 2), "download bf16 tmp");
+        // the temporary: the oracle's product rounded to bf16, or its neighbour where the GPU's fp32 sum
+        // (same terms, another order) lies across a rounding boundary; the output: exactly the rounded
+        // sum of the residual and that temporary
+        size_t off = 0, far = 0;
+        for (size_t i = 0; i < got.size(); ++i) {
+            const int diff = std::abs(static_cast<int>(mid[i]) - static_cast<int>(q8o_f32_to_bf16(prod[i])));
+            off += diff != 0;
+            far += diff > 1;
+            if (got[i] != q8o_f32_to_bf16(q8o_bf16_to_f32(base[i]) + q8o_bf16_to_f32(mid[i]))) ++far;
+        }
+        ok = ok && far == 0 && off * 100 < got.size();
+        report("matmul_add_bf16_batch64", ok, "differing " + std::to_string(off) + ", beyond one step " + std::to_string(far));
     }
 }
 
@@ -742,6 +813,7 @@ int main(int argc, char **argv) {
     struct Case { const char *name; void (*fn)(qw3::HipQ8Backend &); };
     const Case cases[] = {
         {"closed_form", case_closed_form}, {"matvec", case_matvec_family}, {"matmul", case_matmul},
+        {"matmul_add", case_matmul_add_batched},
         {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"gguf", case_gguf}, {"lm_head", case_lm_head_verify}, {"rms_norm", case_rms_norm}, {"graph", case_graph_replay},
     };
     for (const auto &c : cases) {
