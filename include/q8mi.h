@@ -262,6 +262,20 @@ int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y_q8_1, uint32
                                int32_t *accept_out, float *logits, uint32_t stride_logits,
                                void *scratch, void *stream);
 
+/* No counterpart in the reference.  q8mi_lm_head_argmax_accept for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): same arguments without `scratch`, same results bit for bit.  The per-workgroup
+ * partials go to a 64 KiB array the library holds in every GPU's memory from load to exit
+ * (8 verify rows x 1024 workgroups, the most any call needs; a shape that would need more is
+ * Q8MI_REJECTED).  The call allocates and frees nothing.  Its first call on a device looks the
+ * array's address up (make that call outside a capture).  Every call on one GPU uses that GPU's
+ * one array: calls that overlap on the same GPU (two streams, two threads) race on it and must be
+ * serialised by the caller; nothing in it needs clearing between calls. */
+int q8mi_lm_head_argmax_accept_static(const uint8_t *weight, const void *y_q8_1, uint32_t rows, uint32_t cols,
+                                      uint32_t batch, const int32_t *drafts, int drafts_on_device, int32_t eos,
+                                      q8mi_argmax_pair *row_out, int32_t *accept_out, float *logits,
+                                      uint32_t stride_logits, void *stream);
+
 /* ---- weight upload (host side) ------------------------------------------- */
 /* replaces the repack loop of the CudaWeight constructor,
  * src/kernels_cuda.cu:1566-1594: interleaved GGUF Q8_0 blocks (34 B: fp16 d,

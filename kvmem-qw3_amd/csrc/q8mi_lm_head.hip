@@ -17,10 +17,17 @@
 #include "q8mi_gemv_core.hpp"
 #include "q8mi_gemv_mfma_core.hpp"
 
+// Partials of q8mi_lm_head_argmax_accept_static: one {value, index} pair per (verify row, workgroup),
+// at most 8 rows x 1024 workgroups = 64 KiB, held by every GPU the library runs on until the process
+// ends.  In host code this name is only a handle for hipGetSymbolAddress; kernels get the address.
+static __device__ __align__(256) uint8_t scratch[Q8MI_MAX_GEMV_BATCH * 1024 * sizeof(q8mi_argmax_pair)];
+
 namespace q8mi {
 namespace {
 
 constexpr uint32_t kMaxPartials = 1024;
+static_assert(sizeof(scratch) == Q8MI_MAX_GEMV_BATCH * kMaxPartials * sizeof(q8mi_argmax_pair),
+              "the static scratch holds the partials of the largest call");
 constexpr int kMaxDrafts = Q8MI_MAX_GEMV_BATCH - 1;
 
 struct Drafts {
@@ -467,4 +474,45 @@ extern "C" int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y, 
     if (int rc = lm_head_gate(weight, rows, cols, batch, drafts)) return rc;
     return lm_head_run(weight, y, rows, cols, batch, drafts, drafts_on_device, eos, row_out, accept_out, logits,
                        stride_logits, static_cast<q8mi_argmax_pair *>(scratch_arg), stream);
+}
+
+// Address of this device's copy of the static scratch array: looked up once per device, with that
+// device current (every GPU holds its own copy at its own address).
+static int static_scratch_of_current_device(void **out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *ptr_of[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return fail(Q8MI_LAUNCH_ERROR, "lm_head (static scratch): no current device, or a device id beyond %d", kMaxDevices - 1);
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr_of[dev] == nullptr) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "lm_head (static scratch): hipGetSymbolAddress: %s", hipGetErrorString(e));
+        }
+        ptr_of[dev] = p;
+    }
+    *out = ptr_of[dev];
+    return Q8MI_OK;
+}
+
+extern "C" int q8mi_lm_head_argmax_accept_static(const uint8_t *weight, const void *y, uint32_t rows, uint32_t cols,
+                                                 uint32_t batch, const int32_t *drafts, int drafts_on_device,
+                                                 int32_t eos, q8mi_argmax_pair *row_out, int32_t *accept_out,
+                                                 float *logits, uint32_t stride_logits, void *stream) {
+    if (int rc = lm_head_gate(weight, rows, cols, batch, drafts)) return rc;
+    if (q8mi_lm_head_scratch_bytes(rows, cols, batch) > sizeof(scratch))
+        return fail(Q8MI_REJECTED, "lm_head (static scratch): %zu bytes of partials needed, the library holds %zu",
+                    q8mi_lm_head_scratch_bytes(rows, cols, batch), sizeof(scratch));
+    void *partials = nullptr;
+    if (int rc = static_scratch_of_current_device(&partials)) return rc;
+    // nothing in the array has to start at zero: the finalize kernel reads only the partials
+    // [row][0 .. grid) that the stream kernel of the same call has just written
+    return lm_head_run(weight, y, rows, cols, batch, drafts, drafts_on_device, eos, row_out, accept_out, logits,
+                       stride_logits, static_cast<q8mi_argmax_pair *>(partials), stream);
 }

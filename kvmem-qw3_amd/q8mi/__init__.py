@@ -58,6 +58,8 @@ SIGNATURES = {
     "q8mi_lm_head_scratch_bytes": (C.c_size_t, [_u32, _u32, _u32]),
     "q8mi_lm_head_argmax_accept": (_int, [_u8p, _vp, _u32, _u32, _u32, _vp, _int, C.c_int32, _vp, _vp, _vp,
                                           _u32, _vp, _vp]),
+    "q8mi_lm_head_argmax_accept_static": (_int, [_u8p, _vp, _u32, _u32, _u32, _vp, _int, C.c_int32, _vp, _vp, _vp,
+                                                 _u32, _vp]),
     "q8mi_repack_q8_0_split_host": (_int, [_vp, _u64, _u64, _vp]),
     "q8mi_repack_q8_0_split": (_int, [_vp, _u64, _u64, _vp, _vp]),
     "q8mi_qgemv": (_int, [_vp, _vp, _u32, _vp, _int, _u32, _u32, _u32, _u32, _vp]),
