@@ -1,11 +1,13 @@
 // GGUF v3 container reader for the tensors this path consumes, and the step from a
 // Q8_0 tensor in the file to a device-resident split-plane weight.
 //
-// Mirrors the part of the reference's reader that the weight loader uses
-// (include/qw3/gguf.hpp:13-78, src/gguf.cpp:205-392): same class and member
-// names, same error behaviour (std::runtime_error with the same conditions:
-// unreadable/empty file, wrong magic, version != 3, truncated header, tensor rank
-// above 8, tensor outside the file).  The tokenizer/model-info helpers of the
+// Declares the part of the reference's reader interface that the weight loader uses
+// (include/qw3/gguf.hpp:13-78): same class and member names, and a std::runtime_error
+// under the same conditions as the reference's reader (src/gguf.cpp:205-392:
+// unreadable or empty file, wrong magic, version != 3, a file that ends inside the
+// header, tensor rank above 8, a tensor outside the file, a block type that does not
+// divide into whole blocks); the implementation and its messages are this library's
+// own.  The tokenizer/model-info helpers of the
 // reference's class are outside this path and absent.  The file is mapped
 // read-only; tensor data is handed to the backend straight from the mapping, as
 // the reference's model source does (src/model_source.cpp:108-127).

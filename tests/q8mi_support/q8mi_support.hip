@@ -49,6 +49,9 @@ int cu_count() {
 
 hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 
+// by value: a bit cast applied to a vector element directly reads the vector's first bytes
+__device__ __forceinline__ float bits_as_f32(int v) { return __builtin_bit_cast(float, v); }
+
 // ---- checker: int32 block dots on the GPU ------------------------------------
 __global__ __launch_bounds__(256) void block_dots_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ y,
                                                          int layout, uint32_t nb, uint32_t batch,
@@ -138,12 +141,18 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(int *__restrict__ out, 
 // 4 x 4 each: lane l gets a[4 (l/4) + v] * b[l] in register v, which is the layout of the sums),
 // and acc += sum * product is the one FMA.  Operands are loop-invariant registers: nothing but the
 // two pipes is measured.
-__global__ __launch_bounds__(256) void probe_mfma_one_fma_kernel(int *__restrict__ out, uint32_t iters, float a, float b) {
-    v8h ha, hb;
+__global__ __launch_bounds__(256, 2) void probe_mfma_one_fma_kernel(int *__restrict__ out, uint32_t iters, float a, float b) {
+    // one activation fragment and four weight fragments (two K = 16 halves each), four weight scales
+    v8h ya[2], wb[4][2];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-        ha[k] = static_cast<_Float16>(static_cast<int>(threadIdx.x % 7) - 3 + k);
-        hb[k] = static_cast<_Float16>(static_cast<int>(threadIdx.x % 5) - 2 - k);
+        ya[0][k] = static_cast<_Float16>(static_cast<int>(threadIdx.x % 7) - 3 + k);
+        ya[1][k] = static_cast<_Float16>(static_cast<int>(threadIdx.x % 5) - 2 - k);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            wb[p][0][k] = static_cast<_Float16>(static_cast<int>(threadIdx.x % 3) + p - k);
+            wb[p][1][k] = static_cast<_Float16>(static_cast<int>(threadIdx.x % 11) - p + k);
+        }
     }
     float acc[4][16];
 #pragma unroll
@@ -152,23 +161,31 @@ __global__ __launch_bounds__(256) void probe_mfma_one_fma_kernel(int *__restrict
         for (int v = 0; v < 16; ++v) acc[p][v] = 0.0f;
     const v16f zero16 = {0};
     const v4f zero4 = {0, 0, 0, 0};
-    float dy = a + static_cast<float>(threadIdx.x) * 1e-3f, dw = b;
+    float dy[4], dw[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        dy[g] = a + static_cast<float>(threadIdx.x + g) * 1e-3f;
+        dw[g] = b + static_cast<float>(g) * 1e-2f;
+    }
     for (uint32_t i = 0; i < iters; ++i) {
+        // opaque to the optimiser: every round and every patch has operands of its own, as in a
+        // kernel that reads them from LDS
+        asm volatile("" : "+v"(ya[0]), "+v"(ya[1]));
+#pragma unroll
+        for (int p = 0; p < 4; ++p) asm volatile("" : "+v"(wb[p][0]), "+v"(wb[p][1]), "+v"(dw[p]), "+v"(dy[p]));
         v16f s[4];
         v4f pr[4][4];
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            s[p] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ha, hb, zero16, 0, 0, 0);
-            s[p] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hb, ha, s[p], 0, 0, 0);
+            s[p] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ya[0], wb[p][0], zero16, 0, 0, 0);
+            s[p] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ya[1], wb[p][1], s[p], 0, 0, 0);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) pr[p][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(dy, dw, zero4, 0, 0, 0);
+            for (int g = 0; g < 4; ++g) pr[p][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(dy[g], dw[p], zero4, 0, 0, 0);
         }
 #pragma unroll
         for (int p = 0; p < 4; ++p)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[p][v] = fmaf(s[p][v], pr[p][v / 4][v % 4], acc[p][v]);
-        // keep the operands loop-variant so that nothing is hoisted
-        asm volatile("" : "+v"(ha), "+v"(hb), "+v"(dy), "+v"(dw));
     }
     float f = 0.0f;
 #pragma unroll
@@ -180,28 +197,40 @@ __global__ __launch_bounds__(256) void probe_mfma_one_fma_kernel(int *__restrict
 
 // The int8 kernel's own arithmetic with its dependences: four int8 MFMAs seeded with 1.5 * 2^23 and
 // the two FMAs per sum that consume their results (g = fma(F, d_w, -1.5 * 2^23 * d_w), acc += g * d_y).
-__global__ __launch_bounds__(256) void probe_mfma_two_fma_kernel(int *__restrict__ out, uint32_t iters, float a, float b) {
-    v4i va = {static_cast<int>(threadIdx.x), 1, 2, 3}, vb = {4, 5, 6, static_cast<int>(threadIdx.x)};
+__global__ __launch_bounds__(256, 2) void probe_mfma_two_fma_kernel(int *__restrict__ out, uint32_t iters, float a, float b) {
+    v4i ya = {static_cast<int>(threadIdx.x), 1, 2, 3}, wb[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) wb[p] = v4i{4 + p, 5, 6, static_cast<int>(threadIdx.x)};
     v16i seed;
 #pragma unroll
     for (int v = 0; v < 16; ++v) seed[v] = 0x4B400000;
+    asm volatile("" : "+v"(seed));   // kept in registers, as in the kernel
     float acc[4][16];
 #pragma unroll
     for (int p = 0; p < 4; ++p)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[p][v] = 0.0f;
-    float dy = a, dw = b;
+    float dy[16], dw[4];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dy[v] = a + static_cast<float>(v) * 1e-3f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) dw[p] = b + static_cast<float>(p) * 1e-2f;
     for (uint32_t i = 0; i < iters; ++i) {
+        asm volatile("" : "+v"(ya));
+#pragma unroll
+        for (int p = 0; p < 4; ++p) asm volatile("" : "+v"(wb[p]), "+v"(dw[p]));
+#pragma unroll
+        for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(dy[v]));
         v16i r[4];
 #pragma unroll
-        for (int p = 0; p < 4; ++p) r[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(va, vb, seed, 0, 0, 0);
-        const float cw = -12582912.0f * dw;
+        for (int p = 0; p < 4; ++p) r[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ya, wb[p], seed, 0, 0, 0);
 #pragma unroll
-        for (int p = 0; p < 4; ++p)
+        for (int p = 0; p < 4; ++p) {
+            const float cw = -12582912.0f * dw[p];
 #pragma unroll
             for (int v = 0; v < 16; ++v)
-                acc[p][v] = fmaf(fmaf(__builtin_bit_cast(float, r[p][v]), dw, cw), dy, acc[p][v]);
-        asm volatile("" : "+v"(va), "+v"(vb), "+v"(dy), "+v"(dw));
+                acc[p][v] = fmaf(fmaf(bits_as_f32(r[p][v]), dw[p], cw), dy[v], acc[p][v]);
+        }
     }
     float f = 0.0f;
 #pragma unroll
