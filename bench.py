@@ -4,13 +4,14 @@
 One "step" = one pass over the decode GEMV set of one 27B-style layer at M=1
 (BASELINE config 1), through the C ABI exactly as the executor would drive it:
 
-    qgemv_fanout4(x[5120])   Q 5120x6144, K 5120x1024, V 5120x1024   (quantizer fused into the GEMV)
-    qgemv_add(a[6144])       O 6144x5120, residual add               (fused)
-    qgemv_silu_mul(x[5120])  gate, up 5120x17408 each                (fused)
-    qgemv_add(f[17408])      down 17408x5120, residual add           (fused, one 1024-thread workgroup per CU)
+    quantize_q8_1(x[5120])    the normed row, once for the two operators that read it
+    gemv_fanout4              Q 5120x6144, K 5120x1024, V 5120x1024
+    qgemv_add(a[6144])        O 6144x5120, residual add (quantizer inside the GEMV)
+    gemv_silu_mul             gate, up 5120x17408 each
+    quantize_q8_1(f[17408])
+    gemv_add                  down 17408x5120, residual add
 
-which is the routing of the host layer (HipQ8Backend) at batch 1; for batch 2..8 every op is
-quantize_q8_1 + GEMV (two launches), as in the reference.
+for batch 2..8 the O projection is quantize_q8_1 + gemv_add as well (7 launches).
 
 `value` is algorithmic bytes per step / time per step with all inputs resident
 in HBM, cycling through several distinct copies of the layer's weights so that
@@ -84,39 +85,33 @@ class DecodeStep:
         return layer_bytes + act + outs
 
     @property
-    def fused(self):
-        return self.m == 1
-
-    @property
     def launches(self):
-        return 4 if self.fused else 8
+        return 6 if self.m == 1 else 7
 
     def run(self, layer, stream=None):
+        """The host layer's routing: the normed row is quantized once for the fan-out and the SwiGLU
+        (they read the same row); at M=1 the O projection quantizes its input inside the GEMV (one
+        launch instead of two), every other operator reads Q8_1 blocks."""
         L, m, w = self.L, self.m, layer.w
         ok = self.ok
-        if self.fused:
-            ok(L.q8mi_qgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.x.ptr, HIDDEN,
-                                    self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
-                                    HIDDEN, m, QDIM, KVDIM, KVDIM, 0, stream), "qfanout4")
-            ok(L.q8mi_qgemv_add(w["o"].ptr, self.attn.ptr, ATTN_OUT, self.h.ptr, 0, HIDDEN, ATTN_OUT, m, HIDDEN,
-                                stream), "qo")
-            self.run_silu(layer, stream)
-            ok(L.q8mi_qgemv_add(w["down"].ptr, self.ffn.ptr, FFN, self.h.ptr, 0, HIDDEN, FFN, m, HIDDEN, stream), "qdown")
-            return
-        ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize")
+        ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize x")
         ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.y5120.ptr,
                                self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
                                HIDDEN, m, QDIM, KVDIM, KVDIM, 0, stream), "fanout4")
-        ok(L.q8mi_quantize_q8_1(self.attn.ptr, self.y6144.ptr, m, ATTN_OUT, ATTN_OUT, stream), "quantize")
-        ok(L.q8mi_gemv_add(w["o"].ptr, self.y6144.ptr, self.h.ptr, HIDDEN, ATTN_OUT, m, HIDDEN, stream), "o")
-        ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize")
+        if m == 1:
+            ok(L.q8mi_qgemv_add(w["o"].ptr, self.attn.ptr, ATTN_OUT, self.h.ptr, 0, HIDDEN, ATTN_OUT, m, HIDDEN,
+                                stream), "qo")
+        else:
+            ok(L.q8mi_quantize_q8_1(self.attn.ptr, self.y6144.ptr, m, ATTN_OUT, ATTN_OUT, stream), "quantize attn")
+            ok(L.q8mi_gemv_add(w["o"].ptr, self.y6144.ptr, self.h.ptr, HIDDEN, ATTN_OUT, m, HIDDEN, stream), "o")
         self.run_silu(layer, stream)
-        ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, m, FFN, FFN, stream), "quantize")
+        ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, m, FFN, FFN, stream), "quantize ffn")
         ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, m, HIDDEN, stream), "down")
 
     def run_with_norms(self, layer, one_launch, stream=None):
-        """The same four GEMVs at M=1 preceded by the layer's two RMS norms: inside the fan-out and
-        SwiGLU launches (4 launches), or as two launches of their own (6)."""
+        """The same GEMVs at M=1 preceded by the layer's two RMS norms: inside the fan-out and
+        SwiGLU launches (5 launches), or as norm + quantizer kernels of their own in front of
+        them (7)."""
         L, w, ok = self.L, layer.w, self.ok
         if not hasattr(self, "norm_w"):
             import numpy as np
@@ -124,32 +119,38 @@ class DecodeStep:
             self.norm_w = hip.to_device(np.ones(HIDDEN, np.float32))
             self.h_in = hip.to_device(np.linspace(-2.0, 2.0, HIDDEN, dtype=np.float32))
         eps = 1e-6
-        if one_launch:
-            ok(L.q8mi_nqgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.h_in.ptr, self.norm_w.ptr, eps,
-                                     self.x.ptr, self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
-                                     HIDDEN, 1, stream), "nqfanout4")
-        else:
-            ok(L.q8mi_rms_norm(self.h_in.ptr, self.norm_w.ptr, self.x.ptr, 1, HIDDEN, HIDDEN, HIDDEN, eps, stream), "norm")
-            ok(L.q8mi_qgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.x.ptr, HIDDEN,
-                                    self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
-                                    HIDDEN, 1, QDIM, KVDIM, KVDIM, 0, stream), "qfanout4")
+        def fanout():
+            if one_launch:
+                ok(L.q8mi_nqgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.h_in.ptr, self.norm_w.ptr, eps,
+                                         self.x.ptr, self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
+                                         HIDDEN, 1, stream), "nqfanout4")
+                return
+            ok(L.q8mi_rms_norm_quantize_q8_1(self.h_in.ptr, self.norm_w.ptr, self.x.ptr, self.y5120.ptr, 1, HIDDEN, HIDDEN,
+                                             HIDDEN, eps, stream), "norm+quantize")
+            ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.y5120.ptr, self.q.ptr, self.k.ptr,
+                                   self.v.ptr, None, QDIM, KVDIM, KVDIM, 0, HIDDEN, 1, QDIM, KVDIM, KVDIM, 0, stream), "fanout4")
+        def silu():
+            if one_launch:
+                ok(L.q8mi_nqgemv_silu_mul(w["gate"].ptr, w["up"].ptr, self.h_in.ptr, self.norm_w.ptr, eps, self.x.ptr,
+                                          self.ffn.ptr, FFN, HIDDEN, 1, stream), "nqsilu_mul")
+                return
+            ok(L.q8mi_rms_norm_quantize_q8_1(self.h_in.ptr, self.norm_w.ptr, self.x.ptr, self.y5120.ptr, 1, HIDDEN, HIDDEN,
+                                             HIDDEN, eps, stream), "norm+quantize")
+            ok(L.q8mi_gemv_silu_mul(w["gate"].ptr, w["up"].ptr, self.y5120.ptr, self.ffn.ptr, FFN, HIDDEN, 1, FFN, stream),
+               "silu_mul")
+        fanout()
         ok(L.q8mi_qgemv_add(w["o"].ptr, self.attn.ptr, ATTN_OUT, self.h.ptr, 0, HIDDEN, ATTN_OUT, 1, HIDDEN, stream), "qo")
-        if one_launch:
-            ok(L.q8mi_nqgemv_silu_mul(w["gate"].ptr, w["up"].ptr, self.h_in.ptr, self.norm_w.ptr, eps, self.x.ptr,
-                                      self.ffn.ptr, FFN, HIDDEN, 1, stream), "nqsilu_mul")
-        else:
-            ok(L.q8mi_rms_norm(self.h_in.ptr, self.norm_w.ptr, self.x.ptr, 1, HIDDEN, HIDDEN, HIDDEN, eps, stream), "norm")
-            ok(L.q8mi_qgemv_silu_mul(w["gate"].ptr, w["up"].ptr, self.x.ptr, HIDDEN, self.ffn.ptr, FFN, HIDDEN, 1, FFN,
-                                     stream), "qsilu_mul")
-        ok(L.q8mi_qgemv_add(w["down"].ptr, self.ffn.ptr, FFN, self.h.ptr, 0, HIDDEN, FFN, 1, HIDDEN, stream), "qdown")
+        silu()
+        ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, 1, FFN, FFN, stream), "quantize ffn")
+        ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, 1, HIDDEN, stream), "down")
 
     def run_silu(self, layer, stream=None):
-        if self.fused:
-            self.ok(self.L.q8mi_qgemv_silu_mul(layer.w["gate"].ptr, layer.w["up"].ptr, self.x.ptr, HIDDEN,
-                                               self.ffn.ptr, FFN, HIDDEN, self.m, FFN, stream), "qsilu_mul")
-            return
+        """gate/up SwiGLU on the Q8_1 blocks of x (quantized by run(), or by prepare_silu())."""
         self.ok(self.L.q8mi_gemv_silu_mul(layer.w["gate"].ptr, layer.w["up"].ptr, self.y5120.ptr, self.ffn.ptr,
                                           FFN, HIDDEN, self.m, FFN, stream), "silu_mul")
+
+    def prepare_silu(self):
+        self.ok(self.L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, self.m, HIDDEN, HIDDEN, None), "quantize x")
 
     def silu_bytes(self):
         return 2 * w_bytes(FFN, HIDDEN) + q81_bytes(self.m, HIDDEN) + 4 * self.m * FFN
@@ -279,24 +280,33 @@ def cpu_gemm_sample(rows=2048, m=2048, cols=HIDDEN):
 
 
 def bench_config0(q8mi, hip, synth, copies=48, reps=480):
-    """BASELINE config 0: one 5120x5120 GEMV at M=1 from fp32 activations (quantizer fused).
+    """BASELINE config 0: one 5120x5120 GEMV at M=1.  The GEMV proper reads Q8_1 activations
+    (q8mi_gemv: what the bytes of this config count); also timed: the entry point that quantizes
+    fp32 activations inside the GEMV, and quantizer + GEMV as two launches.
     Streaming: cycles through `copies` weight buffers (1.3 GB, no cache hits); resident: one buffer."""
     L, ok = q8mi.lib(), q8mi.ok
     host = synth.q8_0_weight(HIDDEN, HIDDEN, seed=31)
     ws = [hip.to_device(host) for _ in range(copies)]
     x = hip.to_device(synth.normal(1, HIDDEN, seed=32))
+    y = hip.DeviceBuffer(q81_bytes(1, HIDDEN))
     dst = hip.DeviceBuffer(4 * HIDDEN)
-    fn = lambda i: ok(L.q8mi_qgemv(ws[i % copies].ptr, x.ptr, HIDDEN, dst.ptr, 0, HIDDEN, HIDDEN, 1, HIDDEN, None),
-                      "qgemv")
-    one = lambda i: ok(L.q8mi_qgemv(ws[0].ptr, x.ptr, HIDDEN, dst.ptr, 0, HIDDEN, HIDDEN, 1, HIDDEN, None), "qgemv")
-    t_stream = time_loop(hip, fn, reps, copies)
-    t_res = time_loop(hip, one, reps, 10)
+    quant = lambda: ok(L.q8mi_quantize_q8_1(x.ptr, y.ptr, 1, HIDDEN, HIDDEN, None), "quantize")
+    gemv = lambda w: ok(L.q8mi_gemv(w.ptr, y.ptr, dst.ptr, HIDDEN, HIDDEN, 1, HIDDEN, None), "gemv")
+    qgemv = lambda w: ok(L.q8mi_qgemv(w.ptr, x.ptr, HIDDEN, dst.ptr, 0, HIDDEN, HIDDEN, 1, HIDDEN, None), "qgemv")
+    quant()
+    t_stream = time_loop(hip, lambda i: gemv(ws[i % copies]), reps, copies)
+    t_res = time_loop(hip, lambda i: gemv(ws[0]), reps, 10)
+    t_fused = time_loop(hip, lambda i: qgemv(ws[i % copies]), reps, copies)
+    t_two = time_loop(hip, lambda i: (quant(), gemv(ws[i % copies])), reps, copies)
     nbytes = w_bytes(HIDDEN, HIDDEN) + q81_bytes(1, HIDDEN) + 4 * HIDDEN
-    for b in ws + [x, dst]:
+    for b in ws + [x, y, dst]:
         b.free()
-    return {"bytes": nbytes, "streaming_us": round(t_stream * 1e3, 3),
-            "streaming_gbps": round(nbytes / (t_stream * 1e-3) / 1e9, 1),
-            "resident_us": round(t_res * 1e3, 3), "resident_gbps": round(nbytes / (t_res * 1e-3) / 1e9, 1)}
+    gbps = lambda t: round(nbytes / (t * 1e-3) / 1e9, 1)
+    return {"bytes": nbytes, "streaming_us": round(t_stream * 1e3, 3), "streaming_gbps": gbps(t_stream),
+            "frac_of_hbm_peak": round(gbps(t_stream) / HBM_PEAK_GBPS, 4),
+            "resident_us": round(t_res * 1e3, 3), "resident_gbps": gbps(t_res),
+            "fp32_activations_one_launch_us": round(t_fused * 1e3, 3),
+            "fp32_activations_quantizer_plus_gemv_us": round(t_two * 1e3, 3)}
 
 
 def bench_read_probe(synth, hip, nbytes=1 << 30, reps=20):
@@ -470,8 +480,9 @@ def main():
     value = step_bytes / (ms_stream * 1e-3) / 1e9
     ms_resident, _ = time_loop_settled(hip, lambda i: step.run(layers[0]), args.steps, 0, settle_ms=0.0, min_ms=50.0)
 
-    # dominant kernel: the fused gate/up SwiGLU GEMV (52 % of the step's bytes)
+    # dominant kernel: the gate/up SwiGLU GEMV (52 % of the step's bytes)
     n_each = min(max(args.steps, 50), 400)
+    step.prepare_silu()
     mean_ms, med_ms, min_ms = time_each_launch(hip, lambda i: step.run_silu(layers[i % len(layers)]), n_each)
     back_ms = time_loop(hip, lambda i: step.run_silu(layers[i % len(layers)]), n_each, 5)
     silu_bytes = step.silu_bytes()
@@ -493,7 +504,7 @@ def main():
         "resident_gbps": round(step_bytes / (ms_resident * 1e-3) / 1e9, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(),
-                     "kernel": "gemv_kernel<1, 256, 2, true> (SwiGLU with fused quantizer: gate+up 2 x 5120x17408)",
+                     "kernel": "gemv_pairs_kernel<1, 5, true> (SwiGLU: gate+up 2 x 5120x17408, Q8_1 activations)",
                      "bytes_per_launch": silu_bytes, "launch_ms": round(back_ms, 5),
                      "launch_ms_mean": round(mean_ms, 5),
                      "launch_ms_median": round(med_ms, 5), "launch_ms_min": round(min_ms, 5),
@@ -519,7 +530,7 @@ def main():
         result["gemv_layer_gbps_by_m"] = sweep
         # the layer's two RMS norms in front of the fan-out and the SwiGLU: inside those launches, or on their own
         norms = {}
-        for name, one in (("norms_inside_the_gemv_4_launches", True), ("norms_as_2_more_launches", False)):
+        for name, one in (("norms_inside_the_gemv_5_launches", True), ("norm_quantizer_kernels_7_launches", False)):
             t = time_loop(hip, lambda i: step.run_with_norms(layers[i % len(layers)], one), max(args.steps // 2, 20), 5)
             norms[name] = {"ms_per_step": round(t, 5), "gbps": round(step_bytes / (t * 1e-3) / 1e9, 1)}
         result["layer_with_rms_norms_m1"] = norms

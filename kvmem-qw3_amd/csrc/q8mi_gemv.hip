@@ -12,61 +12,12 @@
 // kernel name in a profile).
 #include "q8mi_gemv_core.hpp"
 #include "q8mi_gemv_mfma_core.hpp"
+#include "q8mi_gemv_params.hpp"
 
 namespace q8mi {
 namespace {
 
-enum GemvMode : int {
-    kStoreF32 = 0,
-    kAddF32 = 1,
-    kStoreBF16 = 2,
-    kAddBF16 = 3,
-    kSiluMul = 4,  // w[0] = gate, w[1] = up, one output
-};
 
-struct GemvParams {
-    const uint8_t *w[4];
-    void *dst[4];
-    uint32_t row_end[4];  // cumulative row counts of the concatenated row space
-    uint32_t stride[4];
-    const uint8_t *y;     // Q8_1 blocks, [batch][nb] (null when xf is set)
-    const float *xf;      // fp32 activations to be quantized while staging (fused entry points)
-    uint32_t x_stride;    // floats between rows of xf
-    const float *norm_w;  // RMS-norm weights: xf is one raw row, normalised while staging (else null)
-    float *normalized;    // where the normalised row is also written (may be null)
-    float eps;
-    uint32_t total_rows;  // rows of the concatenated space (SwiGLU: rows of one weight)
-    uint32_t units;
-    uint32_t nb;
-    uint32_t x_bytes;     // LDS bytes of the staged activations (0 when they are read from global)
-    int mode;
-    int interleave;
-};
-
-// Which of the (up to four) concatenated weights a row belongs to.
-struct RowRef {
-    const uint8_t *w;
-    void *dst;
-    uint32_t stride;
-    uint32_t local;
-};
-
-__device__ __forceinline__ RowRef resolve_row(const GemvParams &p, uint32_t row) {
-    uint32_t seg = 0, base = 0;
-    if (row >= p.row_end[0]) { seg = 1; base = p.row_end[0]; }
-    if (row >= p.row_end[1]) { seg = 2; base = p.row_end[1]; }
-    if (row >= p.row_end[2]) { seg = 3; base = p.row_end[2]; }
-    RowRef r;
-    r.w = p.w[0]; r.dst = p.dst[0]; r.stride = p.stride[0];
-    if (seg == 1) { r.w = p.w[1]; r.dst = p.dst[1]; r.stride = p.stride[1]; }
-    if (seg == 2) { r.w = p.w[2]; r.dst = p.dst[2]; r.stride = p.stride[2]; }
-    if (seg == 3) { r.w = p.w[3]; r.dst = p.dst[3]; r.stride = p.stride[3]; }
-    r.local = row - base;
-    return r;
-}
-
-
-__device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, float v);
 
 // Each wave parks the (possibly partial) sums of the units it touched in LDS;
 // after a barrier the workgroup adds the partials of every unit in wave order and
@@ -155,20 +106,6 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
             const RowRef ref = resolve_row(p, row);
             store_out(p.mode, ref.dst, static_cast<uint64_t>(m) * ref.stride + ref.local, total_of(k, mr));
         }
-    }
-}
-
-__device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, float v) {
-    if (mode == kStoreF32) {
-        static_cast<float *>(dst)[idx] = v;
-    } else if (mode == kAddF32) {
-        float *p = static_cast<float *>(dst) + idx;
-        *p = *p + v;
-    } else if (mode == kStoreBF16) {
-        static_cast<uint16_t *>(dst)[idx] = float_to_bf16_bits(v);
-    } else {
-        uint16_t *p = static_cast<uint16_t *>(dst) + idx;
-        *p = float_to_bf16_bits(bf16_bits_to_float(*p) + v);
     }
 }
 
@@ -336,29 +273,8 @@ template <int M, bool SILU>
 int launch_ms(const GemvParams &p, hipStream_t stream) {
     const uint32_t xb = x_lds_bytes(p.nb, M);
     const uint32_t park_256 = 4 * kParkFloats * 4, park_1024 = 16 * kParkFloats * 4;
-    if (p.norm_w != nullptr) {   // fused norm + quantizer: one row, held in registers between the two passes
-        if constexpr (M == 1) {
-            const uint32_t cols = p.nb * kQK;
-            if (cols > StageF32<1, 256, true>::kBatch * 256u * 4u || xb + park_256 > 76u * 1024u)
-                return fail(Q8MI_REJECTED, "nqgemv: rows of %u columns are not served (at most %u)", cols,
-                            StageF32<1, 256, true>::kBatch * 256u * 4u);
-            auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-            if (!al(p.xf) || !al(p.norm_w) || (p.normalized != nullptr && !al(p.normalized)))
-                return fail(Q8MI_REJECTED, "nqgemv: activations, norm weights and normalised output must be 16-byte aligned");
-            return launch_inst<1, 256, kXNormF32, SILU>(p, xb, stream);
-        } else {
-            return fail(Q8MI_REJECTED, "nqgemv: batch %d above 1 (normalise and quantize once, then use the GEMV)", M);
-        }
-    }
-    if (p.xf != nullptr) {   // fused quantizer: the activations must fit LDS
-        if (M > 2) return fail(Q8MI_REJECTED, "qgemv: batch %d above 2 (quantize once and use the GEMV instead)", M);
-        // rows above 8192 columns: one 1024-thread workgroup per CU quantizes them once per CU instead of twice
-        const bool long_rows = p.nb * kQK > 8192u && xb + park_1024 <= kLdsLimit;
-        if (xb + park_256 <= 76u * 1024u && !long_rows)
-            return launch_inst<M, 256, kXF32, SILU>(p, xb, stream);
-        if (xb + park_1024 <= kLdsLimit) return launch_inst<M, 1024, kXF32, SILU>(p, xb, stream);
-        return fail(Q8MI_REJECTED, "qgemv: %u activation rows of %u columns do not fit LDS", M, p.nb * 32);
-    }
+    // fp32 activations (fused quantizer, fused norm) are served by the row-pair kernels only
+    if (p.xf != nullptr) return fail(Q8MI_REJECTED, "qgemv: batch %d, %u columns: not served in one launch", M, p.nb * 32);
     // the LDS staging loads 16 bytes at a time: activations on a 4-byte boundary are read by the lanes
     if (reinterpret_cast<uintptr_t>(p.y) % 16 != 0) return launch_inst<M, 256, kXGlobal, SILU>(p, 0, stream);
     if (xb + park_256 <= 76u * 1024u) return launch_inst<M, 256, kXLds, SILU>(p, xb, stream);   // two per CU fit
@@ -436,6 +352,10 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         if (grid > max_wgs) grid = max_wgs;
         gemv_unaligned_kernel<<<grid, 256, 0, stream>>>(p, batch);
         return check_launch("gemv_unaligned");
+    }
+    if (batch <= 2) {   // whole row pairs per wave, handed out by the dispatcher (q8mi_gemv_pairs.hip)
+        const int rc = launch_pairs(p, batch, stream);
+        if (rc != Q8MI_REJECTED) return rc;
     }
     if (p.xf == nullptr && reinterpret_cast<uintptr_t>(p.y) % 16 == 0 &&
         batch >= kMfmaFromBatch &&

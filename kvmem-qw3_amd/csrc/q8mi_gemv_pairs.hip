@@ -1,0 +1,629 @@
+// Q8_0 x Q8_1 GEMV for batch 1..2 as many small, independent waves (gfx950).
+// Reference semantics: src/mmvq_q8.cu:193-280 (plain), :295-399 (two weights), :414-519 (SwiGLU),
+// :528-606 (residual add), :976-1068 (fan-out); like the reference's kernel, a weight row is read
+// once and reused for every activation row (:221-243).
+//
+// A wave owns whole ROW PAIRS: two weight rows (SwiGLU: a gate row and its up row) from their first
+// to their last column.  Nothing is shared between waves, so there is no LDS staging of partial
+// sums, no barrier after the stream and no combine step: a wave that has its two sums writes them
+// and ends, and the hardware dispatcher hands the next row pairs to whichever CU has room.  That
+// dynamic hand-out is what balances the chip; a static split over resident workgroups loses 3..5 us
+// per launch to CUs that finish one after the other.  Measured on MI355X against the streaming
+// kernels of q8mi_gemv.hip (same bytes): 5120 x 5120 8.9 -> 6.6 us, SwiGLU 2 x 17408 x 5120
+// 33.3 -> 29.6 us, 5120 x 17408 20.4 -> 17.4 us; a plain streaming read of those sizes takes
+// 6.0, 28.8 and 15.4 us.
+//
+// Lane layout.  A 1 KiB step of a row is one coalesced wave load: lane l holds 16 bytes, half of
+// block l/2.  The two rows of a pair swap half sums with one DPP move, so that even lanes end up
+// with the full int32 block dot of the first row and odd lanes with that of the second row: one
+// int32 sum and one fp32 rescale per 32-element block and row, and after a five-step butterfly
+// over the lanes of equal parity lane 0 holds the first row's result and lane 1 the second's.
+//
+// Activations never pass through LDS at batch 1..2 when they arrive as Q8_1 blocks: a lane needs
+// the same 16 bytes and the same scale of every step for every row pair it will ever see, so it
+// loads them once into registers (rows of up to 8 KiB; 25 registers per activation row at 5120
+// columns) or, for longer rows, alongside the weights of each step (served by L2).  fp32
+// activations (the entry points that quantize inside the GEMV) are quantized once per workgroup
+// into LDS by all of its waves, with the stand-alone quantizer's code, and then read into the
+// same registers.
+#include "q8mi_gemv_core.hpp"
+#include "q8mi_gemv_params.hpp"
+
+namespace q8mi {
+namespace {
+
+// 16 bytes of a Q8_1 block: 4-byte aligned by type
+struct __attribute__((packed, aligned(4))) Dwords4 {
+    int x, y, z, w;
+};
+__device__ __forceinline__ v4i load_x16(const uint8_t *p) {
+    const Dwords4 q = *reinterpret_cast<const Dwords4 *>(p);
+    return v4i{q.x, q.y, q.z, q.w};
+}
+
+// Row pairs of the concatenated row space: pairs never straddle two weights (a weight with an odd
+// number of rows ends with a pair whose second row is a repeat that is not written).
+struct PairSpace {
+    uint32_t pair_end[4];   // cumulative pair counts per weight
+    uint32_t pairs;
+    uint32_t ppw;           // consecutive pairs per wave
+};
+
+struct PairRows {
+    const uint8_t *r0, *r1;   // scale planes of the two rows
+    void *dst;
+    uint32_t stride;
+    uint32_t row0;            // row of r0 within its weight (SwiGLU: the output row)
+    bool two;                 // the second row exists
+};
+
+template <bool SILU>
+__device__ __forceinline__ PairRows resolve_pair(const GemvParams &p, const PairSpace &ps, uint32_t pair, uint64_t row_bytes) {
+    PairRows r;
+    if constexpr (SILU) {
+        r.r0 = p.w[0] + pair * row_bytes;
+        r.r1 = p.w[1] + pair * row_bytes;
+        r.dst = p.dst[0];
+        r.stride = p.stride[0];
+        r.row0 = pair;
+        r.two = true;
+    } else {
+        uint32_t seg = 0, base = 0, row_base = 0;
+        if (pair >= ps.pair_end[0]) { seg = 1; base = ps.pair_end[0]; row_base = p.row_end[0]; }
+        if (pair >= ps.pair_end[1]) { seg = 2; base = ps.pair_end[1]; row_base = p.row_end[1]; }
+        if (pair >= ps.pair_end[2]) { seg = 3; base = ps.pair_end[2]; row_base = p.row_end[2]; }
+        const uint8_t *w = p.w[0];
+        r.dst = p.dst[0]; r.stride = p.stride[0];
+        uint32_t rows = p.row_end[0];
+        if (seg == 1) { w = p.w[1]; r.dst = p.dst[1]; r.stride = p.stride[1]; rows = p.row_end[1] - row_base; }
+        if (seg == 2) { w = p.w[2]; r.dst = p.dst[2]; r.stride = p.stride[2]; rows = p.row_end[2] - row_base; }
+        if (seg == 3) { w = p.w[3]; r.dst = p.dst[3]; r.stride = p.stride[3]; rows = p.row_end[3] - row_base; }
+        r.row0 = 2 * (pair - base);
+        r.two = r.row0 + 1 < rows;
+        r.r0 = w + r.row0 * row_bytes;
+        r.r1 = r.two ? r.r0 + row_bytes : r.r0;
+    }
+    return r;
+}
+
+// Sum over the lanes of equal parity (xor 2 .. 32): every lane ends with its parity's total.
+__device__ __forceinline__ float parity_sum(float v) {
+    v += lane_xor<2>(v);
+    v += lane_xor<4>(v);
+    v += lane_xor<8>(v);
+    v += lane_xor<16>(v);
+    v += lane_xor<32>(v);
+    return v;
+}
+
+// Lane 0 holds the first row's totals, lane 1 the second row's (SwiGLU: gate and up).
+template <int M, bool SILU>
+__device__ __forceinline__ void write_pair(const GemvParams &p, const PairRows &rows, uint32_t lane, const float (&tot)[M]) {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        if constexpr (SILU) {
+            const float up = dpp_f32<kDppXor1>(tot[m]);
+            if (lane == 0)
+                static_cast<float *>(rows.dst)[static_cast<uint64_t>(m) * rows.stride + rows.row0] =
+                    (tot[m] / (1.0f + __expf(-tot[m]))) * up;
+        } else {
+            if (lane == 0 || (lane == 1 && rows.two))
+                store_out(p.mode, rows.dst, static_cast<uint64_t>(m) * rows.stride + rows.row0 + lane, tot[m]);
+        }
+    }
+}
+
+// ---- rows of NSTEPS KiB exactly: activations in registers, a pair's weights loaded at once ----------
+template <int NSTEPS>
+struct PairWeights {
+    v4i q0[NSTEPS], q1[NSTEPS];
+    uint16_t d0[NSTEPS], d1[NSTEPS];
+};
+
+template <int NSTEPS>
+__device__ __forceinline__ void issue_pair(PairWeights<NSTEPS> &r, const PairRows &rows, uint32_t lane) {
+    constexpr uint32_t nb = NSTEPS * 32;
+#pragma unroll
+    for (int s = 0; s < NSTEPS; ++s) {
+        r.q0[s] = load_q16(rows.r0 + 2 * nb + s * 1024 + lane * 16);
+        r.q1[s] = load_q16(rows.r1 + 2 * nb + s * 1024 + lane * 16);
+        r.d0[s] = reinterpret_cast<const uint16_t *>(rows.r0)[32 * s + (lane >> 1)];
+        r.d1[s] = reinterpret_cast<const uint16_t *>(rows.r1)[32 * s + (lane >> 1)];
+    }
+}
+
+template <int M, int NSTEPS>
+__device__ __forceinline__ void compute_pair(const PairWeights<NSTEPS> &r, const v4i (&xq)[M][NSTEPS],
+                                             const float (&dx)[M][NSTEPS], bool odd, float (&tot)[M]) {
+    float acc[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NSTEPS; ++s) {
+        const float dw = half_bits_to_float(odd ? r.d1[s] : r.d0[s]);
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const int sa = dot16(r.q0[s], xq[m][s]);
+            const int sb = dot16(r.q1[s], xq[m][s]);
+            const int S = (odd ? sb : sa) + dpp_i32<kDppXor1>(odd ? sa : sb);   // full 32-element block dot
+            acc[m] = fmaf(dw * dx[m][s], static_cast<float>(S), acc[m]);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < M; ++m) tot[m] = parity_sum(acc[m]);
+}
+
+// The wave's pairs, two register sets: the next pair's loads are in flight while one is consumed.
+template <int M, int NSTEPS, bool SILU, bool DOUBLE>
+__device__ __forceinline__ void run_pairs(const GemvParams &p, const PairSpace &ps, uint32_t first, uint32_t end,
+                                          const v4i (&xq)[M][NSTEPS], const float (&dx)[M][NSTEPS], uint32_t lane,
+                                          PairWeights<NSTEPS> &a, PairRows ra) {
+    constexpr uint64_t row_bytes = static_cast<uint64_t>(NSTEPS) * 32 * 34;
+    const bool odd = lane & 1u;
+    float tot[M];
+    if constexpr (DOUBLE) {
+        PairWeights<NSTEPS> b;
+        PairRows rb = ra;
+        uint32_t pair = first;
+        while (true) {
+            const bool more1 = pair + 1 < end;
+            if (more1) { rb = resolve_pair<SILU>(p, ps, pair + 1, row_bytes); issue_pair<NSTEPS>(b, rb, lane); }
+            compute_pair<M, NSTEPS>(a, xq, dx, odd, tot);
+            write_pair<M, SILU>(p, ra, lane, tot);
+            if (!more1) break;
+            ++pair;
+            const bool more2 = pair + 1 < end;
+            if (more2) { ra = resolve_pair<SILU>(p, ps, pair + 1, row_bytes); issue_pair<NSTEPS>(a, ra, lane); }
+            compute_pair<M, NSTEPS>(b, xq, dx, odd, tot);
+            write_pair<M, SILU>(p, rb, lane, tot);
+            if (!more2) break;
+            ++pair;
+        }
+    } else {
+        for (uint32_t pair = first; pair < end; ++pair) {
+            compute_pair<M, NSTEPS>(a, xq, dx, odd, tot);
+            const PairRows done = ra;
+            if (pair + 1 < end) { ra = resolve_pair<SILU>(p, ps, pair + 1, row_bytes); issue_pair<NSTEPS>(a, ra, lane); }
+            write_pair<M, SILU>(p, done, lane, tot);
+        }
+    }
+}
+
+// Q8_1 activations from global memory, one wave per workgroup.
+template <int M, int NSTEPS, bool SILU>
+__global__ __launch_bounds__(kWave) void gemv_pairs_kernel(const GemvParams p, const PairSpace ps) {
+    constexpr uint32_t nb = NSTEPS * 32;
+    constexpr uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t first = blockIdx.x * ps.ppw;
+    if (first >= ps.pairs) return;
+    const uint32_t end = first + ps.ppw < ps.pairs ? first + ps.ppw : ps.pairs;
+    // activations first (they arrive first), the first pair's weights right behind them
+    v4i xq[M][NSTEPS];
+    uint16_t dxh[M][NSTEPS];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int s = 0; s < NSTEPS; ++s) {
+            const uint8_t *blk = p.y + static_cast<uint64_t>(m * nb + 32 * s + (lane >> 1)) * kQ81Bytes;
+            xq[m][s] = load_x16(blk + 4 + (lane & 1u) * 16);
+            dxh[m][s] = *reinterpret_cast<const uint16_t *>(blk);
+        }
+    PairWeights<NSTEPS> a;
+    const PairRows ra = resolve_pair<SILU>(p, ps, first, row_bytes);
+    issue_pair<NSTEPS>(a, ra, lane);
+    float dx[M][NSTEPS];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int s = 0; s < NSTEPS; ++s) dx[m][s] = half_bits_to_float(dxh[m][s]);
+    run_pairs<M, NSTEPS, SILU, M == 1>(p, ps, first, end, xq, dx, lane, a, ra);
+}
+
+// Sum of the squares of one fp32 row in the order of the stand-alone RMS norm (q8mi_rms_norm.hip):
+// thread t of the first 256 adds chunks t, t + 256, ... in that order, the 256 partials meet in a
+// balanced tree (64 lanes by DPP, then the four wave sums).  Every thread of the workgroup must
+// call it (one barrier inside); `red` = four floats of LDS.  partial: this thread's sum, 0 for
+// threads beyond the first 256.
+__device__ __forceinline__ float first256_tree_sum(float partial, float *red) {
+    const uint32_t wave = threadIdx.x / kWave;
+    if (wave < 4) {   // wave-uniform
+        const float s = wave_sum(partial);
+        if (threadIdx.x % kWave == 0) red[wave] = s;
+    }
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// fp32 activations: the workgroup's waves quantize the row into LDS together (the stand-alone
+// quantizer's code, so the same bits), one barrier, then every wave goes its own way.  One
+// activation row; up to sixteen waves, so at most 128 registers per lane.
+// NORM: the row is RMS-normalised first, with the arithmetic of the stand-alone norm kernel
+// (same bits); workgroup 0 also writes the normalised row.  At most eight waves then.
+template <int NSTEPS, bool SILU, bool NORM>
+__global__ __launch_bounds__(NORM ? 512 : 1024) void gemv_pairs_f32_kernel(const GemvParams p, const PairSpace ps) {
+    constexpr uint32_t nb = NSTEPS * 32;
+    constexpr uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    constexpr uint32_t kChunks = nb * 8;   // float4 chunks of the row
+    __shared__ __align__(16) uint32_t lds_q[kChunks];
+    __shared__ float lds_d[nb];
+    __shared__ float red[4];
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t waves = blockDim.x / kWave;
+    const uint32_t first = (blockIdx.x * waves + wave) * ps.ppw;
+    const bool live = first < ps.pairs;
+    const uint32_t end = first + ps.ppw < ps.pairs ? first + ps.ppw : ps.pairs;
+    const bool vec = NORM || (reinterpret_cast<uintptr_t>(p.xf) % 16 == 0);   // the norm's entry points demand alignment
+    // activation loads first, the first pair's weights behind them, then the conversion
+    constexpr uint32_t kMaxTrips = (kChunks + 255) / 256;   // at least four waves
+    Float4 sq[NORM ? kMaxTrips : 1];    // NORM: the chunks whose squares this thread adds
+    Float4 nw[NORM ? kMaxTrips : 1];    // NORM: the norm's weights of the chunks this thread quantizes
+    if constexpr (NORM) {
+        if (threadIdx.x < kNormThreads) {
+#pragma unroll
+            for (uint32_t k = 0; k < kMaxTrips; ++k) {
+                const uint32_t c = k * kNormThreads + threadIdx.x;
+                sq[k] = load4<true>(p.xf + (c < kChunks ? c : 0u) * 4);
+            }
+        }
+    }
+    Float4 xv[kMaxTrips];
+#pragma unroll
+    for (uint32_t t = 0; t < kMaxTrips; ++t) {
+        if (t * blockDim.x >= kChunks) break;   // workgroup-uniform: larger workgroups need fewer trips
+        const uint32_t c = t * blockDim.x + threadIdx.x;
+        const uint32_t cc = c < kChunks ? c : 0u;
+        xv[t] = vec ? load4<true>(p.xf + cc * 4) : load4<false>(p.xf + cc * 4);
+        if constexpr (NORM) nw[t] = load4<true>(p.norm_w + cc * 4);
+    }
+    asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
+    PairWeights<NSTEPS> a;
+    PairRows ra{};
+    if (live) {
+        ra = resolve_pair<SILU>(p, ps, first, row_bytes);
+        issue_pair<NSTEPS>(a, ra, lane);
+    }
+    asm volatile("" ::: "memory");   // ... and the weight loads ahead of the barriers
+    if constexpr (NORM) {
+        float partial = 0.0f;
+        if (threadIdx.x < kNormThreads) {
+#pragma unroll
+            for (uint32_t k = 0; k < kMaxTrips; ++k) {
+                const float q = chunk_squares(sq[k]);
+                partial += (k * kNormThreads + threadIdx.x < kChunks) ? q : 0.0f;
+            }
+        }
+        const float scale = rms_scale(first256_tree_sum(partial, red), nb * 32, p.eps);
+#pragma unroll
+        for (uint32_t t = 0; t < kMaxTrips; ++t) {
+            if (t * blockDim.x >= kChunks) break;
+            xv[t] = rms_apply(xv[t], scale, nw[t]);
+            const uint32_t c = t * blockDim.x + threadIdx.x;
+            if (p.normalized != nullptr && blockIdx.x == 0 && c < kChunks)
+                *reinterpret_cast<float4 *>(p.normalized + c * 4) = make_float4(xv[t].x, xv[t].y, xv[t].z, xv[t].w);
+        }
+    }
+#pragma unroll
+    for (uint32_t t = 0; t < kMaxTrips; ++t) {
+        if (t * blockDim.x >= kChunks) break;
+        const uint32_t c = t * blockDim.x + threadIdx.x;
+        float d;
+        const uint32_t packed = quantize4_q8_1(xv[t], d);   // all lanes take part in the exchanges
+        if (c < kChunks) {
+            lds_q[c] = packed;
+            if (c % 8 == 0) lds_d[c / 8] = half_bits_to_float(float_to_half_bits(d));
+        }
+    }
+    __syncthreads();
+    if (!live) return;
+    v4i xq[1][NSTEPS];
+    float dx[1][NSTEPS];
+#pragma unroll
+    for (int s = 0; s < NSTEPS; ++s) {
+        xq[0][s] = *reinterpret_cast<const v4i *>(&lds_q[s * 256 + lane * 4]);
+        dx[0][s] = lds_d[32 * s + (lane >> 1)];
+    }
+    run_pairs<1, NSTEPS, SILU, false>(p, ps, first, end, xq, dx, lane, a, ra);
+}
+
+// ---- rows of any length: a rolling pipeline over (pair, step) items -------------------------------
+// Slot d of the ring holds the two rows' 16 bytes of one step, their scales, and the activation
+// bytes and scale of that step (read from global memory with the weights: L2 serves them).  kRing
+// items are in flight; the trip count is padded to whole rings with repeats of the last item whose
+// sums are never written, so that the load counter the compiler waits on stays exact.
+constexpr int kRing = 4;
+
+template <int M, bool XF32>
+struct RingSlot {
+    v4i q0, q1;
+    v4i xq[XF32 ? 1 : M];        // unused when the activations sit in LDS
+    uint16_t d0, d1;
+    uint16_t dxh[XF32 ? 1 : M];
+};
+
+// LDS bytes of M quantized activation rows (XF32): packed int8 then fp32 scales.
+inline uint32_t ring_x_lds_bytes(uint32_t nb, uint32_t m) { return m * nb * (32 + 4); }
+
+// XF32: fp32 activations, quantized into LDS by the whole workgroup before the first item is
+// consumed (the first loads of every wave are already in flight by then); otherwise one wave per
+// workgroup and Q8_1 blocks from global memory.
+// NORM (XF32, one row): the row is RMS-normalised before it is quantized, see gemv_pairs_f32_kernel.
+template <int M, bool SILU, bool XF32, bool NORM = false>
+__global__ __launch_bounds__(XF32 ? 512 : kWave) void gemv_pairs_ring_kernel(const GemvParams p, const PairSpace ps) {
+    static_assert(!NORM || (XF32 && M == 1), "the fused norm handles one fp32 row");
+    extern __shared__ __align__(16) uint8_t smem[];
+    __shared__ float red[4];
+    const uint32_t nb = p.nb;
+    const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    const uint32_t lane = threadIdx.x % kWave;
+    const bool odd = lane & 1u;
+    const uint32_t npieces = nb * 2, nsteps = (npieces + 63) / 64;
+    const uint32_t wave_id = XF32 ? blockIdx.x * (blockDim.x / kWave) + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave)
+                                  : blockIdx.x;
+    const uint32_t first = wave_id * ps.ppw;
+    const bool live = first < ps.pairs;
+    if (!XF32 && !live) return;
+    const uint32_t end = first + ps.ppw < ps.pairs ? first + ps.ppw : ps.pairs;
+    const uint32_t n_items = live ? (end - first) * nsteps : 0u;
+    const uint32_t n_padded = (n_items + kRing - 1) / kRing * kRing;
+    uint32_t *lds_q = reinterpret_cast<uint32_t *>(smem);
+    float *lds_d = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nb * 32);
+
+    RingSlot<M, XF32> ring[kRing];
+    uint32_t ipair = first, istep = 0, ileft = n_items;
+    PairRows irows{};
+    if (live) irows = resolve_pair<SILU>(p, ps, ipair, row_bytes);
+    auto issue = [&](RingSlot<M, XF32> &sl) {
+        const uint32_t piece = istep * 64 + lane;
+        const uint32_t pc = piece < npieces ? piece : 0u;   // past the row's end: re-read its start, masked below
+        const uint32_t blk = pc >> 1;
+        sl.q0 = load_q16(irows.r0 + 2 * nb + pc * 16);
+        sl.q1 = load_q16(irows.r1 + 2 * nb + pc * 16);
+        sl.d0 = reinterpret_cast<const uint16_t *>(irows.r0)[blk];
+        sl.d1 = reinterpret_cast<const uint16_t *>(irows.r1)[blk];
+        if constexpr (!XF32) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const uint8_t *xb = p.y + static_cast<uint64_t>(m * nb + blk) * kQ81Bytes;
+                sl.xq[m] = load_x16(xb + 4 + (pc & 1u) * 16);
+                sl.dxh[m] = *reinterpret_cast<const uint16_t *>(xb);
+            }
+        }
+        if (ileft > 1) {   // otherwise: keep re-reading the last real item
+            --ileft;
+            if (++istep == nsteps) {
+                istep = 0;
+                ++ipair;
+                irows = resolve_pair<SILU>(p, ps, ipair, row_bytes);
+            }
+        }
+    };
+    if (live) {
+#pragma unroll
+        for (int d = 0; d < kRing; ++d) issue(ring[d]);
+    }
+    if constexpr (XF32) {
+        asm volatile("" ::: "memory");   // the weight loads above stay ahead of the staging
+        const uint32_t per_row = nb * 8, total = static_cast<uint32_t>(M) * per_row;   // float4 chunks
+        const bool vec = NORM || ((reinterpret_cast<uintptr_t>(p.xf) % 16 == 0) && (p.x_stride % 4 == 0));
+        float scale = 1.0f;
+        if constexpr (NORM) {
+            float partial = 0.0f;
+            if (threadIdx.x < kNormThreads)
+                for (uint32_t c = threadIdx.x; c < per_row; c += kNormThreads) partial += chunk_squares(load4<true>(p.xf + c * 4));
+            scale = rms_scale(first256_tree_sum(partial, red), nb * 32, p.eps);
+        }
+        for (uint32_t base = 0; base < total; base += blockDim.x) {
+            const uint32_t c = base + threadIdx.x;
+            const uint32_t cc = c < total ? c : 0u;
+            uint32_t m, within;
+            split_index<M>(cc, per_row, m, within);
+            const float *src = p.xf + static_cast<uint64_t>(m) * p.x_stride + within * 4;
+            Float4 v = vec ? load4<true>(src) : load4<false>(src);
+            if constexpr (NORM) {
+                v = rms_apply(v, scale, load4<true>(p.norm_w + cc * 4));
+                if (p.normalized != nullptr && blockIdx.x == 0 && c < total)
+                    *reinterpret_cast<float4 *>(p.normalized + cc * 4) = make_float4(v.x, v.y, v.z, v.w);
+            }
+            float d;
+            const uint32_t packed = quantize4_q8_1(v, d);   // all lanes take part in the exchanges
+            if (c < total) {
+                lds_q[cc] = packed;
+                if (within % 8 == 0) lds_d[m * nb + within / 8] = half_bits_to_float(float_to_half_bits(d));
+            }
+        }
+        __syncthreads();
+        if (!live) return;
+    }
+
+    float acc[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+    uint32_t cstep = 0, cpair = first;
+    for (uint32_t t = 0; t < n_padded; t += kRing) {
+#pragma unroll
+        for (int d = 0; d < kRing; ++d) {
+            const RingSlot<M, XF32> &sl = ring[d];
+            const uint32_t piece = cstep * 64 + lane;
+            const bool valid = piece < npieces;
+            const float dw = valid ? half_bits_to_float(odd ? sl.d1 : sl.d0) : 0.0f;
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                v4i xq;
+                float dxv;
+                if constexpr (XF32) {
+                    const uint32_t pc = valid ? piece : 0u;
+                    xq = *reinterpret_cast<const v4i *>(&lds_q[(m * nb) * 8 + pc * 4]);
+                    dxv = lds_d[m * nb + (pc >> 1)];
+                } else {
+                    xq = sl.xq[m];
+                    dxv = half_bits_to_float(sl.dxh[m]);
+                }
+                const int sa = dot16(sl.q0, xq);
+                const int sb = dot16(sl.q1, xq);
+                const int S = (odd ? sb : sa) + dpp_i32<kDppXor1>(odd ? sa : sb);
+                acc[m] = fmaf(dw * dxv, static_cast<float>(S), acc[m]);
+            }
+            ++cstep;
+            const uint32_t done = t + d + 1;   // items consumed so far, repeats included
+            if (cstep == nsteps && done <= n_items) {   // wave-uniform
+                float tot[M];
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    tot[m] = parity_sum(acc[m]);
+                    acc[m] = 0.0f;
+                }
+                write_pair<M, SILU>(p, resolve_pair<SILU>(p, ps, cpair, row_bytes), lane, tot);
+                cstep = 0;
+                ++cpair;
+            }
+            issue(ring[d]);
+        }
+    }
+}
+
+// ---- host side -----------------------------------------------------------------------------------
+PairSpace pair_space(const GemvParams &p, bool silu) {
+    PairSpace ps{};
+    if (silu) {
+        for (int i = 0; i < 4; ++i) ps.pair_end[i] = p.total_rows;
+        ps.pairs = p.total_rows;
+    } else {
+        uint32_t prev = 0, total = 0;
+        for (int i = 0; i < 4; ++i) {
+            total += (p.row_end[i] - prev + 1) / 2;
+            prev = p.row_end[i];
+            ps.pair_end[i] = total;
+        }
+        ps.pairs = total;
+    }
+    ps.ppw = 1;
+    return ps;
+}
+
+template <int M, int NSTEPS>
+int launch_regs(const GemvParams &p, PairSpace ps, hipStream_t stream) {
+    // One activation row: two pairs per wave once there are plenty (measured: 17408 pairs 30.2 -> 29.6 us,
+    // 2560 pairs 6.6 -> 6.8 us).  Two rows: a wave loads twice the activation bytes, so two pairs always
+    // (layer of a 27B model 93 -> 86 us; four pairs 88 us).
+    ps.ppw = (M == 2 || ps.pairs >= 8192) ? 2 : 1;
+    const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
+    if (p.mode == kSiluMul) gemv_pairs_kernel<M, NSTEPS, true><<<grid, kWave, 0, stream>>>(p, ps);
+    else gemv_pairs_kernel<M, NSTEPS, false><<<grid, kWave, 0, stream>>>(p, ps);
+    return check_launch("gemv (row pairs)");
+}
+
+template <int M>
+int launch_ring(const GemvParams &p, PairSpace ps, hipStream_t stream) {
+    ps.ppw = 2;   // measured at 17408 columns: 17.4 us against 18.0..18.8 with one pair per wave
+    const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
+    if (p.mode == kSiluMul) gemv_pairs_ring_kernel<M, true, false><<<grid, kWave, 0, stream>>>(p, ps);
+    else gemv_pairs_ring_kernel<M, false, false><<<grid, kWave, 0, stream>>>(p, ps);
+    return check_launch("gemv (row pairs, ring)");
+}
+
+// Waves per workgroup and pairs per wave of the kernels whose workgroups quantize fp32 activations
+// together: one workgroup per CU while a CU's share is at most two pairs for each of max_waves
+// waves; beyond that, workgroups of eight waves with two pairs each, handed out by the dispatcher.
+void f32_geometry(PairSpace &ps, uint32_t max_waves, uint32_t &waves, uint32_t &grid) {
+    const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+    const uint32_t share = (ps.pairs + cus - 1) / cus;
+    if (share <= 2 * max_waves) {
+        // one workgroup per CU: the fewest pairs per wave, then the wave count that wastes no slot
+        ps.ppw = (share + max_waves - 1) / max_waves;
+        waves = (share + ps.ppw - 1) / ps.ppw;
+        if (waves < 4) waves = 4;
+    } else {
+        waves = 8;
+        ps.ppw = 2;
+    }
+    const uint32_t per_wg = waves * ps.ppw;
+    grid = (ps.pairs + per_wg - 1) / per_wg;
+}
+
+template <int M>
+int launch_ring_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
+    const uint32_t lds = ring_x_lds_bytes(p.nb, M);
+    if (lds > kLdsLimit - 1024)   // rows this long keep their activations in L2 (two-step form)
+        return fail(Q8MI_REJECTED, "qgemv: %u activation rows of %u columns do not fit LDS", M, p.nb * 32);
+    uint32_t waves, grid;
+    f32_geometry(ps, 8, waves, grid);
+    auto launch = [&](auto kern) {
+        static KernelGeometry geometry;
+        if (!geometry.grant(reinterpret_cast<const void *>(kern), kLdsLimit - 1024))
+            return fail(Q8MI_LAUNCH_ERROR, "gemv (row pairs): cannot reserve %u bytes of LDS", lds);
+        kern<<<grid, waves * kWave, lds, stream>>>(p, ps);
+        return check_launch("gemv (row pairs, ring, fp32 activations)");
+    };
+    if constexpr (M == 1) {
+        if (p.norm_w != nullptr) {
+            if (p.mode == kSiluMul) return launch(gemv_pairs_ring_kernel<1, true, true, true>);
+            return launch(gemv_pairs_ring_kernel<1, false, true, true>);
+        }
+    }
+    if (p.mode == kSiluMul) return launch(gemv_pairs_ring_kernel<M, true, true>);
+    return launch(gemv_pairs_ring_kernel<M, false, true>);
+}
+
+template <int NSTEPS>
+int launch_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
+    uint32_t waves, grid;
+    if (p.norm_w != nullptr) {
+        f32_geometry(ps, 8, waves, grid);
+        if (p.mode == kSiluMul) gemv_pairs_f32_kernel<NSTEPS, true, true><<<grid, waves * kWave, 0, stream>>>(p, ps);
+        else gemv_pairs_f32_kernel<NSTEPS, false, true><<<grid, waves * kWave, 0, stream>>>(p, ps);
+        return check_launch("gemv (row pairs, fp32 activations, fused norm)");
+    }
+    f32_geometry(ps, 16, waves, grid);
+    if (p.mode == kSiluMul) gemv_pairs_f32_kernel<NSTEPS, true, false><<<grid, waves * kWave, 0, stream>>>(p, ps);
+    else gemv_pairs_f32_kernel<NSTEPS, false, false><<<grid, waves * kWave, 0, stream>>>(p, ps);
+    return check_launch("gemv (row pairs, fp32 activations)");
+}
+
+}  // namespace
+
+int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
+    if (batch == 0 || batch > 2 || p.nb % 8 != 0) return Q8MI_REJECTED;
+    if (p.norm_w != nullptr) {   // fused norm + quantizer: one row, at most kMaxNormCols columns
+        constexpr uint32_t kMaxNormCols = 6144;
+        if (batch != 1) return fail(Q8MI_REJECTED, "nqgemv: batch %u above 1 (normalise and quantize once, then use the GEMV)", batch);
+        if (p.nb * kQK > kMaxNormCols)
+            return fail(Q8MI_REJECTED, "nqgemv: rows of %u columns are not served (at most %u)", p.nb * kQK, kMaxNormCols);
+        auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+        if (!al(p.xf) || !al(p.norm_w) || (p.normalized != nullptr && !al(p.normalized)))
+            return fail(Q8MI_REJECTED, "nqgemv: activations, norm weights and normalised output must be 16-byte aligned");
+    }
+    const PairSpace ps = pair_space(p, p.mode == kSiluMul);
+    if (ps.pairs == 0) return Q8MI_REJECTED;
+    const uint32_t cols = p.nb * kQK;
+    if (p.xf != nullptr) {
+        if (batch == 1) {
+            switch (cols) {
+                case 4096: return launch_f32<4>(p, ps, stream);
+                case 5120: return launch_f32<5>(p, ps, stream);
+                case 6144: return launch_f32<6>(p, ps, stream);
+                default: return launch_ring_f32<1>(p, ps, stream);
+            }
+        }
+        return launch_ring_f32<2>(p, ps, stream);
+    }
+    if (reinterpret_cast<uintptr_t>(p.y) % 4 != 0) return Q8MI_REJECTED;
+    if (batch == 1) {
+        switch (cols) {
+            case 4096: return launch_regs<1, 4>(p, ps, stream);
+            case 5120: return launch_regs<1, 5>(p, ps, stream);
+            case 6144: return launch_regs<1, 6>(p, ps, stream);
+            case 8192: return launch_regs<1, 8>(p, ps, stream);
+            default: return launch_ring<1>(p, ps, stream);
+        }
+    }
+    switch (cols) {
+        case 4096: return launch_regs<2, 4>(p, ps, stream);
+        case 5120: return launch_regs<2, 5>(p, ps, stream);
+        case 6144: return launch_regs<2, 6>(p, ps, stream);
+        default: return launch_ring<2>(p, ps, stream);
+    }
+}
+
+}  // namespace q8mi

@@ -12,6 +12,7 @@ SOURCES = [
     "q8mi_host.hip",
     "q8mi_quantize.hip",
     "q8mi_gemv.hip",
+    "q8mi_gemv_pairs.hip",
     "q8mi_lm_head.hip",
     "q8mi_argmax.hip",
     "q8mi_get_rows.hip",
