@@ -27,6 +27,8 @@ constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
 constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
 constexpr int kDppRowHalfMirror = 0x141;
 constexpr int kDppRowMirror = 0x140;
+constexpr int kDppRowShl4 = 0x104;     // lane i of every row of 16 reads lane i + 4
+constexpr int kDppRowShr4 = 0x114;     // lane i of every row of 16 reads lane i - 4
 
 template <int CTRL>
 __device__ __forceinline__ int dpp_i32(int v) {

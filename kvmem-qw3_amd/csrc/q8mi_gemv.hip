@@ -112,7 +112,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
 // ---- matrix-core variant for batch 3..32 (see q8mi_gemv_mfma_core.hpp) --------------------------
 // Unit u covers rows 4u .. 4u+3 of the concatenated row space; for SwiGLU gate rows 2u, 2u+1
 // (fragment rows 0, 1) and the matching up rows (fragment rows 2, 3).
-template <int MG, int THREADS, bool SILU, bool HS, bool D4, int DEPTH>
+template <int MG, int THREADS, bool SILU, bool HS, bool D4, int DEPTH, bool STREAMING>
 __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, uint32_t batch,
                                                             uint32_t park_floats) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
     constexpr uint32_t kPerUnit = 4 * kMfmaUnitRows * MP;   // [chunk][row][activation row]
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, r = lane & 3u;
+    const uint32_t c = lane >> 2, r = lane & 3u;   // after the stream: chunk and fragment row of lanes 0 .. 15
     const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
     const uint64_t row_bytes = static_cast<uint64_t>(p.nb) * 34;
     const UnitSeq useq = group_units(p.units, blockIdx.x, gridDim.x, p.interleave);
@@ -133,20 +133,20 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
     float *my_park = park_base + wave * park_floats;
     const uint32_t last_row = p.total_rows - 1;
 
-    auto row_ptr = [&](uint32_t u) -> const uint8_t * {   // fragment row q is the one this lane loads
+    auto row_ptr = [&](uint32_t u) -> const uint8_t * {   // fragment row r is the one this lane loads
         if constexpr (SILU) {
-            uint32_t row = 2 * u + (q & 1u);
+            uint32_t row = 2 * u + (r & 1u);
             row = row < last_row ? row : last_row;
-            return (q < 2 ? p.w[0] : p.w[1]) + row * row_bytes;
+            return (r < 2 ? p.w[0] : p.w[1]) + row * row_bytes;
         } else {
-            uint32_t row = 4 * u + q;
+            uint32_t row = 4 * u + r;
             row = row < last_row ? row : last_row;
             const RowRef a = resolve_row(p, row);
             return a.w + a.local * row_bytes;
         }
     };
     auto park = [&](uint32_t kk, auto &acc) {
-        if (q == c) {
+        if (lane < 16) {
             float *dst = my_park + kk * kPerUnit + (c * kMfmaUnitRows + r) * MP;
 #pragma unroll
             for (int g = 0; g < MG; ++g) {
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
             }
         }
     };
-    mfma_stream<MG, THREADS, HS, D4, DEPTH>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
+    mfma_stream<MG, THREADS, HS, D4, DEPTH, STREAMING>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
     __syncthreads();
 
     // unit ranges of the waves, worked out once (wave w touched unit ordinals kf[w] .. kl[w])
@@ -294,11 +294,16 @@ constexpr uint64_t kMfmaShallowMaxRows = 65536;
 template <int MG, bool SILU, bool HS, bool D4, int DEPTH>
 int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     constexpr int THREADS = 512;
-    auto kern = gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH>;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
     p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG, HS);
     p.interleave = kGemvInterleave;
+    // the streaming hint pays on long streams only (measured at batch 4: 2 x 17408 x 5120 36.2 -> 33.6 us,
+    // 5120 x 17408 22.0 -> 20.6 us, but 8192 x 5120 11.7 -> 12.5 us and 5120 x 6144 10.1 -> 10.8 us)
+    constexpr uint64_t kStreamFrom = 64ull * 1000 * 1000;
+    const bool streaming = (SILU ? 2ull : 1ull) * p.total_rows * p.nb * 34 >= kStreamFrom;
+    auto kern = streaming ? gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, true>
+                          : gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, false>;
     const uint32_t grid = p.units < cus ? p.units : cus;
     const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
     const uint32_t per_group = (p.units + grid - 1) / grid;
@@ -306,8 +311,8 @@ int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     const uint32_t lds = p.x_bytes + (THREADS / kWave) * park_floats * 4;
     constexpr uint32_t kDynLimit = kLdsLimit - 256;   // the kernel also has a few static LDS words
     if (lds > kDynLimit) return fail(Q8MI_REJECTED, "gemv (matrix-core variant): %u bytes of LDS needed", lds);
-    static KernelGeometry geometry;
-    if (!geometry.grant(reinterpret_cast<const void *>(kern), kDynLimit))
+    static KernelGeometry geometry[2];
+    if (!geometry[streaming].grant(reinterpret_cast<const void *>(kern), kDynLimit))
         return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
     kern<<<grid, THREADS, lds, stream>>>(p, batch, park_floats);
     return check_launch("gemv_mfma");
@@ -357,7 +362,7 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         const int rc = launch_pairs(p, batch, stream);
         if (rc != Q8MI_REJECTED) return rc;
     }
-    if (p.xf == nullptr && reinterpret_cast<uintptr_t>(p.y) % 16 == 0 &&
+    if (p.xf == nullptr && reinterpret_cast<uintptr_t>(p.y) % 4 == 0 &&
         batch >= kMfmaFromBatch &&
         (mfma_fits(p.nb, batch, false) || mfma_fits(p.nb, batch, true))) {
         const int rc = launch_mfma_any(p, batch, stream);

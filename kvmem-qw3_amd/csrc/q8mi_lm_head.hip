@@ -146,7 +146,7 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
     constexpr uint32_t kPerUnit = 4 * kMfmaUnitRows * MP;   // [chunk][row][activation row]
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const uint32_t q = lane >> 4, c = (lane >> 2) & 3u, r = lane & 3u;
+    const uint32_t c = lane >> 2, r = lane & 3u;   // after the stream: chunk and fragment row of lanes 0 .. 15
     const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
     const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
     const uint32_t units = (rows + kMfmaUnitRows - 1) / kMfmaUnitRows;
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
     for (uint32_t m = 0; m < MP; ++m) { bv[m] = -INFINITY; bi[m] = -1; }
 
     auto row_ptr = [&](uint32_t u) -> const uint8_t * {
-        uint32_t row = kMfmaUnitRows * u + q;
+        uint32_t row = kMfmaUnitRows * u + r;
         row = row < rows - 1 ? row : rows - 1;
         return w + row * row_bytes;
     };
@@ -179,11 +179,11 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
             for (int g = 0; g < MG; ++g) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    // chunk c of fragment row r sits in lane 20 c + r
+                    // chunk c of fragment row r sits in lane 4 c + r
                     const float e0 = acc[g][v];
-                    const float e1 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((20 + r) * 4), as_i32(e0)));
-                    const float e2 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((40 + r) * 4), as_i32(e0)));
-                    const float e3 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((60 + r) * 4), as_i32(e0)));
+                    const float e1 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((4 + r) * 4), as_i32(e0)));
+                    const float e2 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((8 + r) * 4), as_i32(e0)));
+                    const float e3 = as_f32(__builtin_amdgcn_ds_bpermute(static_cast<int>((12 + r) * 4), as_i32(e0)));
                     const float s = 0.0f + (((e0 + e1) + e2) + e3);   // the sum the combine below forms
                     const uint32_t m = 4 * g + v;
                     if (lane < kMfmaUnitRows && static_cast<uint32_t>(row) < rows && m < batch) {
@@ -192,7 +192,7 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
                     }
                 }
             }
-        } else if (q == c) {
+        } else if (lane < 16) {
             float *dst = my_park + (k == kf_mine ? 0 : 1) * kPerUnit + (c * kMfmaUnitRows + r) * MP;
 #pragma unroll
             for (int g = 0; g < MG; ++g) {
@@ -375,15 +375,16 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
     return check_launch("lm_head");
 }
 
-// Matrix-core variant: for weights of up to 65536 rows under the GEMV's own rule (same kernel
-// family and geometry as q8mi_gemv at that batch, so the optional logits are the GEMV's bits), for
-// taller ones (the vocabulary) only from 7 verify rows on: there the dot-product variant streams
-// faster up to 6 rows (measured: 237..257 us against 245..265 us at 4..6 rows, 296 against 265 at 8).
+// Which variant streams the weight: the matrix-core one from 3 verify rows on (the same family and
+// geometry as q8mi_gemv at that batch, so the optional logits are the GEMV's bits) whenever the
+// activations fit LDS beside the parked sums.  Measured on the 248 320-row vocabulary, dot-product
+// against matrix-core variant: 220 / 209 us at 3 rows, 216 / 212 at 4, 227 / 221 at 5, 234 / 225 at 6,
+// 296 / 230 at 8.
 bool lm_head_uses_mfma(uint32_t rows, uint32_t nb, uint32_t batch) {
+    (void)rows;
     const uint32_t mg = (batch + 3) / 4;
     if (batch < kMfmaFromBatch) return false;
-    if (mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u > kLdsLimit - 256) return false;
-    return rows <= 65536u || batch >= 7;
+    return mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u <= kLdsLimit - 256;
 }
 
 template <int M>
@@ -422,7 +423,7 @@ static int lm_head_run(const uint8_t *weight, const void *y, uint32_t rows, uint
     const auto *yb = static_cast<const uint8_t *>(y);
     hipStream_t s = as_stream(stream);
     int rc = Q8MI_REJECTED;
-    if (reinterpret_cast<uintptr_t>(yb) % 16 == 0 && lm_head_uses_mfma(rows, nb, batch)) {
+    if (reinterpret_cast<uintptr_t>(yb) % 4 == 0 && lm_head_uses_mfma(rows, nb, batch)) {
         rc = batch <= 4 ? launch_lm_head_mfma<1>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s)
                         : launch_lm_head_mfma<2>(weight, yb, rows, nb, batch, partial, logits, stride_logits, &grid, s);
     }

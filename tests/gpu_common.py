@@ -40,15 +40,16 @@ def quantize_d4(x, cols=None, stride=None, stream=NULL):
     return dy, dy.download(np.uint8, n)
 
 
-# what -> {"n", "max_rel", "beyond_rel"}: filled by assert_close_fp32, written out as JSON when the
+# what -> {"n", "max_rel", "beyond_rel", "max_of_bound", "max_of_floor"}: filled by assert_close_fp32, written out as JSON when the
 # test session ends (tests/conftest.py)
 TOLERANCE_STATS = {}
 
 
-def _record(what, err, ref, rel):
+def _record(what, err, ref, rel, lim, floor_term):
     """Per check family (the text of `what` up to its first digit): the largest relative error
-    seen and how many outputs were beyond rel*|ref| alone, i.e. passed only through the
-    sum|t_kb| term of the bound."""
+    seen, how many outputs were beyond rel*|ref| alone, i.e. passed only through the
+    sum|t_kb| term of the bound, the largest share of the whole bound any output used, and
+    the largest error in units of the sum|t_kb| term (how much of that term is needed)."""
     key = what
     for i, ch in enumerate(what):
         if ch.isdigit():
@@ -57,10 +58,16 @@ def _record(what, err, ref, rel):
     live = np.abs(ref) > 0
     relerr = np.zeros_like(err)
     relerr[live] = err[live] / np.abs(ref[live])
-    s = TOLERANCE_STATS.setdefault(key, {"n": 0, "max_rel": 0.0, "beyond_rel": 0})
+    s = TOLERANCE_STATS.setdefault(key, {"n": 0, "max_rel": 0.0, "beyond_rel": 0, "max_of_bound": 0.0,
+                                         "max_of_floor": 0.0})
     s["n"] += int(err.size)
     s["max_rel"] = max(s["max_rel"], float(relerr.max()) if err.size else 0.0)
     s["beyond_rel"] += int(np.count_nonzero(err > rel * np.abs(ref)))
+    ok_lim, ok_floor = lim > 0, floor_term > 0
+    if ok_lim.any():
+        s["max_of_bound"] = max(s["max_of_bound"], float((err[ok_lim] / lim[ok_lim]).max()))
+    if ok_floor.any():
+        s["max_of_floor"] = max(s["max_of_floor"], float((err[ok_floor] / floor_term[ok_floor]).max()))
 
 
 def assert_close_fp32(got, ref, absum, what, rel=1e-5, floor=1e-6):
@@ -76,7 +83,7 @@ def assert_close_fp32(got, ref, absum, what, rel=1e-5, floor=1e-6):
     absum = np.asarray(absum, np.float64).reshape(-1)
     err = np.abs(got - ref)
     lim = rel * np.abs(ref) + floor * absum
-    _record(what, err, ref, rel)
+    _record(what, err, ref, rel, lim, floor * absum)
     bad = np.nonzero(~(err <= lim))[0]
     if bad.size:
         i = bad[0]
