@@ -97,17 +97,19 @@ int q8mi_gemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uint
 /* ---- GEMV with the Q8_1 quantizer fused in (batch 1..2) --------------------
  * The results of q8mi_quantize_q8_1 followed by the matching q8mi_gemv* call,
  * in one launch: every workgroup quantizes the fp32 activations
- * (x: [batch][stride_x_row] floats) while it stages them in LDS, so no Q8_1
- * scratch buffer and no quantizer launch are needed.  The quantized values
- * and the per-block products are the same bits; for rows of up to 8192
- * columns so are the outputs, longer rows run with another workgroup size and
- * add the same products in another order (inside the GEMV's tolerance).  This is what
+ * (x: [batch][stride_x_row] floats) into LDS with the quantizer's own code
+ * before its waves stream their weight rows, so no Q8_1 scratch buffer and no
+ * quantizer launch are needed.  The quantized values and the per-block
+ * products are the same bits as in the two-step form.  At batch 1 so are the
+ * outputs for rows of up to 8192 columns; longer rows, and batch 2 (where the
+ * Q8_1 entry points may run another kernel), add the same products in another
+ * order (inside the GEMV's tolerance).  This is what
  * the reference's operators do in two steps (src/kernels_cuda.cu:10764-10888,
  * 11244-11302, 12035-12069, 12227-12258: launch_quantize_q8_1 then the
  * launcher); the fusion itself has no counterpart in the reference.
  * Q8MI_REJECTED (nothing launched; use the two-step form) when batch is above
- * 2 (every workgroup repeats the quantization, which stops paying there), when
- * cols is not a multiple of 256, or when the activation rows do not fit LDS.  dst_is_bf16: 0 = fp32 outputs, 1 = bf16 bit patterns. */
+ * 2 (every workgroup repeats the quantization, which stops paying there) or
+ * cols is not a multiple of 256.  dst_is_bf16: 0 = fp32 outputs, 1 = bf16 bit patterns. */
 int q8mi_qgemv(const uint8_t *weight, const float *x, uint32_t stride_x_row, void *dst, int dst_is_bf16,
                uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
 int q8mi_qgemv_add(const uint8_t *weight, const float *x, uint32_t stride_x_row, void *dst, int dst_is_bf16,

@@ -358,15 +358,17 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         gemv_unaligned_kernel<<<grid, 256, 0, stream>>>(p, batch);
         return check_launch("gemv_unaligned");
     }
+    const uint64_t row_pairs = p.mode == kSiluMul ? p.total_rows : (p.total_rows + 1) / 2;
+    const bool mfma_first = p.xf == nullptr && gemv_prefers_mfma(row_pairs, batch) &&
+                            reinterpret_cast<uintptr_t>(p.y) % 4 == 0 &&
+                            (mfma_fits(p.nb, batch, false) || mfma_fits(p.nb, batch, true));
+    if (mfma_first) {
+        const int rc = launch_mfma_any(p, batch, stream);
+        if (rc != Q8MI_REJECTED) return rc;   // a unit list whose parked sums do not fit: below
+    }
     if (batch <= 2) {   // whole row pairs per wave, handed out by the dispatcher (q8mi_gemv_pairs.hip)
         const int rc = launch_pairs(p, batch, stream);
         if (rc != Q8MI_REJECTED) return rc;
-    }
-    if (p.xf == nullptr && reinterpret_cast<uintptr_t>(p.y) % 4 == 0 &&
-        batch >= kMfmaFromBatch &&
-        (mfma_fits(p.nb, batch, false) || mfma_fits(p.nb, batch, true))) {
-        const int rc = launch_mfma_any(p, batch, stream);
-        if (rc != Q8MI_REJECTED) return rc;   // a unit list whose parked sums do not fit: dot-product variant
     }
     switch (batch) {
         case 1: return launch_m<1>(p, stream);

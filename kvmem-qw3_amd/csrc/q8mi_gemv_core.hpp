@@ -545,7 +545,14 @@ __host__ __device__ inline uint32_t max_units_touched(uint32_t group_units_max, 
 // (neighbouring workgroups read neighbouring rows), the matrix-core variant from batch 3 on.
 constexpr uint32_t kGemvWgsPerCu = 2;
 constexpr int kGemvInterleave = 1;        // unit assignment, see group_units
-constexpr uint32_t kMfmaFromBatch = 3;    // smallest batch served by the matrix-core variant
+constexpr uint32_t kMfmaFromBatch = 2;    // smallest batch served by the matrix-core variant
+// Batch 2 goes to the matrix cores unless the launch has row pairs enough to fill the chip with
+// independent waves (measured at batch 2, row-pair against matrix-core kernel: 8192 x 5120 fan-out
+// 14.1 / 11.9 us, 5120 x 6144 11.5 / 10.2, 5120 x 17408 21.0 / 20.0, but SwiGLU 2 x 17408 x 5120
+// 31.9 / 34.1); from batch 3 on always.
+inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch) {
+    return batch >= 3 || (batch == 2 && row_pairs < 8192);
+}
 
 // Per kernel instantiation (one static instance each): the dynamic LDS limit is raised once, to
 // the most any launch of this kernel may ask for and never lowered again, so launches from
