@@ -309,6 +309,53 @@ def bench_config0(q8mi, hip, synth, copies=48, reps=480):
             "fp32_activations_quantizer_plus_gemv_us": round(t_two * 1e3, 3)}
 
 
+def bench_launches_m1(q8mi, hip, synth, step, layers, reps=300):
+    """Every launch of the M=1 step on its own, back to back over the rotating weight copies, beside
+    a plain streaming read of the same number of bytes (windows of a 1 GiB buffer, so the
+    memory-side cache cannot serve it): time, bytes, rate, and time / read time."""
+    L, ok, m = q8mi.lib(), q8mi.ok, 1
+    big, sink = hip.DeviceBuffer(1 << 30), hip.DeviceBuffer(64)
+    nl = len(layers)
+
+    def probe_us(nbytes):
+        span = (nbytes + 4095) // 4096 * 4096
+        windows = (1 << 30) // span
+        fn = lambda i: synth.ok(synth.lib().q8sup_probe_read(big.at((i % windows) * span), nbytes, 2, sink.ptr, None),
+                                "probe_read")
+        return time_loop(hip, fn, reps, 20) * 1e3
+
+    def fan(i):
+        w = layers[i % nl].w
+        ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, step.y5120.ptr, step.q.ptr, step.k.ptr,
+                               step.v.ptr, None, QDIM, KVDIM, KVDIM, 0, HIDDEN, m, QDIM, KVDIM, KVDIM, 0, None), "fanout4")
+    ops = [
+        ("quantize_q8_1 x (5120 floats)", 0,
+         lambda i: ok(L.q8mi_quantize_q8_1(step.x.ptr, step.y5120.ptr, m, HIDDEN, HIDDEN, None), "quantize")),
+        ("gemv_fanout4 q/k/v 8192x5120", w_bytes(QDIM + 2 * KVDIM, HIDDEN), fan),
+        ("qgemv_add o 5120x6144 (fp32 in)", w_bytes(HIDDEN, ATTN_OUT),
+         lambda i: ok(L.q8mi_qgemv_add(layers[i % nl].w["o"].ptr, step.attn.ptr, ATTN_OUT, step.h.ptr, 0, HIDDEN,
+                                       ATTN_OUT, m, HIDDEN, None), "qo")),
+        ("gemv_silu_mul gate/up 2x17408x5120", 2 * w_bytes(FFN, HIDDEN), lambda i: step.run_silu(layers[i % nl])),
+        ("quantize_q8_1 ffn (17408 floats)", 0,
+         lambda i: ok(L.q8mi_quantize_q8_1(step.ffn.ptr, step.y17408.ptr, m, FFN, FFN, None), "quantize")),
+        ("gemv_add down 5120x17408", w_bytes(HIDDEN, FFN),
+         lambda i: ok(L.q8mi_gemv_add(layers[i % nl].w["down"].ptr, step.y17408.ptr, step.h.ptr, HIDDEN, FFN, m,
+                                      HIDDEN, None), "down")),
+    ]
+    step.prepare_silu()
+    out = []
+    for name, nbytes, fn in ops:
+        us = time_loop(hip, fn, reps, 20) * 1e3
+        row = {"launch": name, "weight_bytes": nbytes, "us": round(us, 2)}
+        if nbytes:
+            pus = probe_us(nbytes)
+            row.update({"gbps": round(nbytes / us / 1e3, 1), "plain_read_us": round(pus, 2), "ratio": round(us / pus, 3)})
+        out.append(row)
+    big.free()
+    sink.free()
+    return out
+
+
 def bench_read_probe(synth, hip, nbytes=1 << 30, reps=20):
     """Measured ceiling of a plain streaming read (every lane 16 bytes per load, grid-stride)."""
     buf, sink = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(64)
@@ -411,7 +458,7 @@ def bench_lm_head(q8mi, hip, synth, reps=100):
     return out
 
 
-TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv_silu_m1_hbm_traffic.txt")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv_pairs_silu_m1_hbm_traffic.txt")
 COPY_BYTES = 1 << 28
 
 
@@ -534,6 +581,7 @@ def main():
             t = time_loop(hip, lambda i: step.run_with_norms(layers[i % len(layers)], one), max(args.steps // 2, 20), 5)
             norms[name] = {"ms_per_step": round(t, 5), "gbps": round(step_bytes / (t * 1e-3) / 1e9, 1)}
         result["layer_with_rms_norms_m1"] = norms
+        result["launches_m1"] = bench_launches_m1(q8mi, hip, synth, step, layers)
     for l in layers[1:]:
         for b in l.w.values():
             b.free()

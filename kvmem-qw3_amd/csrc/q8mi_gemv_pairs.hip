@@ -26,6 +26,8 @@
 // activations (the entry points that quantize inside the GEMV) are quantized once per workgroup
 // into LDS by all of its waves, with the stand-alone quantizer's code, and then read into the
 // same registers.
+#include <type_traits>
+
 #include "q8mi_gemv_core.hpp"
 #include "q8mi_gemv_params.hpp"
 
@@ -332,7 +334,7 @@ __global__ __launch_bounds__(NORM ? 512 : 1024) void gemv_pairs_f32_kernel(const
 // bytes and scale of that step (read from global memory with the weights: L2 serves them).  kRing
 // items are in flight; the trip count is padded to whole rings with repeats of the last item whose
 // sums are never written, so that the load counter the compiler waits on stays exact.
-constexpr int kRing = 4;
+constexpr int kRing = 4;   // 6 changes nothing, 8 is slower (19.4 against 18.1 us at 5120 x 17408)
 
 template <int M, bool XF32>
 struct RingSlot {
@@ -483,6 +485,116 @@ __global__ __launch_bounds__(XF32 ? 512 : kWave) void gemv_pairs_ring_kernel(con
     }
 }
 
+// ---- long rows of NSTEPS KiB: the waves of a workgroup share every pair -----------------------------
+// A row of 17 KiB is too long for one wave's registers, and a wave that streams it alone re-reads the
+// activations from L2 step by step (as much L1 traffic again as the weights).  Here the WAVES waves of
+// a workgroup cut every row into interleaved 1 KiB steps: wave w takes steps w, w + WAVES, ... and a
+// 1 / WAVES share of the steps that remain (its first lanes only), so each wave needs the
+// activations of its own steps only, once, in registers, for all the pairs of the workgroup, and
+// the workgroup as a whole reads each pair as one contiguous stretch.  A slot is refilled with the
+// next pair's bytes as soon as it is consumed.  The waves' partial sums meet in LDS after the last
+// pair (one barrier per workgroup), added in wave order.
+template <int M, int NSTEPS, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave, 5) void gemv_pairs_ksplit_kernel(const GemvParams p, const PairSpace ps) {
+    constexpr uint32_t nb = NSTEPS * 32;
+    constexpr uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    constexpr int S = NSTEPS / WAVES;                              // whole steps per wave
+    constexpr uint32_t kTail = (NSTEPS - S * WAVES) * 64 / WAVES;  // 16-byte pieces per wave of the steps left over
+    static_assert((NSTEPS - S * WAVES) * 64 % WAVES == 0 && kTail % 2 == 0, "the left-over steps split evenly");
+    constexpr int SL = S + (kTail ? 1 : 0);                        // register slots per wave
+    constexpr uint32_t kMaxPairs = 4;
+    __shared__ float part[kMaxPairs][WAVES][M][2];
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const bool odd = lane & 1u;
+    const uint32_t first = blockIdx.x * ps.ppw;
+    if (first >= ps.pairs) return;
+    const uint32_t end = first + ps.ppw < ps.pairs ? first + ps.ppw : ps.pairs;
+    // the 16-byte piece of a row this lane owns in slot j, and whether the slot is live in this lane
+    auto piece_of = [&](int j) -> uint32_t {
+        return j < S ? (static_cast<uint32_t>(j) * WAVES + w) * 64 + lane : static_cast<uint32_t>(S) * WAVES * 64 + w * kTail + lane;
+    };
+    auto live_in = [&](int j) -> bool { return j < S || lane < kTail; };
+
+    v4i xq[M][SL];
+    uint16_t dxh[M][SL];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int j = 0; j < SL; ++j) {
+            xq[m][j] = v4i{0, 0, 0, 0};
+            dxh[m][j] = 0;
+            if (live_in(j)) {
+                const uint32_t piece = piece_of(j);
+                const uint8_t *blk = p.y + static_cast<uint64_t>(m * nb + (piece >> 1)) * kQ81Bytes;
+                xq[m][j] = load_x16(blk + 4 + (piece & 1u) * 16);
+                dxh[m][j] = *reinterpret_cast<const uint16_t *>(blk);
+            }
+        }
+    v4i q0[SL], q1[SL];
+    uint16_t d0[SL], d1[SL];
+    auto issue = [&](int j, const PairRows &rows) {
+        const uint32_t piece = live_in(j) ? piece_of(j) : 0u;   // dead lanes of the tail slot: piece 0, zero activation scale
+        q0[j] = load_q16(rows.r0 + 2 * nb + piece * 16);
+        q1[j] = load_q16(rows.r1 + 2 * nb + piece * 16);
+        d0[j] = reinterpret_cast<const uint16_t *>(rows.r0)[piece >> 1];
+        d1[j] = reinterpret_cast<const uint16_t *>(rows.r1)[piece >> 1];
+    };
+    PairRows rows = resolve_pair<false>(p, ps, first, row_bytes);
+#pragma unroll
+    for (int j = 0; j < SL; ++j) issue(j, rows);
+    float dx[M][SL];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int j = 0; j < SL; ++j) dx[m][j] = half_bits_to_float(dxh[m][j]);
+
+    // one pair: REFILL = its slots are refilled with the next pair's bytes as they are consumed (every
+    // pair but the last; a separate copy of the loop body, so that no branch sits between the loads
+    // and the compiler's load counters stay exact)
+    auto do_pair = [&](uint32_t pair, auto refill_tag) {
+        constexpr bool REFILL = decltype(refill_tag)::value;
+        PairRows next = rows;
+        if constexpr (REFILL) next = resolve_pair<false>(p, ps, pair + 1, row_bytes);
+        float acc[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < SL; ++j) {
+            const float dw = half_bits_to_float(odd ? d1[j] : d0[j]);
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const int sa = dot16(q0[j], xq[m][j]);
+                const int sb = dot16(q1[j], xq[m][j]);
+                const int sum = (odd ? sb : sa) + dpp_i32<kDppXor1>(odd ? sa : sb);
+                acc[m] = fmaf(dw * dx[m][j], static_cast<float>(sum), acc[m]);
+            }
+            if constexpr (REFILL) {
+                issue(j, next);
+                __builtin_amdgcn_sched_barrier(0);   // the refill stays here: the compiler otherwise gathers all refills after the last slot
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const float tot = parity_sum(acc[m]);
+            if (lane < 2) part[pair - first][w][m][lane] = tot;
+        }
+        rows = next;
+    };
+    for (uint32_t pair = first; pair + 1 < end; ++pair) do_pair(pair, std::true_type{});
+    do_pair(end - 1, std::false_type{});
+    __syncthreads();
+    const uint32_t n = (end - first) * M * 2;
+    if (threadIdx.x < n) {
+        const uint32_t k = threadIdx.x / (2 * M), m = (threadIdx.x / 2) % M, r = threadIdx.x % 2;
+        float tot = 0.0f;
+#pragma unroll
+        for (int v = 0; v < WAVES; ++v) tot += part[k][v][m][r];
+        const PairRows out = resolve_pair<false>(p, ps, first + k, row_bytes);
+        if (r == 0 || out.two) store_out(p.mode, out.dst, static_cast<uint64_t>(m) * out.stride + out.row0 + r, tot);
+    }
+}
+
 // ---- host side -----------------------------------------------------------------------------------
 PairSpace pair_space(const GemvParams &p, bool silu) {
     PairSpace ps{};
@@ -512,6 +624,14 @@ int launch_regs(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     if (p.mode == kSiluMul) gemv_pairs_kernel<M, NSTEPS, true><<<grid, kWave, 0, stream>>>(p, ps);
     else gemv_pairs_kernel<M, NSTEPS, false><<<grid, kWave, 0, stream>>>(p, ps);
     return check_launch("gemv (row pairs)");
+}
+
+template <int M, int NSTEPS, int WAVES>
+int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
+    ps.ppw = 2;   // measured at 5120 x 17408: 16.9 us; one pair 17.8, three 18.1, four 17.9
+    const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
+    gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
+    return check_launch("gemv (row pairs, rows shared by the waves of a workgroup)");
 }
 
 template <int M>
@@ -615,6 +735,9 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
             case 5120: return launch_regs<1, 5>(p, ps, stream);
             case 6144: return launch_regs<1, 6>(p, ps, stream);
             case 8192: return launch_regs<1, 8>(p, ps, stream);
+            case 17408:   // four waves per pair (two waves spill, eight: 17.1 us against 16.9)
+                if (p.mode != kSiluMul) return launch_ksplit<1, 17, 4>(p, ps, stream);
+                return launch_ring<1>(p, ps, stream);
             default: return launch_ring<1>(p, ps, stream);
         }
     }
