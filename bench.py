@@ -496,7 +496,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
     ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["gemm", "lm_head"], help="one secondary figure alone (for profiling runs)")
+    ap.add_argument("--only", choices=["gemm", "lm_head", "ceilings"], help="one secondary figure alone (for profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's throughput; run with --gpus 1 "
@@ -513,6 +513,9 @@ def main():
     if args.only == "gemm":
         print(json.dumps({"gemm_int8": bench_gemm(q8mi, hip, synth, reps=10),
                           "gemm_medium_batches": bench_gemm_medium(q8mi, hip, synth)}))
+        return
+    if args.only == "ceilings":
+        print(json.dumps({"measured_ceilings": bench_mfma_ceilings(synth, hip)}))
         return
     if args.only == "lm_head":
         print(json.dumps({"lm_head_fused": bench_lm_head(q8mi, hip, synth)}))
