@@ -217,9 +217,11 @@ def test_gemv_fused_variants(gpu, oracle, batch):
     assert diff.max() <= 1 and (diff != 0).mean() < 0.01
 
 
-@pytest.mark.parametrize("batch", [1, 3, 8])
-def test_gemv_fanout4(gpu, oracle, batch):
-    cols = 1024
+# columns: a streamed row length, one whose activations stay in registers at batch 1..2, and the
+# 17 KiB rows that the waves of a workgroup share at batch 1 (odd row counts end in a single-row pair)
+@pytest.mark.parametrize("cols", [1024, 5120, 17408])
+@pytest.mark.parametrize("batch", [1, 2, 3, 8])
+def test_gemv_fanout4(gpu, oracle, batch, cols):
     rows = [96, 0, 17, 130]           # slot 1 is empty, as when the executor passes 3 weights
     ws = [synth.q8_0_weight(r, cols, seed=50 + i) if r else None for i, r in enumerate(rows)]
     x = synth.normal(batch, cols, seed=77)
