@@ -68,9 +68,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
     auto park = [&](uint32_t kk, float total) {
         if (lane < kPerUnit) my_park[kk * kPerUnit + lane] = total;
     };
-    // the reduction of the fused norm borrows the first floats of the park area, which is not
-    // written before the staging barrier
-    const XIn in{p.y, p.xf, p.x_stride, p.norm_w, p.eps, p.normalized, park_base};
+    const XIn in{p.y};
     gemv_stream<M, R, THREADS, XMODE>(smem, in, p.nb, useq, i0, i1, rows_of, park);
     __syncthreads();
 

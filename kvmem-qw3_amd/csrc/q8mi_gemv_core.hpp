@@ -48,20 +48,13 @@ constexpr int kDepth = Q8MI_GEMV_DEPTH;        // items in flight per wave
 constexpr uint32_t kLdsLimit = 160u * 1024u;    // LDS per CU on gfx950
 constexpr uint32_t kParkFloats = 1024;           // per-wave LDS area (floats) for the sums of the units it touched
 
-// Where a lane finds the activations: Q8_1 blocks staged in LDS, Q8_1 blocks read from
-// global memory, fp32 activations quantized to Q8_1 while they are staged in LDS, or one fp32
-// row that is RMS-normalised and then quantized while it is staged.
-enum XMode : int { kXLds = 0, kXGlobal = 1, kXF32 = 2, kXNormF32 = 3 };
+// Where a lane finds the activations: Q8_1 blocks staged in LDS, or Q8_1 blocks read from
+// global memory.  (fp32 activations are served by the row-pair kernels of q8mi_gemv_pairs.hip.)
+enum XMode : int { kXLds = 0, kXGlobal = 1 };
 
 // The activations of a launch as the staging code sees them.
 struct XIn {
-    const uint8_t *y;      // Q8_1 blocks (kXLds, kXGlobal)
-    const float *xf;       // fp32 rows (kXF32, kXNormF32)
-    uint32_t stride_x;     // floats between rows of xf
-    const float *norm_w;   // kXNormF32: the norm's weights, one per column
-    float eps;
-    float *normalized;     // kXNormF32: where workgroup 0 leaves the normalised row (may be null)
-    float *red;            // kXNormF32: four floats of LDS for the reduction
+    const uint8_t *y;      // Q8_1 blocks
 };
 
 // LDS footprint of `batch` activation rows: per 64-block step 128 16-byte
@@ -178,102 +171,6 @@ struct StageLds {
     }
 };
 
-// Same LDS image as StageLds, produced from fp32 activations: every workgroup quantizes
-// the M rows itself (M * cols / 4 float4 loads spread over the workgroup), with the code the
-// stand-alone quantizer uses, so the int8 values and the fp16-rounded scales are the same bits.
-// The block sum `s` of Q8_1 is not needed by Q8_0 dots and is not formed.  x rows are
-// stride_x floats apart; cols = 32 * nb.  Ends with a workgroup barrier.
-//
-// NORM: the single row (M == 1, at most kBatch * THREADS * 4 columns, THREADS == 256) is
-// RMS-normalised first, with the stand-alone kernel's arithmetic: the sum of squares over the
-// registers already loaded, one more workgroup barrier, then (x * scale) * weight.
-template <int M, int THREADS, bool NORM = false>
-struct StageF32 {
-    static constexpr int kBatch = 6;   // float4 loads in flight per thread: one trip for a 6144-column row at 256 threads
-    static_assert(!NORM || (M == 1 && THREADS == kNormThreads), "the fused norm handles one row per 256-thread workgroup");
-    Float4 v[kBatch];
-    Float4 nw[NORM ? kBatch : 1];
-
-    __device__ __forceinline__ static Float4 fetch(const float *x, uint32_t stride_x, uint32_t per_row,
-                                                   uint32_t total, uint32_t c, bool vec) {
-        const uint32_t cc = c < total ? c : 0;
-        uint32_t m, within;
-        split_index<M>(cc, per_row, m, within);
-        const float *src = x + static_cast<uint64_t>(m) * stride_x + within * 4;
-        return vec ? load4<true>(src) : load4<false>(src);
-    }
-
-    // First trip of loads only (see StageLds::issue).
-    __device__ __forceinline__ void issue(const XIn &in, uint32_t nb) {
-        const float *x = in.xf;
-        const uint32_t stride_x = in.stride_x;
-        const uint32_t per_row = nb * 8, total = static_cast<uint32_t>(M) * per_row;
-        const bool vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride_x % 4 == 0);
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) v[u] = fetch(x, stride_x, per_row, total, u * THREADS + threadIdx.x, vec);
-        if constexpr (NORM) {   // the host only takes this path with 16-byte aligned weights
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) nw[u] = fetch(in.norm_w, 0, per_row, total, u * THREADS + threadIdx.x, true);
-        }
-    }
-
-    __device__ __forceinline__ void finish(uint8_t *smem, const XIn &in, uint32_t nb) {
-        const float *x = in.xf;
-        const uint32_t stride_x = in.stride_x;
-        if constexpr (NORM) {
-            const uint32_t chunks = nb * 8;   // <= kBatch * THREADS, checked on the host
-            float partial = 0.0f;
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                const float q = chunk_squares(v[u]);
-                partial += (u * THREADS + threadIdx.x < chunks) ? q : 0.0f;   // fetch() re-reads chunk 0 past the end
-            }
-            const float scale = rms_scale(block_tree_sum_256(partial, in.red), nb * 32, in.eps);
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                v[u] = rms_apply(v[u], scale, nw[u]);
-                const uint32_t c = u * THREADS + threadIdx.x;
-                if (in.normalized != nullptr && blockIdx.x == 0 && c < chunks)
-                    *reinterpret_cast<float4 *>(in.normalized + c * 4) = make_float4(v[u].x, v[u].y, v[u].z, v[u].w);
-            }
-        }
-        const uint32_t nsteps = (nb * 2 + 127) / 128;
-        uint32_t *wq = reinterpret_cast<uint32_t *>(smem);
-        float *wd = reinterpret_cast<float *>(smem + static_cast<size_t>(M) * nsteps * 128 * 16);
-        const uint32_t blocks_padded = nsteps * 64;
-        const uint32_t per_row = nb * 8;                        // float4 chunks per activation row
-        const uint32_t total = static_cast<uint32_t>(M) * per_row;   // multiple of 8: lanes of a block stay together
-        const bool vec = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (stride_x % 4 == 0);
-        auto quantize_put = [&](uint32_t c, const Float4 &f) {
-            float d;
-            const uint32_t packed = quantize4_q8_1(f, d);   // all lanes take part in the exchanges
-            if (c < total) {
-                uint32_t m, within;
-                split_index<M>(c, per_row, m, within);
-                const uint32_t blk = m * blocks_padded + within / 8;
-                wq[blk * 8 + within % 8] = packed;
-                if (within % 8 == 0) wd[blk] = half_bits_to_float(float_to_half_bits(d));
-            }
-        };
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) quantize_put(u * THREADS + threadIdx.x, v[u]);
-        for (uint32_t base = THREADS * kBatch; base < total; base += THREADS * kBatch) {
-            Float4 t[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) t[u] = fetch(x, stride_x, per_row, total, base + u * THREADS + threadIdx.x, vec);
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) quantize_put(base + u * THREADS + threadIdx.x, t[u]);
-        }
-        const uint32_t pad = blocks_padded - nb;
-        for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(M) * pad * 9; i += THREADS) {
-            const uint32_t b = i / 9, part = i % 9;
-            const uint32_t blk = (b / pad) * blocks_padded + nb + b % pad;
-            if (part == 0) wd[blk] = 0.0f; else wq[blk * 8 + (part - 1)] = 0u;
-        }
-        __syncthreads();
-    }
-};
-
 // Activations of the workgroup into LDS, by mode, in two halves: issue() puts the first trip of
 // activation loads in flight, finish() consumes them (and any further trips) and ends with a
 // workgroup barrier.  Loads return in order, so the weight loads a caller issues between the two
@@ -282,14 +179,11 @@ struct StageF32 {
 template <int M, int THREADS, int XMODE>
 struct XStage {
     StageLds<M, THREADS> lds;
-    StageF32<M, THREADS, XMODE == kXNormF32> f32;
     __device__ __forceinline__ void issue(const XIn &in, uint32_t nb) {
         if constexpr (XMODE == kXLds) lds.issue(in.y, nb);
-        if constexpr (XMODE == kXF32 || XMODE == kXNormF32) f32.issue(in, nb);
     }
     __device__ __forceinline__ void finish(uint8_t *smem, const XIn &in, uint32_t nb) {
         if constexpr (XMODE == kXLds) lds.finish(smem, in.y, nb);
-        if constexpr (XMODE == kXF32 || XMODE == kXNormF32) f32.finish(smem, in, nb);
     }
 };
 

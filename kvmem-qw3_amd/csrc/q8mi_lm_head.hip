@@ -74,7 +74,7 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
     auto park = [&](uint32_t kk, float total) {
         if (lane < kPerUnit) my_park[kk * kPerUnit + lane] = total;
     };
-    const XIn in{y, nullptr, 0, nullptr, 0.0f, nullptr, nullptr};
+    const XIn in{y};
     gemv_stream<M, R, THREADS, XMODE>(smem, in, nb, useq, i0, i1, rows_of, park);
     __syncthreads();
 
