@@ -2,7 +2,7 @@
 """Bench of the Q8_0 quantized-linear hot path on one MI355X.
 
 One "step" = one pass over the decode GEMV set of one 27B-style layer at M=1
-(BASELINE config 1), through the C ABI exactly as the executor would drive it:
+(config 1 of the benchmark definition), through the C ABI exactly as the executor would drive it:
 
     quantize_q8_1(x[5120])    the normed row, once for the two operators that read it
     gemv_fanout4              Q 5120x6144, K 5120x1024, V 5120x1024
@@ -232,7 +232,7 @@ def time_each_launch(hip, fn, n, warmup=5):
 
 
 def cpu_baseline(seconds=12.0):
-    """The oracle's scalar GEMV (oracle/q8_oracle.c) on BASELINE config 0
+    """The oracle's scalar GEMV (oracle/q8_oracle.c) on benchmark config 0
     (5120x5120, M=1), timed on this host: once on one core, once row-parallel."""
     sys.path.insert(0, ROOT)
     from oracle import q8_oracle as o
@@ -280,7 +280,7 @@ def cpu_gemm_sample(rows=2048, m=2048, cols=HIDDEN):
 
 
 def bench_config0(q8mi, hip, synth, copies=48, reps=480):
-    """BASELINE config 0: one 5120x5120 GEMV at M=1.  The GEMV proper reads Q8_1 activations
+    """Benchmark config 0: one 5120x5120 GEMV at M=1.  The GEMV proper reads Q8_1 activations
     (q8mi_gemv: what the bytes of this config count); also timed: the entry point that quantizes
     fp32 activations inside the GEMV, and quantizer + GEMV as two launches.
     Streaming: cycles through `copies` weight buffers (1.3 GB, no cache hits); resident: one buffer."""

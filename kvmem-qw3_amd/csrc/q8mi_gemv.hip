@@ -2,22 +2,25 @@
 // Reference semantics: src/mmvq_q8.cu:193-280 (plain), :295-399 (two weights),
 // :414-519 (SwiGLU), :528-606 (residual add), :976-1068 (four-weight fan-out).
 //
-// The weights are read exactly once from HBM and nothing else is large, so the
-// kernel is a stream over the int8 plane of each row (see q8mi_gemv_core.hpp
-// for the streaming core).  This file adds what differs between the entry
-// points: which rows form a unit, and what happens to a finished unit (store,
-// residual add, bf16 rounding, SwiGLU).  Store/add/bf16 are wave-uniform and run
-// once per unit, so they are a runtime switch; SwiGLU changes which rows a unit
-// streams and is a template parameter (its launches also show up under their own
-// kernel name in a profile).
+// The weights are read exactly once from HBM and nothing else is large, so every kernel here is a
+// stream over the int8 plane of each row.  This file holds the entry points, the routing between
+// the kernel families, and two of the families:
+//   batch 1, and batch 2 on launches with row pairs to spare: independent waves that own whole
+//       row pairs (q8mi_gemv_pairs.hip)
+//   batch 2..16: the matrix-core kernel below (core in q8mi_gemv_mfma_core.hpp), one workgroup per
+//       CU whose waves split the items of its units and combine partial sums through LDS
+//   fallbacks: the dot-product kernel below (core in q8mi_gemv_core.hpp) with the same static
+//       split, for activations that fit LDS in no other layout, and a one-lane-per-block kernel
+//       for rows whose planes are not 16-byte aligned (cols / 32 not a multiple of 8)
+// Store / add / bf16 are wave-uniform and run once per unit, so they are a runtime switch; SwiGLU
+// changes which rows a unit streams and is a template parameter (its launches also show up under
+// their own kernel name in a profile).
 #include "q8mi_gemv_core.hpp"
 #include "q8mi_gemv_mfma_core.hpp"
 #include "q8mi_gemv_params.hpp"
 
 namespace q8mi {
 namespace {
-
-
 
 // Each wave parks the (possibly partial) sums of the units it touched in LDS;
 // after a barrier the workgroup adds the partials of every unit in wave order and

@@ -22,7 +22,9 @@
 // Activations never pass through LDS at batch 1..2 when they arrive as Q8_1 blocks: a lane needs
 // the same 16 bytes and the same scale of every step for every row pair it will ever see, so it
 // loads them once into registers (rows of up to 8 KiB; 25 registers per activation row at 5120
-// columns) or, for longer rows, alongside the weights of each step (served by L2).  fp32
+// columns) or, for other row lengths, alongside the weights of each step (served by L2); rows of
+// 17 KiB are shared by the four waves of a workgroup, each of which keeps the activations of its
+// own steps in registers (gemv_pairs_ksplit_kernel).  fp32
 // activations (the entry points that quantize inside the GEMV) are quantized once per workgroup
 // into LDS by all of its waves, with the stand-alone quantizer's code, and then read into the
 // same registers.

@@ -72,7 +72,7 @@ def normal(rows, cols, seed, scale=1.0, threads=None):
 
 
 def student_t3(rows, cols, seed, scale=1.0, outlier_ppm=1000, outlier_gain=20.0, threads=None):
-    """Unit-variance Student-t(nu=3) with a seeded set of outlier columns (BASELINE config 4: 0.1 % of the
+    """Unit-variance Student-t(nu=3) with a seeded set of outlier columns (benchmark config 4: 0.1 % of the
     channels at 20 x)."""
     out = np.empty((rows, cols), np.float32)
     ok(lib().q8sup_synth_f32(out.ctypes.data_as(C.c_void_p), rows, cols, seed, 1, scale, outlier_ppm, outlier_gain,

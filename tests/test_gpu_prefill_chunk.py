@@ -1,4 +1,4 @@
-"""GPU parity at BASELINE config 3's own shapes: the prefill chunk M = 2048 on the two FFN
+"""GPU parity at the shapes of benchmark config 3: the prefill chunk M = 2048 on the two FFN
 projections, K=5120 -> N=17408 (2176 main tiles: four full rounds and a quarter round whose tiles
 are cut in two along K) and K=17408 -> N=5120 (640 tiles: one round and a K-split quarter round),
 i.e. exactly the launches bench.py times.  Reference shape: src/mmq_q8.cu:2394-2420 (128 x 128
