@@ -575,13 +575,13 @@ def main():
         for m in (1, 2, 4, 6, 8):
             st = step if m == 1 else DecodeStep(q8mi, hip, m=m)
             b = st.algorithmic_bytes(layers[0].bytes)
-            t = time_loop(hip, lambda i: st.run(layers[i % len(layers)]), max(args.steps // 2, 20), 5)
+            t = time_loop(hip, lambda i: st.run(layers[i % len(layers)]), max(args.steps // 2, 300), 50)
             sweep[f"m{m}"] = {"ms_per_step": round(t, 5), "gbps": round(b / (t * 1e-3) / 1e9, 1)}
         result["gemv_layer_gbps_by_m"] = sweep
         # the layer's two RMS norms in front of the fan-out and the SwiGLU: inside those launches, or on their own
         norms = {}
         for name, one in (("norms_inside_the_gemv_5_launches", True), ("norm_quantizer_kernels_7_launches", False)):
-            t = time_loop(hip, lambda i: step.run_with_norms(layers[i % len(layers)], one), max(args.steps // 2, 20), 5)
+            t = time_loop(hip, lambda i: step.run_with_norms(layers[i % len(layers)], one), max(args.steps // 2, 300), 50)
             norms[name] = {"ms_per_step": round(t, 5), "gbps": round(step_bytes / (t * 1e-3) / 1e9, 1)}
         result["layer_with_rms_norms_m1"] = norms
         result["launches_m1"] = bench_launches_m1(q8mi, hip, synth, step, layers)
