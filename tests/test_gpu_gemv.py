@@ -149,9 +149,11 @@ def test_gemv_stride_and_rejections(gpu, oracle):
     assert np.all(out.download(np.float32).reshape(batch, stride)[:, rows:] == 123.0)
 
 
+# (rows, cols): a streamed row length; rows whose activations stay in registers at batch 1..2; the
+# 17 KiB rows shared by the waves of a workgroup at batch 1 (odd row count: a single-row last pair)
+@pytest.mark.parametrize("rows,cols", [(200, 2048), (130, 6144), (67, 17408)])
 @pytest.mark.parametrize("batch", [1, 2, 5, 8])
-def test_gemv_fused_variants(gpu, oracle, batch):
-    rows, cols = 200, 2048
+def test_gemv_fused_variants(gpu, oracle, batch, rows, cols):
     w0 = synth.q8_0_weight(rows, cols, seed=10)
     w1 = synth.q8_0_weight(rows, cols, seed=11)
     x = synth.normal(batch, cols, seed=12 + batch)
