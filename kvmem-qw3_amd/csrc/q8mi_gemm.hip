@@ -240,9 +240,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_kernel(
 
 
 // ---- direct-to-LDS variant (rows whose int8 plane is 16-byte aligned) ----------------------
-// Workgroup tile: 32*RB weight rows x 128 activation rows; RB = 4 is the main tile, RB = 1 a
-// quarter tile with the same two stages (what problems too small to fill the chip with main tiles
-// used before the ring-staged tiles below; selectable for comparison).
+// Workgroup tile: 32*RB weight rows x 128 activation rows.  Only RB = 4, the main tile, is
+// launched (problems too small to fill the chip with main tiles go to the ring-staged tiles below).
 // Stage layout (two stages; TR = 32*RB):
 //   weight quants      TR rows x 128 B; 16-byte piece p of row r sits in slot p ^ swz(r), so equal
 //                      pieces of 8 or 16 consecutive rows fall on distinct banks
