@@ -516,18 +516,20 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_zero_split_tiles_kernel(
 // The waves split the tile by activation group first (CB groups of 32 rows) and by K second:
 // S = W / CB waves share an output patch, each taking 4 / S of the four blocks of every step; their
 // partial sums are added through LDS at the end as a balanced tree (deterministic).
-template <int CB, int W>
+template <int CB, int W, int RB = 1>
 struct RingTile {
     static constexpr int kCols = 32 * CB;
+    static constexpr int kRows = 32 * RB;                             // weight rows of the tile: RB blocks of 32
     static constexpr int kShares = W / CB;                             // waves per output patch (K split)
+    static constexpr int kWItems = 4 * RB;                             // 1 KB pieces of the weight quants (8 rows each)
     static constexpr int kYChunks = (kCols * kRec + 1023) / 1024;     // 1 KB pieces of the activation records
     static constexpr int kDyItems = CB * 2;                            // 64 lanes fill two 32-float slots
-    static constexpr int kItems = 4 + kYChunks + kDyItems + 1;         // weight pieces, records, scales, weight scales
+    static constexpr int kItems = kWItems + kYChunks + kDyItems + RB;  // weight pieces, records, scales, weight scales
     static constexpr int kLoads = (kItems + W - 1) / W;                // load instructions per wave and step
-    static constexpr int kOffYr = 32 * 128;
+    static constexpr int kOffYr = kRows * 128;
     static constexpr int kOffDy = kOffYr + kYChunks * 1024;            // fp32 activation scales, [group][block][32]
     static constexpr int kOffWsc = kOffDy + CB * 4 * 128;              // raw fp16 weight scales, [row][4]
-    static constexpr int kStage = kOffWsc + 256;
+    static constexpr int kStage = kOffWsc + 256 * RB;
     static_assert(W % CB == 0 && 4 % kShares == 0, "a patch is shared by 1, 2 or 4 waves");
 };
 
@@ -552,12 +554,13 @@ __device__ __forceinline__ void wait_ring(uint32_t steps) {
     }
 }
 
-template <int CB, int W, int NS, bool KSPLIT>
+template <int CB, int W, int NS, bool KSPLIT, int RB = 1>
 __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
         const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
         uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles) {
     constexpr bool ksplit = KSPLIT;
-    using T = RingTile<CB, W>;
+    static_assert(!KSPLIT || RB == 1, "only the narrowest tile is cut along K");
+    using T = RingTile<CB, W, RB>;
     constexpr uint32_t S = T::kShares;
     extern __shared__ __align__(16) uint8_t smem[];
     const uint32_t lane = threadIdx.x % kWave;
@@ -570,7 +573,7 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     const uint32_t xcd = id % 8u, seq = id / 8u;
     const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
     if (rt >= row_tiles) return;   // uniform for the workgroup
-    const uint32_t row0 = rt * 32u, col0 = ct * T::kCols;
+    const uint32_t row0 = rt * T::kRows, col0 = ct * T::kCols;
     const uint32_t nsb_all = nb / 4;
     const uint32_t sb0 = (ksplit && k_half) ? nsb_all / 2 : 0u;                   // first super-block of this workgroup
     const uint32_t nsb = ((ksplit && !k_half) ? nsb_all / 2 : nsb_all) - sb0;     // and how many it covers
@@ -585,18 +588,19 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     for (int i = 0; i < T::kLoads; ++i) {
         uint32_t item = wave + W * i;
         item = item < T::kItems ? item : T::kItems - 1;
-        if (item < 4) {                                   // 8 weight rows x 128 B
+        if (item < T::kWItems) {                          // 8 weight rows x 128 B
             const uint32_t r = item * 8 + lane / 8;
             lane_off[i] = clamp_row(r) * static_cast<uint32_t>(row_bytes) + ((lane & 7u) ^ swz(r)) * 16;
-        } else if (item < 4 + T::kYChunks) {              // 1 KB of activation records
-            lane_off[i] = (item - 4) * 1024 + lane * 16;
-        } else if (item < 4 + T::kYChunks + T::kDyItems) {   // the scales of two (group, block) pairs
-            const uint32_t sl = (item - 4 - T::kYChunks) * 2 + lhalf;
+        } else if (item < T::kWItems + T::kYChunks) {     // 1 KB of activation records
+            lane_off[i] = (item - T::kWItems) * 1024 + lane * 16;
+        } else if (item < T::kWItems + T::kYChunks + T::kDyItems) {   // the scales of two (group, block) pairs
+            const uint32_t sl = (item - T::kWItems - T::kYChunks) * 2 + lhalf;
             uint32_t j = col0 + (sl / 4) * 32 + l32;
             j = j < batch ? j : batch - 1;
             lane_off[i] = (j - col0) * kRec + (sl % 4) * 4;
-        } else {                                          // fp16 weight scales: 32 rows x 8 B
-            lane_off[i] = clamp_row(lane / 2) * static_cast<uint32_t>(row_bytes) + (lane & 1u) * 4;
+        } else {                                          // fp16 weight scales: 32 rows x 8 B per item
+            const uint32_t r = (item - T::kWItems - T::kYChunks - T::kDyItems) * 32 + lane / 2;
+            lane_off[i] = clamp_row(r) * static_cast<uint32_t>(row_bytes) + (lane & 1u) * 4;
         }
     }
     const uint8_t *wd_base0 = uniform_ptr(w + row0 * row_bytes);
@@ -617,15 +621,15 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
         for (int i = 0; i < T::kLoads; ++i) {
             uint32_t item = wave + W * i;
             item = item < T::kItems ? item : T::kItems - 1;
-            if (item < 4) {
+            if (item < T::kWItems) {
                 dma16(wq_base, lane_off[i], stage_off + item * 1024);
-            } else if (item < 4 + T::kYChunks) {
+            } else if (item < T::kWItems + T::kYChunks) {
                 const uint32_t off = lane_off[i] <= y_limit ? lane_off[i] : y_limit;   // never past the buffer
-                dma16(y_base, off, stage_off + T::kOffYr + (item - 4) * 1024);
-            } else if (item < 4 + T::kYChunks + T::kDyItems) {
-                dma4(y_base, lane_off[i], stage_off + T::kOffDy + (item - 4 - T::kYChunks) * 256);
+                dma16(y_base, off, stage_off + T::kOffYr + (item - T::kWItems) * 1024);
+            } else if (item < T::kWItems + T::kYChunks + T::kDyItems) {
+                dma4(y_base, lane_off[i], stage_off + T::kOffDy + (item - T::kWItems - T::kYChunks) * 256);
             } else {
-                dma4(wd_base, lane_off[i], stage_off + T::kOffWsc);
+                dma4(wd_base, lane_off[i], stage_off + T::kOffWsc + (item - T::kWItems - T::kYChunks - T::kDyItems) * 256);
             }
         }
     };
@@ -634,9 +638,11 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) seed[i] = static_cast<int>(kMagicBits);
     asm volatile("" : "+v"(seed));
-    float acc[16];
+    float acc[RB][16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rb][v] = 0.0f;
 
     const uint32_t ahead = nsb < NS - 1 ? nsb : NS - 1;
     for (uint32_t s = 0; s < ahead; ++s) issue(s);
@@ -653,18 +659,22 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
         for (uint32_t t = 0; t < 4 / S; ++t) {
             const uint32_t sub = share * (4 / S) + t;
             const v4i a = *reinterpret_cast<const v4i *>(cur + a_off + sub * 32);
-            const v4i b = *reinterpret_cast<const v4i *>(cur + l32 * 128 + (((2 * sub + lhalf) ^ fl) * 16));
-            const float dw = half_bits_to_float(*reinterpret_cast<const uint16_t *>(cur + T::kOffWsc + l32 * 8 + sub * 2));
             float dy[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const float4 q = *reinterpret_cast<const float4 *>(cur + dy_off + sub * 128 + g * 32);
                 dy[4 * g + 0] = q.x; dy[4 * g + 1] = q.y; dy[4 * g + 2] = q.z; dy[4 * g + 3] = q.w;
             }
-            const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, seed, 0, 0, 0);
-            const float cw = -kMagic * dw;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[v] = fmaf(fmaf(as_f32(r[v]), dw, cw), dy[v], acc[v]);
+            for (int rb = 0; rb < RB; ++rb) {   // the activation fragment serves every 32-row block of the tile
+                const uint32_t wr = rb * 32 + l32;
+                const v4i b = *reinterpret_cast<const v4i *>(cur + wr * 128 + (((2 * sub + lhalf) ^ fl) * 16));
+                const float dw = half_bits_to_float(*reinterpret_cast<const uint16_t *>(cur + T::kOffWsc + wr * 8 + sub * 2));
+                const v16i r = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, seed, 0, 0, 0);
+                const float cw = -kMagic * dw;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[rb][v] = fmaf(fmaf(as_f32(r[v]), dw, cw), dy[v], acc[rb][v]);
+            }
         }
         if (sb + 1 < nsb) {
             const uint32_t later = nsb - 2 - sb;   // steps issued beyond the next one
@@ -674,8 +684,8 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     }
 
     // D[i][n]: n = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (activation row of the group)
-    const uint32_t r_out = row0 + l32;
-    auto store = [&](int v, float value) {
+    auto store = [&](int rb, int v, float value) {
+        const uint32_t r_out = row0 + rb * 32 + l32;
         const uint32_t j = col0 + grp * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
         if (r_out < rows && j < batch) {
             float *out = &dst[static_cast<uint64_t>(j) * stride_dst + r_out];
@@ -685,23 +695,29 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     };
     if constexpr (S == 1) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) store(v, acc[v]);
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) store(rb, v, acc[rb][v]);
     } else {
         // every load has landed and every wave is past its last read of the stages: reuse them
         float *part = reinterpret_cast<float *>(smem);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) part[(wave * 16 + v) * kWave + lane] = acc[v];
-        __syncthreads();
-        constexpr int kMine = 16 / S;   // outputs of the patch this wave finishes
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int k = 0; k < kMine; ++k) {
-            const int v = share * kMine + k;
-            auto p = [&](uint32_t s) { return part[((s * CB + grp) * 16 + v) * kWave + lane]; };
-            float total;
-            if constexpr (S == 2) total = p(0) + p(1);
-            else total = (p(0) + p(1)) + (p(2) + p(3));
-            store(v, total);
-        }
+            for (int v = 0; v < 16; ++v) part[((wave * RB + rb) * 16 + v) * kWave + lane] = acc[rb][v];
+        __syncthreads();
+        constexpr int kMine = 16 / S;   // outputs of each patch this wave finishes
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int k = 0; k < kMine; ++k) {
+                const int v = share * kMine + k;
+                auto p = [&](uint32_t s) { return part[(((s * CB + grp) * RB + rb) * 16 + v) * kWave + lane]; };
+                float total;
+                if constexpr (S == 2) total = p(0) + p(1);
+                else total = (p(0) + p(1)) + (p(2) + p(3));
+                store(rb, v, total);
+            }
     }
 }
 
@@ -791,32 +807,32 @@ int launch_dma_rows(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
 // little: problems with at least 0.4 main tiles per resident slot (two per CU) use main tiles
 // throughout (measured crossover on MI355X: between 160 and 256 main tiles); smaller ones use the
 // ring-staged 32-row tiles.
-template <int CB, int W, int NS, bool KSPLIT>
+template <int CB, int W, int NS, bool KSPLIT, int RB = 1>
 int launch_ring_inst(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
                      uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid, hipStream_t stream) {
-    using T = RingTile<CB, W>;
+    using T = RingTile<CB, W, RB>;
     constexpr int lds = NS * T::kStage;
-    static_assert(lds >= W * 16 * kWave * 4, "the stages are reused for the partial sums of the waves");
+    static_assert(lds >= W * RB * 16 * kWave * 4, "the stages are reused for the partial sums of the waves");
     static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
     if (!granted) {
         if (lds > 64 * 1024 &&
-            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS, KSPLIT>),
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS, KSPLIT, RB>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
             (void)hipGetLastError();
             return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", lds);
         }
         granted = true;
     }
-    gemm_d4_ring_kernel<CB, W, NS, KSPLIT><<<grid, kWave * W, lds, stream>>>(
+    gemm_d4_ring_kernel<CB, W, NS, KSPLIT, RB><<<grid, kWave * W, lds, stream>>>(
         w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
     return check_launch("gemm");
 }
 
-template <int CB, int W, int NS>
+template <int CB, int W, int NS, int RB = 1>
 int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
                 uint32_t stride, hipStream_t stream) {
-    using T = RingTile<CB, W>;
-    const uint32_t row_tiles = (rows + 31u) / 32u;
+    using T = RingTile<CB, W, RB>;
+    const uint32_t row_tiles = (rows + T::kRows - 1) / T::kRows;
     const uint32_t col_tiles = (batch + T::kCols - 1) / T::kCols;
     const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
     if (grid64 > 0x3fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
@@ -827,7 +843,7 @@ int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, u
     // (up to 32 activation rows, four waves): measured on MI355X 19.2 -> 15.5 us at 5120 x 5120 and
     // 58.6 -> 44.6 us at K = 17408, batch 32; the wider tiles already split K over their waves
     // and gain nothing (64 rows) or lose (128 rows, sixteen waves: 29 -> 35 us).
-    if constexpr (CB == 1) {
+    if constexpr (CB == 1 && RB == 1) {
         if (static_cast<uint64_t>(row_tiles) * col_tiles <= static_cast<uint32_t>(device_cu_count()) &&
             nb / 4 >= 8 && batch <= 65535u) {
             gemm_zero_dst_kernel<<<dim3((rows + 1023u) / 1024u, batch), 256, 0, stream>>>(dst, rows, stride);
@@ -835,8 +851,8 @@ int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, u
                                                      static_cast<uint32_t>(grid64 * 2), stream);
         }
     }
-    return launch_ring_inst<CB, W, NS, false>(w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles,
-                                              static_cast<uint32_t>(grid64), stream);
+    return launch_ring_inst<CB, W, NS, false, RB>(w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles,
+                                                  static_cast<uint32_t>(grid64), stream);
 }
 
 int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
@@ -847,6 +863,12 @@ int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
     const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
     if (tiles * 5 >= slots * 2) return launch_dma_rows<4>(w, y, dst, rows, nb, batch, stride, stream);
     // too few main tiles to fill the chip: 32-row tiles behind a ring of stages, as wide as the batch needs
+    // Batches of 33..64 rows on matrices tall enough for more than 1.5 32-row tiles per CU take 64-row
+    // tiles: half as many workgroups re-read the activation records of a step (measured at
+    // 17408 x 5120, batch 64: 59 -> 51 us).  The 32- and 128-row-wide tiles lose with 64 rows (54
+    // against 43 us, 88 against 77 us): their rings then leave room for one workgroup per CU only.
+    if (batch > 32 && batch <= 64 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * static_cast<uint32_t>(device_cu_count()))
+        return launch_ring<2, kRingWaves2, kRing2, 2>(w, y, dst, rows, nb, batch, stride, stream);
     if (batch <= 32) return launch_ring<1, 4, kRing1>(w, y, dst, rows, nb, batch, stride, stream);
     if (batch <= 64) return launch_ring<2, kRingWaves2, kRing2>(w, y, dst, rows, nb, batch, stride, stream);
     // at most one tile per CU: sixteen waves (four K shares per group) instead of eight

@@ -141,6 +141,7 @@ GEMM_CASES = [
     (2048, 2048, 512, "128 x 128 tiles, direct-to-LDS staging"),
     (1024, 2304, 640, "128 x 128 tiles, register staging (int8 plane 8-byte aligned)"),
     (1000, 33, 1024, "ring tiles, 64 activation rows wide"),
+    (12320, 50, 512, "ring tiles, 64 weight rows x 64 activation rows (tall matrix)"),
     (1000, 100, 1024, "ring tiles, 128 activation rows wide"),
     (1000, 200, 5120, "ring tiles, 128 wide, two column tiles"),
     (4000, 29, 5120, "ring tiles, 32 wide, cut in two along K"),

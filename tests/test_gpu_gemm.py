@@ -325,12 +325,15 @@ def test_gemm_rejections(gpu):
     assert L.q8mi_gemm_medium(b.ptr, b.ptr, b.ptr, 128, 128, 65, 128, NULL) == q8mi.REJECTED
 
 
-@pytest.mark.parametrize("rows,cols", [(1000, 256), (333, 1024), (5120, 5120), (640, 17408), (160, 2304)])
+@pytest.mark.parametrize("rows,cols", [(1000, 256), (333, 1024), (5120, 5120), (640, 17408), (160, 2304),
+                                       (12320, 512), (17408, 1024)])
 @pytest.mark.parametrize("batch", [33, 48, 64, 65, 100, 128, 200])
 def test_gemm_medium_batches(gpu, oracle, rows, cols, batch):
     """Batches too small to fill the chip with 128 x 128 tiles run 32-row tiles behind a ring of
     LDS stages, 32, 64 or 128 activation rows wide, the narrow ones with K split over the waves:
-    rows and batch ragged against every tile width, K shorter and much longer than the ring."""
+    rows and batch ragged against every tile width, K shorter and much longer than the ring.  The
+    last two matrices are tall enough for the 64-row tiles that batches of 33..64 then take (one
+    of them ragged against 64 rows)."""
     w = synth.q8_0_weight(rows, cols, seed=rows * 3 + cols)
     x = synth.normal(batch, cols, seed=batch * 17 + cols)
     x[batch // 2, :128] = 0.0
