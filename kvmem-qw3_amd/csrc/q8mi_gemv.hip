@@ -360,7 +360,7 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         return check_launch("gemv_unaligned");
     }
     const uint64_t row_pairs = p.mode == kSiluMul ? p.total_rows : (p.total_rows + 1) / 2;
-    const bool mfma_first = p.xf == nullptr && gemv_prefers_mfma(row_pairs, batch) &&
+    const bool mfma_first = p.xf == nullptr && gemv_prefers_mfma(row_pairs, batch, p.nb, p.mode == kSiluMul) &&
                             reinterpret_cast<uintptr_t>(p.y) % 4 == 0 &&
                             (mfma_fits(p.nb, batch, false) || mfma_fits(p.nb, batch, true));
     if (mfma_first) {

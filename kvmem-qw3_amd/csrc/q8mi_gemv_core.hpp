@@ -442,10 +442,14 @@ constexpr int kGemvInterleave = 1;        // unit assignment, see group_units
 constexpr uint32_t kMfmaFromBatch = 2;    // smallest batch served by the matrix-core variant
 // Batch 2 goes to the matrix cores unless the launch has row pairs enough to fill the chip with
 // independent waves (measured at batch 2, row-pair against matrix-core kernel: 8192 x 5120 fan-out
-// 14.1 / 11.9 us, 5120 x 6144 11.5 / 10.2, 5120 x 17408 21.0 / 20.0, but SwiGLU 2 x 17408 x 5120
-// 31.9 / 34.1); from batch 3 on always.
-inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch) {
-    return batch >= 3 || (batch == 2 && row_pairs < 8192);
+// 14.1 / 11.9 us, 5120 x 6144 11.5 / 10.2, but SwiGLU 2 x 17408 x 5120 31.9 / 34.1) or rows of 17 KiB,
+// which the row-pair family serves with a kernel of their own (5120 x 17408: 18.8 / 20.0 us); from
+// batch 3 on always.  nb: blocks per row; silu: the SwiGLU form (whose long rows have no such kernel).
+inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch, uint32_t nb, bool silu) {
+    if (batch >= 3) return true;
+    if (batch != 2) return false;
+    if (nb == 544 && !silu) return false;
+    return row_pairs < 8192;
 }
 
 // Per kernel instantiation (one static instance each): the dynamic LDS limit is raised once, to
