@@ -448,7 +448,8 @@ constexpr uint32_t kMfmaFromBatch = 2;    // smallest batch served by the matrix
 inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch, uint32_t nb, bool silu) {
     if (batch >= 3) return true;
     if (batch != 2) return false;
-    if (nb == 544 && !silu) return false;
+    if (nb == 544 || nb == 128 || nb == 160 || nb == 192 || nb == 256) return false;   // row lengths the K-split kernel serves
+    (void)silu;
     return row_pairs < 8192;
 }
 

@@ -1,17 +1,16 @@
-// Q8_0 x Q8_1 GEMV for batch 1..2 as many small, independent waves (gfx950).
+// Q8_0 x Q8_1 GEMV for batch 1..2 as many small, independent workgroups (gfx950).
 // Reference semantics: src/mmvq_q8.cu:193-280 (plain), :295-399 (two weights), :414-519 (SwiGLU),
 // :528-606 (residual add), :976-1068 (fan-out); like the reference's kernel, a weight row is read
 // once and reused for every activation row (:221-243).
 //
-// A wave owns whole ROW PAIRS: two weight rows (SwiGLU: a gate row and its up row) from their first
-// to their last column.  Nothing is shared between waves, so there is no LDS staging of partial
-// sums, no barrier after the stream and no combine step: a wave that has its two sums writes them
-// and ends, and the hardware dispatcher hands the next row pairs to whichever CU has room.  That
-// dynamic hand-out is what balances the chip; a static split over resident workgroups loses 3..5 us
-// per launch to CUs that finish one after the other.  Measured on MI355X against the streaming
-// kernels of q8mi_gemv.hip (same bytes): 5120 x 5120 8.9 -> 6.6 us, SwiGLU 2 x 17408 x 5120
-// 33.3 -> 29.6 us, 5120 x 17408 20.4 -> 17.4 us; a plain streaming read of those sizes takes
-// 6.0, 28.8 and 15.4 us.
+// The unit of work is a ROW PAIR: two weight rows (SwiGLU: a gate row and its up row) from their
+// first to their last column.  Workgroups are small (one wave, or the few waves that share a pair),
+// own a handful of pairs, write their sums and end; the hardware dispatcher hands the next ones to
+// whichever CU has room.  That dynamic hand-out is what balances the chip: a static split of the
+// rows over resident workgroups loses 3..5 us per launch to CUs that finish one after the other.
+// Measured on MI355X against the static streaming kernels of q8mi_gemv.hip (same bytes):
+// 5120 x 5120 8.9 -> 6.6 us, SwiGLU 2 x 17408 x 5120 33.3 -> 28.7 us, 5120 x 17408 20.4 -> 16.7 us;
+// a plain streaming read of those sizes takes 6.0, 28.1 and 15.1 us.
 //
 // Lane layout.  A 1 KiB step of a row is one coalesced wave load: lane l holds 16 bytes, half of
 // block l/2.  The two rows of a pair swap half sums with one DPP move, so that even lanes end up
@@ -19,15 +18,17 @@
 // int32 sum and one fp32 rescale per 32-element block and row, and after a five-step butterfly
 // over the lanes of equal parity lane 0 holds the first row's result and lane 1 the second's.
 //
-// Activations never pass through LDS at batch 1..2 when they arrive as Q8_1 blocks: a lane needs
-// the same 16 bytes and the same scale of every step for every row pair it will ever see, so it
-// loads them once into registers (rows of up to 8 KiB; 25 registers per activation row at 5120
-// columns) or, for other row lengths, alongside the weights of each step (served by L2); rows of
-// 17 KiB are shared by the four waves of a workgroup, each of which keeps the activations of its
-// own steps in registers (gemv_pairs_ksplit_kernel).  fp32
-// activations (the entry points that quantize inside the GEMV) are quantized once per workgroup
-// into LDS by all of its waves, with the stand-alone quantizer's code, and then read into the
-// same registers.
+// Three kernels, by where the activations live:
+//   gemv_pairs_ksplit_kernel   rows of 4, 5, 6, 8 and 17 KiB (Q8_1 activations): the waves of a
+//       workgroup cut every row into interleaved 1 KiB steps, so each wave needs the activations of
+//       its own steps only, loads them once into registers (5 per step and activation row) and
+//       keeps them for all pairs of the workgroup; partial sums meet in LDS after the last pair
+//   gemv_pairs_ring_kernel     any other row length: one wave per pair, the activation bytes of a
+//       step travel with its weights through a ring of steps in flight (L2 serves them)
+//   gemv_pairs_f32_kernel (and the ring kernel's fp32 form)   fp32 activations (the entry points
+//       that quantize inside the GEMV, optionally after an RMS norm): quantized once per workgroup
+//       into LDS by all of its waves, with the stand-alone quantizer's code, then read into
+//       registers by waves that own whole pairs
 #include <type_traits>
 
 #include "q8mi_gemv_core.hpp"
@@ -117,7 +118,7 @@ __device__ __forceinline__ void write_pair(const GemvParams &p, const PairRows &
     }
 }
 
-// ---- rows of NSTEPS KiB exactly: activations in registers, a pair's weights loaded at once ----------
+// ---- a pair's weights loaded at once, activations in registers (used by the fp32-activation kernel) ---
 template <int NSTEPS>
 struct PairWeights {
     v4i q0[NSTEPS], q1[NSTEPS];
@@ -136,12 +137,15 @@ __device__ __forceinline__ void issue_pair(PairWeights<NSTEPS> &r, const PairRow
     }
 }
 
+// The sums are formed in the order of gemv_pairs_ksplit_kernel with one step per wave (what the
+// Q8_1 entry points run on these row lengths), so that the entry points which quantize fp32
+// activations inside the GEMV give the bits of quantizer + GEMV: each step's products are added
+// over the lanes first, the step totals then in ascending order onto zero.
 template <int M, int NSTEPS>
 __device__ __forceinline__ void compute_pair(const PairWeights<NSTEPS> &r, const v4i (&xq)[M][NSTEPS],
                                              const float (&dx)[M][NSTEPS], bool odd, float (&tot)[M]) {
-    float acc[M];
 #pragma unroll
-    for (int m = 0; m < M; ++m) acc[m] = 0.0f;
+    for (int m = 0; m < M; ++m) tot[m] = 0.0f;
 #pragma unroll
     for (int s = 0; s < NSTEPS; ++s) {
         const float dw = half_bits_to_float(odd ? r.d1[s] : r.d0[s]);
@@ -150,11 +154,9 @@ __device__ __forceinline__ void compute_pair(const PairWeights<NSTEPS> &r, const
             const int sa = dot16(r.q0[s], xq[m][s]);
             const int sb = dot16(r.q1[s], xq[m][s]);
             const int S = (odd ? sb : sa) + dpp_i32<kDppXor1>(odd ? sa : sb);   // full 32-element block dot
-            acc[m] = fmaf(dw * dx[m][s], static_cast<float>(S), acc[m]);
+            tot[m] += parity_sum(fmaf(dw * dx[m][s], static_cast<float>(S), 0.0f));
         }
     }
-#pragma unroll
-    for (int m = 0; m < M; ++m) tot[m] = parity_sum(acc[m]);
 }
 
 // The wave's pairs, two register sets: the next pair's loads are in flight while one is consumed.
@@ -191,37 +193,6 @@ __device__ __forceinline__ void run_pairs(const GemvParams &p, const PairSpace &
             write_pair<M, SILU>(p, done, lane, tot);
         }
     }
-}
-
-// Q8_1 activations from global memory, one wave per workgroup.
-template <int M, int NSTEPS, bool SILU>
-__global__ __launch_bounds__(kWave) void gemv_pairs_kernel(const GemvParams p, const PairSpace ps) {
-    constexpr uint32_t nb = NSTEPS * 32;
-    constexpr uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
-    const uint32_t lane = threadIdx.x;
-    const uint32_t first = blockIdx.x * ps.ppw;
-    if (first >= ps.pairs) return;
-    const uint32_t end = first + ps.ppw < ps.pairs ? first + ps.ppw : ps.pairs;
-    // activations first (they arrive first), the first pair's weights right behind them
-    v4i xq[M][NSTEPS];
-    uint16_t dxh[M][NSTEPS];
-#pragma unroll
-    for (int m = 0; m < M; ++m)
-#pragma unroll
-        for (int s = 0; s < NSTEPS; ++s) {
-            const uint8_t *blk = p.y + static_cast<uint64_t>(m * nb + 32 * s + (lane >> 1)) * kQ81Bytes;
-            xq[m][s] = load_x16(blk + 4 + (lane & 1u) * 16);
-            dxh[m][s] = *reinterpret_cast<const uint16_t *>(blk);
-        }
-    PairWeights<NSTEPS> a;
-    const PairRows ra = resolve_pair<SILU>(p, ps, first, row_bytes);
-    issue_pair<NSTEPS>(a, ra, lane);
-    float dx[M][NSTEPS];
-#pragma unroll
-    for (int m = 0; m < M; ++m)
-#pragma unroll
-        for (int s = 0; s < NSTEPS; ++s) dx[m][s] = half_bits_to_float(dxh[m][s]);
-    run_pairs<M, NSTEPS, SILU, M == 1>(p, ps, first, end, xq, dx, lane, a, ra);
 }
 
 // Sum of the squares of one fp32 row in the order of the stand-alone RMS norm (q8mi_rms_norm.hip):
@@ -487,16 +458,19 @@ __global__ __launch_bounds__(XF32 ? 512 : kWave) void gemv_pairs_ring_kernel(con
     }
 }
 
-// ---- long rows of NSTEPS KiB: the waves of a workgroup share every pair -----------------------------
-// A row of 17 KiB is too long for one wave's registers, and a wave that streams it alone re-reads the
-// activations from L2 step by step (as much L1 traffic again as the weights).  Here the WAVES waves of
-// a workgroup cut every row into interleaved 1 KiB steps: wave w takes steps w, w + WAVES, ... and a
-// 1 / WAVES share of the steps that remain (its first lanes only), so each wave needs the
-// activations of its own steps only, once, in registers, for all the pairs of the workgroup, and
-// the workgroup as a whole reads each pair as one contiguous stretch.  A slot is refilled with the
-// next pair's bytes as soon as it is consumed.  The waves' partial sums meet in LDS after the last
-// pair (one barrier per workgroup), added in wave order.
-template <int M, int NSTEPS, int WAVES>
+// ---- rows of NSTEPS KiB: the waves of a workgroup share every pair ----------------------------------
+// A wave that streams whole rows must hold the activations of the whole row (registers that then
+// are not there for loads in flight) or re-read them step by step (as much L1 traffic again as the
+// weights).  Here the WAVES waves of a workgroup cut every row into interleaved 1 KiB steps: wave
+// w takes steps w, w + WAVES, ... and a 1 / WAVES share of the steps that remain (its first lanes
+// only), so each wave needs the activations of its own steps only, once, in registers, for all
+// the pairs of the workgroup, and the workgroup as a whole reads each pair as one contiguous
+// stretch.  A slot is refilled with the next pair's bytes as soon as it is consumed.  The waves'
+// partial sums meet in LDS after the last pair (one barrier per workgroup), added in wave order.
+// Measured against one wave per pair with the whole row's activations in registers (batch 1):
+// 8192 x 5120 fan-out 9.3 -> 8.7 us, SwiGLU 2 x 17408 x 5120 29.9 -> 28.7 us, 5120 x 5120 6.9 -> 6.6 us;
+// against one wave per pair with the activations read per step: 5120 x 17408 18.0 -> 16.7 us.
+template <int M, int NSTEPS, int WAVES, bool SILU = false>
 // (waves per SIMD the registers are budgeted for: five with one activation row, three with two)
 __global__ __launch_bounds__(WAVES * kWave, M == 1 ? 5 : 3) void gemv_pairs_ksplit_kernel(const GemvParams p, const PairSpace ps) {
     constexpr uint32_t nb = NSTEPS * 32;
@@ -505,7 +479,7 @@ __global__ __launch_bounds__(WAVES * kWave, M == 1 ? 5 : 3) void gemv_pairs_kspl
     constexpr uint32_t kTail = (NSTEPS - S * WAVES) * 64 / WAVES;  // 16-byte pieces per wave of the steps left over
     static_assert((NSTEPS - S * WAVES) * 64 % WAVES == 0 && kTail % 2 == 0, "the left-over steps split evenly");
     constexpr int SL = S + (kTail ? 1 : 0);                        // register slots per wave
-    constexpr uint32_t kMaxPairs = 4;
+    constexpr uint32_t kMaxPairs = 8;
     __shared__ float part[kMaxPairs][WAVES][M][2];
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -543,7 +517,7 @@ __global__ __launch_bounds__(WAVES * kWave, M == 1 ? 5 : 3) void gemv_pairs_kspl
         d0[j] = reinterpret_cast<const uint16_t *>(rows.r0)[piece >> 1];
         d1[j] = reinterpret_cast<const uint16_t *>(rows.r1)[piece >> 1];
     };
-    PairRows rows = resolve_pair<false>(p, ps, first, row_bytes);
+    PairRows rows = resolve_pair<SILU>(p, ps, first, row_bytes);
 #pragma unroll
     for (int j = 0; j < SL; ++j) issue(j, rows);
     float dx[M][SL];
@@ -558,7 +532,7 @@ __global__ __launch_bounds__(WAVES * kWave, M == 1 ? 5 : 3) void gemv_pairs_kspl
     auto do_pair = [&](uint32_t pair, auto refill_tag) {
         constexpr bool REFILL = decltype(refill_tag)::value;
         PairRows next = rows;
-        if constexpr (REFILL) next = resolve_pair<false>(p, ps, pair + 1, row_bytes);
+        if constexpr (REFILL) next = resolve_pair<SILU>(p, ps, pair + 1, row_bytes);
         float acc[M];
 #pragma unroll
         for (int m = 0; m < M; ++m) acc[m] = 0.0f;
@@ -587,14 +561,26 @@ __global__ __launch_bounds__(WAVES * kWave, M == 1 ? 5 : 3) void gemv_pairs_kspl
     for (uint32_t pair = first; pair + 1 < end; ++pair) do_pair(pair, std::true_type{});
     do_pair(end - 1, std::false_type{});
     __syncthreads();
-    const uint32_t n = (end - first) * M * 2;
-    if (threadIdx.x < n) {
-        const uint32_t k = threadIdx.x / (2 * M), m = (threadIdx.x / 2) % M, r = threadIdx.x % 2;
-        float tot = 0.0f;
+    if constexpr (SILU) {   // the two rows of a pair are a gate row and its up row: one output
+        const uint32_t n = (end - first) * M;
+        if (threadIdx.x < n) {
+            const uint32_t k = threadIdx.x / M, m = threadIdx.x % M;
+            float g = 0.0f, u = 0.0f;
 #pragma unroll
-        for (int v = 0; v < WAVES; ++v) tot += part[k][v][m][r];
-        const PairRows out = resolve_pair<false>(p, ps, first + k, row_bytes);
-        if (r == 0 || out.two) store_out(p.mode, out.dst, static_cast<uint64_t>(m) * out.stride + out.row0 + r, tot);
+            for (int v = 0; v < WAVES; ++v) { g += part[k][v][m][0]; u += part[k][v][m][1]; }
+            const PairRows out = resolve_pair<true>(p, ps, first + k, row_bytes);
+            static_cast<float *>(out.dst)[static_cast<uint64_t>(m) * out.stride + out.row0] = (g / (1.0f + __expf(-g))) * u;
+        }
+    } else {
+        const uint32_t n = (end - first) * M * 2;
+        if (threadIdx.x < n) {
+            const uint32_t k = threadIdx.x / (2 * M), m = (threadIdx.x / 2) % M, r = threadIdx.x % 2;
+            float tot = 0.0f;
+#pragma unroll
+            for (int v = 0; v < WAVES; ++v) tot += part[k][v][m][r];
+            const PairRows out = resolve_pair<false>(p, ps, first + k, row_bytes);
+            if (r == 0 || out.two) store_out(p.mode, out.dst, static_cast<uint64_t>(m) * out.stride + out.row0 + r, tot);
+        }
     }
 }
 
@@ -617,23 +603,18 @@ PairSpace pair_space(const GemvParams &p, bool silu) {
     return ps;
 }
 
-template <int M, int NSTEPS>
-int launch_regs(const GemvParams &p, PairSpace ps, hipStream_t stream) {
-    // One activation row: two pairs per wave once there are plenty (measured: 17408 pairs 30.2 -> 29.6 us,
-    // 2560 pairs 6.6 -> 6.8 us).  Two rows: a wave loads twice the activation bytes, so two pairs always
-    // (layer of a 27B model 93 -> 86 us; four pairs 88 us).
-    ps.ppw = (M == 2 || ps.pairs >= 8192) ? 2 : 1;
-    const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
-    if (p.mode == kSiluMul) gemv_pairs_kernel<M, NSTEPS, true><<<grid, kWave, 0, stream>>>(p, ps);
-    else gemv_pairs_kernel<M, NSTEPS, false><<<grid, kWave, 0, stream>>>(p, ps);
-    return check_launch("gemv (row pairs)");
-}
-
 template <int M, int NSTEPS, int WAVES>
 int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
-    ps.ppw = 2;   // measured at 5120 x 17408: 16.9 us; one pair 17.8, three 18.1, four 17.9
+    // Pairs per workgroup, measured on MI355X.  17 KiB rows (5120 x 17408, batch 1): two 16.9 us, one 17.8,
+    // three 18.1, four 17.9.  5 KiB rows at batch 1: SwiGLU (17408 pairs) one 30.1 us, two 28.7, three 30.8,
+    // four 29.4; fan-out (4096 pairs) one 8.7, two 9.0, four 9.0.  At batch 2: SwiGLU two 30.8, four 30.2;
+    // fan-out two 9.5, four 9.3; 5120 x 6144 (2560 pairs) two 8.0, four 8.2.
+    if (NSTEPS >= 17) ps.ppw = 2;
+    else if (M == 1) ps.ppw = ps.pairs >= 8192 ? 2 : 1;
+    else ps.ppw = ps.pairs >= 4096 ? 4 : 2;
     const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
-    gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
+    if (p.mode == kSiluMul) gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES, true><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
+    else gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES, false><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
     return check_launch("gemv (row pairs, rows shared by the waves of a workgroup)");
 }
 
@@ -732,25 +713,25 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         return launch_ring_f32<2>(p, ps, stream);
     }
     if (reinterpret_cast<uintptr_t>(p.y) % 4 != 0) return Q8MI_REJECTED;
+    // rows of 4, 5, 6, 8 and 17 KiB: shared by the waves of a workgroup, activations in registers;
+    // any other length: one wave per pair, activations read with every step
     if (batch == 1) {
         switch (cols) {
-            case 4096: return launch_regs<1, 4>(p, ps, stream);
-            case 5120: return launch_regs<1, 5>(p, ps, stream);
-            case 6144: return launch_regs<1, 6>(p, ps, stream);
-            case 8192: return launch_regs<1, 8>(p, ps, stream);
-            case 17408:   // four waves per pair (two waves spill, eight: 17.1 us against 16.9)
-                if (p.mode != kSiluMul) return launch_ksplit<1, 17, 4>(p, ps, stream);
-                return launch_ring<1>(p, ps, stream);
+            case 4096: return launch_ksplit<1, 4, 4>(p, ps, stream);
+            case 5120: return launch_ksplit<1, 5, 5>(p, ps, stream);
+            case 6144: return launch_ksplit<1, 6, 6>(p, ps, stream);
+            // (8 KiB rows: 12.7 us on 8192 x 8192 against 13.1 below, but the fp32-activation form of that
+            // length runs the ring kernel, and the two forms give the same bits only on the same kernel)
+            case 17408: return launch_ksplit<1, 17, 4>(p, ps, stream);   // two waves spill, eight: 17.1 us against 16.9
             default: return launch_ring<1>(p, ps, stream);
         }
     }
     switch (cols) {
-        case 4096: return launch_regs<2, 4>(p, ps, stream);
-        case 5120: return launch_regs<2, 5>(p, ps, stream);
-        case 6144: return launch_regs<2, 6>(p, ps, stream);
-        case 17408:   // 18.8 us at 5120 x 17408 against 20.0 on the matrix cores
-            if (p.mode != kSiluMul) return launch_ksplit<2, 17, 4>(p, ps, stream);
-            return launch_ring<2>(p, ps, stream);
+        case 4096: return launch_ksplit<2, 4, 4>(p, ps, stream);
+        case 5120: return launch_ksplit<2, 5, 5>(p, ps, stream);
+        case 6144: return launch_ksplit<2, 6, 6>(p, ps, stream);
+        case 8192: return launch_ksplit<2, 8, 8>(p, ps, stream);
+        case 17408: return launch_ksplit<2, 17, 4>(p, ps, stream);   // 18.8 us at 5120 x 17408 against 20.0 on the matrix cores
         default: return launch_ring<2>(p, ps, stream);
     }
 }
