@@ -367,7 +367,7 @@ int launch_any(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         const int rc = launch_mfma_any(p, batch, stream);
         if (rc != Q8MI_REJECTED) return rc;   // a unit list whose parked sums do not fit: below
     }
-    if (batch <= 2) {   // whole row pairs per wave, handed out by the dispatcher (q8mi_gemv_pairs.hip)
+    if (batch <= kPairsMaxBatch) {   // row pairs, handed out by the dispatcher (q8mi_gemv_pairs.hip)
         const int rc = launch_pairs(p, batch, stream);
         if (rc != Q8MI_REJECTED) return rc;
     }

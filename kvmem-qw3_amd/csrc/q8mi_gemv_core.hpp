@@ -440,17 +440,24 @@ __host__ __device__ inline uint32_t max_units_touched(uint32_t group_units_max, 
 constexpr uint32_t kGemvWgsPerCu = 2;
 constexpr int kGemvInterleave = 1;        // unit assignment, see group_units
 constexpr uint32_t kMfmaFromBatch = 2;    // smallest batch served by the matrix-core variant
-// Batch 2 goes to the matrix cores unless the launch has row pairs enough to fill the chip with
-// independent waves (measured at batch 2, row-pair against matrix-core kernel: 8192 x 5120 fan-out
-// 14.1 / 11.9 us, 5120 x 6144 11.5 / 10.2, but SwiGLU 2 x 17408 x 5120 31.9 / 34.1) or rows of 17 KiB,
-// which the row-pair family serves with a kernel of their own (5120 x 17408: 18.8 / 20.0 us); from
-// batch 3 on always.  nb: blocks per row; silu: the SwiGLU form (whose long rows have no such kernel).
+constexpr uint32_t kPairsMaxBatch = 4;    // largest batch the row-pair family serves
+// Which GEMV family serves a launch of batch 2 and more (measured on MI355X, row-pair kernel with
+// the rows shared by the waves of a workgroup against matrix-core kernel, us):
+//   rows of 4, 5, 6 or 8 KiB   batch 2: always row pairs (8192 x 5120 fan-out 9.3 / 11.9, SwiGLU 30.2 / 34.1);
+//                              batch 3: row pairs (fan-out 10.0 / 11.9, 5120 x 6144 9.2 / 10.3, SwiGLU 32.0 / 33.9);
+//                              batch 4: row pairs but for the SwiGLU form (fan-out 10.8 / 11.7, 5120 x 6144
+//                              10.2 / 10.2, SwiGLU 33.7 / 33.7 at best); from batch 5 the dot products bind
+//                              (batch 6: 13.1 / 12.3 on the fan-out)
+//   rows of 17 KiB             batch 2: row pairs (5120 x 17408: 18.8 / 20.0); batch 3 and 4: 22.4 / 20.3, 30.0 / 20.6
+//   any other length           batch 2 with 8192 row pairs or more: row pairs (ring kernel); else matrix cores
+// nb: blocks per row; silu: the SwiGLU form.
 inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch, uint32_t nb, bool silu) {
-    if (batch >= 3) return true;
-    if (batch != 2) return false;
-    if (nb == 544 || nb == 128 || nb == 160 || nb == 192 || nb == 256) return false;   // row lengths the K-split kernel serves
-    (void)silu;
-    return row_pairs < 8192;
+    if (batch < 2) return false;
+    if (batch > kPairsMaxBatch) return true;
+    const bool short_rows = nb == 128 || nb == 160 || nb == 192 || nb == 256;
+    if (batch == 2) return !short_rows && nb != 544 && row_pairs < 8192;
+    if (batch == 3) return !short_rows;
+    return !short_rows || silu;
 }
 
 // Per kernel instantiation (one static instance each): the dynamic LDS limit is raised once, to

@@ -471,8 +471,8 @@ __global__ __launch_bounds__(XF32 ? 512 : kWave) void gemv_pairs_ring_kernel(con
 // 8192 x 5120 fan-out 9.3 -> 8.7 us, SwiGLU 2 x 17408 x 5120 29.9 -> 28.7 us, 5120 x 5120 6.9 -> 6.6 us;
 // against one wave per pair with the activations read per step: 5120 x 17408 18.0 -> 16.7 us.
 template <int M, int NSTEPS, int WAVES, bool SILU = false>
-// (waves per SIMD the registers are budgeted for: five with one activation row, three with two)
-__global__ __launch_bounds__(WAVES * kWave, M == 1 ? 5 : 3) void gemv_pairs_ksplit_kernel(const GemvParams p, const PairSpace ps) {
+// (waves per SIMD the registers are budgeted for: three at batch 2, which also serves the 17 KiB rows; five otherwise)
+__global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_ksplit_kernel(const GemvParams p, const PairSpace ps) {
     constexpr uint32_t nb = NSTEPS * 32;
     constexpr uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
     constexpr int S = NSTEPS / WAVES;                              // whole steps per wave
@@ -608,10 +608,12 @@ int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     // Pairs per workgroup, measured on MI355X.  17 KiB rows (5120 x 17408, batch 1): two 16.9 us, one 17.8,
     // three 18.1, four 17.9.  5 KiB rows at batch 1: SwiGLU (17408 pairs) one 30.1 us, two 28.7, three 30.8,
     // four 29.4; fan-out (4096 pairs) one 8.7, two 9.0, four 9.0.  At batch 2: SwiGLU two 30.8, four 30.2;
-    // fan-out two 9.5, four 9.3; 5120 x 6144 (2560 pairs) two 8.0, four 8.2.
+    // fan-out two 9.5, four 9.3; 5120 x 6144 (2560 pairs) two 8.0, four 8.2.  At batch 3: SwiGLU four 32.7,
+    // eight 32.0; 5120 x 6144 four 9.2, eight 10.8.
     if (NSTEPS >= 17) ps.ppw = 2;
     else if (M == 1) ps.ppw = ps.pairs >= 8192 ? 2 : 1;
-    else ps.ppw = ps.pairs >= 4096 ? 4 : 2;
+    else if (M == 2) ps.ppw = ps.pairs >= 4096 ? 4 : 2;
+    else ps.ppw = ps.pairs >= 8192 ? 8 : 4;
     const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
     if (p.mode == kSiluMul) gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES, true><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
     else gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES, false><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
@@ -688,7 +690,8 @@ int launch_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
 }  // namespace
 
 int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
-    if (batch == 0 || batch > 2 || p.nb % 8 != 0) return Q8MI_REJECTED;
+    if (batch == 0 || batch > kPairsMaxBatch || p.nb % 8 != 0) return Q8MI_REJECTED;
+    if (p.xf != nullptr && batch > 2) return Q8MI_REJECTED;   // the quantizer runs inside the kernel at batch 1 and 2 only
     if (p.norm_w != nullptr) {   // fused norm + quantizer: one row, at most kMaxNormCols columns
         constexpr uint32_t kMaxNormCols = 6144;
         if (batch != 1) return fail(Q8MI_REJECTED, "nqgemv: batch %u above 1 (normalise and quantize once, then use the GEMV)", batch);
@@ -726,13 +729,26 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
             default: return launch_ring<1>(p, ps, stream);
         }
     }
-    switch (cols) {
-        case 4096: return launch_ksplit<2, 4, 4>(p, ps, stream);
-        case 5120: return launch_ksplit<2, 5, 5>(p, ps, stream);
-        case 6144: return launch_ksplit<2, 6, 6>(p, ps, stream);
-        case 8192: return launch_ksplit<2, 8, 8>(p, ps, stream);
-        case 17408: return launch_ksplit<2, 17, 4>(p, ps, stream);   // 18.8 us at 5120 x 17408 against 20.0 on the matrix cores
-        default: return launch_ring<2>(p, ps, stream);
+    auto by_cols = [&](auto mtag) -> int {
+        constexpr int M = decltype(mtag)::value;
+        switch (cols) {
+            case 4096: return launch_ksplit<M, 4, 4>(p, ps, stream);
+            case 5120: return launch_ksplit<M, 5, 5>(p, ps, stream);
+            case 6144: return launch_ksplit<M, 6, 6>(p, ps, stream);
+            case 8192: return launch_ksplit<M, 8, 8>(p, ps, stream);
+            default: break;
+        }
+        if constexpr (M == 2) {
+            if (cols == 17408) return launch_ksplit<2, 17, 4>(p, ps, stream);   // 18.8 us at 5120 x 17408 against 20.0 on the matrix cores
+            return launch_ring<2>(p, ps, stream);
+        }
+        return Q8MI_REJECTED;   // batch 3 and 4 on other lengths: the matrix-core kernel
+    };
+    switch (batch) {
+        case 2: return by_cols(std::integral_constant<int, 2>{});
+        case 3: return by_cols(std::integral_constant<int, 3>{});
+        case 4: return by_cols(std::integral_constant<int, 4>{});
+        default: return Q8MI_REJECTED;
     }
 }
 

@@ -383,7 +383,7 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
 // 296 / 230 at 8.
 bool lm_head_uses_mfma(uint32_t rows, uint32_t nb, uint32_t batch) {
     const uint32_t mg = (batch + 3) / 4;
-    if (!gemv_prefers_mfma((static_cast<uint64_t>(rows) + 1) / 2, batch, nb, false)) return false;   // q8mi_gemv's own rule
+    if (batch < 3 && !gemv_prefers_mfma((static_cast<uint64_t>(rows) + 1) / 2, batch, nb, false)) return false;   // 2 rows: q8mi_gemv's own rule
     return mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u <= kLdsLimit - 256;
 }
 

@@ -48,7 +48,7 @@ GEMV_SHAPES = [(1000, 5120), (515, 6144), (160, 17408), (37, 2048)]
 @pytest.mark.parametrize("rows,cols", GEMV_SHAPES)
 @pytest.mark.parametrize("batch", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_gemv_bits(gpu, oracle, rows, cols, batch):
-    """q8mi_gemv: dot-product kernel at batch 1..2, matrix-core kernel from 3 on."""
+    """q8mi_gemv: every batch, so both the dot-product kernels and the matrix-core kernel."""
     w = ex.weight(rows, cols, seed=rows + cols)
     x = ex.activations(batch, cols, seed=batch * 7 + cols)
     dw = dev(w)
@@ -60,7 +60,7 @@ def test_gemv_bits(gpu, oracle, rows, cols, batch):
     same_bits(out.download(np.float32).reshape(batch, rows), ref, f"gemv {rows}x{cols} M={batch}")
 
 
-@pytest.mark.parametrize("batch", [1, 2, 4, 8])
+@pytest.mark.parametrize("batch", [1, 2, 3, 4, 8])
 def test_gemv_fused_forms_bits(gpu, oracle, batch):
     """Residual add (fp32 and bf16), bf16 store, two weights and the four-way fan-out."""
     rows, cols = 300, 5120

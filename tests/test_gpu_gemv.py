@@ -29,8 +29,9 @@ def block_dot_check(oracle, dw, w, dy, y, rows, cols, batch, seed, n=4096):
     assert np.array_equal(got, ref)
 
 
-# (rows, cols): aligned planes (cols % 256 == 0), ragged step counts, tiny rows
-SHAPES = [(5120, 5120), (64, 256), (7, 512), (300, 2304), (129, 6144), (33, 17408)]
+# (rows, cols): aligned planes (cols % 256 == 0), ragged step counts, tiny rows; rows of 4, 5, 6, 8
+# and 17 KiB have kernels of their own at batch 1..4 (odd row counts end in a single-row pair)
+SHAPES = [(5120, 5120), (64, 256), (7, 512), (300, 2304), (129, 6144), (33, 17408), (131, 4096), (75, 8192)]
 
 
 @pytest.mark.parametrize("rows,cols", SHAPES)
@@ -152,7 +153,7 @@ def test_gemv_stride_and_rejections(gpu, oracle):
 # (rows, cols): a streamed row length; rows whose activations stay in registers at batch 1..2; the
 # 17 KiB rows shared by the waves of a workgroup at batch 1 (odd row count: a single-row last pair)
 @pytest.mark.parametrize("rows,cols", [(200, 2048), (130, 6144), (67, 17408)])
-@pytest.mark.parametrize("batch", [1, 2, 5, 8])
+@pytest.mark.parametrize("batch", [1, 2, 3, 4, 5, 8])
 def test_gemv_fused_variants(gpu, oracle, batch, rows, cols):
     w0 = synth.q8_0_weight(rows, cols, seed=10)
     w1 = synth.q8_0_weight(rows, cols, seed=11)
@@ -222,7 +223,7 @@ def test_gemv_fused_variants(gpu, oracle, batch, rows, cols):
 # columns: a streamed row length, one whose activations stay in registers at batch 1..2, and the
 # 17 KiB rows that the waves of a workgroup share at batch 1 (odd row counts end in a single-row pair)
 @pytest.mark.parametrize("cols", [1024, 5120, 17408])
-@pytest.mark.parametrize("batch", [1, 2, 3, 8])
+@pytest.mark.parametrize("batch", [1, 2, 3, 4, 8])
 def test_gemv_fanout4(gpu, oracle, batch, cols):
     rows = [96, 0, 17, 130]           # slot 1 is empty, as when the executor passes 3 weights
     ws = [synth.q8_0_weight(r, cols, seed=50 + i) if r else None for i, r in enumerate(rows)]
