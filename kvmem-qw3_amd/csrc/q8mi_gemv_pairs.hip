@@ -18,17 +18,18 @@
 // int32 sum and one fp32 rescale per 32-element block and row, and after a five-step butterfly
 // over the lanes of equal parity lane 0 holds the first row's result and lane 1 the second's.
 //
-// Three kernels, by where the activations live:
-//   gemv_pairs_ksplit_kernel   rows of 4, 5, 6, 8 and 17 KiB (Q8_1 activations): the waves of a
-//       workgroup cut every row into interleaved 1 KiB steps, so each wave needs the activations of
-//       its own steps only, loads them once into registers (5 per step and activation row) and
-//       keeps them for all pairs of the workgroup; partial sums meet in LDS after the last pair
+// Two kernels, by where the activations live:
+//   gemv_pairs_ksplit_kernel   rows of 4, 5, 6, 8 and 17 KiB: the waves of a workgroup cut every row
+//       into interleaved 1 KiB steps, so each wave needs the activations of its own steps only,
+//       loads them once into registers (5 per step and activation row) and keeps them for all
+//       pairs of the workgroup; partial sums meet in LDS after the last pair.  With fp32
+//       activations (the entry points that quantize inside the GEMV, optionally after an RMS norm;
+//       one row of 4..8 KiB) every wave quantizes the 1024 floats of its own step in registers,
+//       with the stand-alone quantizer's arithmetic; only the norm's sum of squares crosses the
+//       waves, through LDS, in the stand-alone norm's order
 //   gemv_pairs_ring_kernel     any other row length: one wave per pair, the activation bytes of a
-//       step travel with its weights through a ring of steps in flight (L2 serves them)
-//   gemv_pairs_f32_kernel (and the ring kernel's fp32 form)   fp32 activations (the entry points
-//       that quantize inside the GEMV, optionally after an RMS norm): quantized once per workgroup
-//       into LDS by all of its waves, with the stand-alone quantizer's code, then read into
-//       registers by waves that own whole pairs
+//       step travel with its weights through a ring of steps in flight (L2 serves them); fp32
+//       activations are quantized once per workgroup into LDS by all of its waves
 #include <type_traits>
 
 #include "q8mi_gemv_core.hpp"
@@ -118,83 +119,6 @@ __device__ __forceinline__ void write_pair(const GemvParams &p, const PairRows &
     }
 }
 
-// ---- a pair's weights loaded at once, activations in registers (used by the fp32-activation kernel) ---
-template <int NSTEPS>
-struct PairWeights {
-    v4i q0[NSTEPS], q1[NSTEPS];
-    uint16_t d0[NSTEPS], d1[NSTEPS];
-};
-
-template <int NSTEPS>
-__device__ __forceinline__ void issue_pair(PairWeights<NSTEPS> &r, const PairRows &rows, uint32_t lane) {
-    constexpr uint32_t nb = NSTEPS * 32;
-#pragma unroll
-    for (int s = 0; s < NSTEPS; ++s) {
-        r.q0[s] = load_q16(rows.r0 + 2 * nb + s * 1024 + lane * 16);
-        r.q1[s] = load_q16(rows.r1 + 2 * nb + s * 1024 + lane * 16);
-        r.d0[s] = reinterpret_cast<const uint16_t *>(rows.r0)[32 * s + (lane >> 1)];
-        r.d1[s] = reinterpret_cast<const uint16_t *>(rows.r1)[32 * s + (lane >> 1)];
-    }
-}
-
-// The sums are formed in the order of gemv_pairs_ksplit_kernel with one step per wave (what the
-// Q8_1 entry points run on these row lengths), so that the entry points which quantize fp32
-// activations inside the GEMV give the bits of quantizer + GEMV: each step's products are added
-// over the lanes first, the step totals then in ascending order onto zero.
-template <int M, int NSTEPS>
-__device__ __forceinline__ void compute_pair(const PairWeights<NSTEPS> &r, const v4i (&xq)[M][NSTEPS],
-                                             const float (&dx)[M][NSTEPS], bool odd, float (&tot)[M]) {
-#pragma unroll
-    for (int m = 0; m < M; ++m) tot[m] = 0.0f;
-#pragma unroll
-    for (int s = 0; s < NSTEPS; ++s) {
-        const float dw = half_bits_to_float(odd ? r.d1[s] : r.d0[s]);
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-            const int sa = dot16(r.q0[s], xq[m][s]);
-            const int sb = dot16(r.q1[s], xq[m][s]);
-            const int S = (odd ? sb : sa) + dpp_i32<kDppXor1>(odd ? sa : sb);   // full 32-element block dot
-            tot[m] += parity_sum(fmaf(dw * dx[m][s], static_cast<float>(S), 0.0f));
-        }
-    }
-}
-
-// The wave's pairs, two register sets: the next pair's loads are in flight while one is consumed.
-template <int M, int NSTEPS, bool SILU, bool DOUBLE>
-__device__ __forceinline__ void run_pairs(const GemvParams &p, const PairSpace &ps, uint32_t first, uint32_t end,
-                                          const v4i (&xq)[M][NSTEPS], const float (&dx)[M][NSTEPS], uint32_t lane,
-                                          PairWeights<NSTEPS> &a, PairRows ra) {
-    constexpr uint64_t row_bytes = static_cast<uint64_t>(NSTEPS) * 32 * 34;
-    const bool odd = lane & 1u;
-    float tot[M];
-    if constexpr (DOUBLE) {
-        PairWeights<NSTEPS> b;
-        PairRows rb = ra;
-        uint32_t pair = first;
-        while (true) {
-            const bool more1 = pair + 1 < end;
-            if (more1) { rb = resolve_pair<SILU>(p, ps, pair + 1, row_bytes); issue_pair<NSTEPS>(b, rb, lane); }
-            compute_pair<M, NSTEPS>(a, xq, dx, odd, tot);
-            write_pair<M, SILU>(p, ra, lane, tot);
-            if (!more1) break;
-            ++pair;
-            const bool more2 = pair + 1 < end;
-            if (more2) { ra = resolve_pair<SILU>(p, ps, pair + 1, row_bytes); issue_pair<NSTEPS>(a, ra, lane); }
-            compute_pair<M, NSTEPS>(b, xq, dx, odd, tot);
-            write_pair<M, SILU>(p, rb, lane, tot);
-            if (!more2) break;
-            ++pair;
-        }
-    } else {
-        for (uint32_t pair = first; pair < end; ++pair) {
-            compute_pair<M, NSTEPS>(a, xq, dx, odd, tot);
-            const PairRows done = ra;
-            if (pair + 1 < end) { ra = resolve_pair<SILU>(p, ps, pair + 1, row_bytes); issue_pair<NSTEPS>(a, ra, lane); }
-            write_pair<M, SILU>(p, done, lane, tot);
-        }
-    }
-}
-
 // Sum of the squares of one fp32 row in the order of the stand-alone RMS norm (q8mi_rms_norm.hip):
 // thread t of the first 256 adds chunks t, t + 256, ... in that order, the 256 partials meet in a
 // balanced tree (64 lanes by DPP, then the four wave sums).  Every thread of the workgroup must
@@ -208,98 +132,6 @@ __device__ __forceinline__ float first256_tree_sum(float partial, float *red) {
     }
     __syncthreads();
     return (red[0] + red[1]) + (red[2] + red[3]);
-}
-
-// fp32 activations: the workgroup's waves quantize the row into LDS together (the stand-alone
-// quantizer's code, so the same bits), one barrier, then every wave goes its own way.  One
-// activation row; up to sixteen waves, so at most 128 registers per lane.
-// NORM: the row is RMS-normalised first, with the arithmetic of the stand-alone norm kernel
-// (same bits); workgroup 0 also writes the normalised row.  At most eight waves then.
-template <int NSTEPS, bool SILU, bool NORM>
-__global__ __launch_bounds__(NORM ? 512 : 1024) void gemv_pairs_f32_kernel(const GemvParams p, const PairSpace ps) {
-    constexpr uint32_t nb = NSTEPS * 32;
-    constexpr uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
-    constexpr uint32_t kChunks = nb * 8;   // float4 chunks of the row
-    __shared__ __align__(16) uint32_t lds_q[kChunks];
-    __shared__ float lds_d[nb];
-    __shared__ float red[4];
-    const uint32_t lane = threadIdx.x % kWave;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const uint32_t waves = blockDim.x / kWave;
-    const uint32_t first = (blockIdx.x * waves + wave) * ps.ppw;
-    const bool live = first < ps.pairs;
-    const uint32_t end = first + ps.ppw < ps.pairs ? first + ps.ppw : ps.pairs;
-    const bool vec = NORM || (reinterpret_cast<uintptr_t>(p.xf) % 16 == 0);   // the norm's entry points demand alignment
-    // activation loads first, the first pair's weights behind them, then the conversion
-    constexpr uint32_t kMaxTrips = (kChunks + 255) / 256;   // at least four waves
-    Float4 sq[NORM ? kMaxTrips : 1];    // NORM: the chunks whose squares this thread adds
-    Float4 nw[NORM ? kMaxTrips : 1];    // NORM: the norm's weights of the chunks this thread quantizes
-    if constexpr (NORM) {
-        if (threadIdx.x < kNormThreads) {
-#pragma unroll
-            for (uint32_t k = 0; k < kMaxTrips; ++k) {
-                const uint32_t c = k * kNormThreads + threadIdx.x;
-                sq[k] = load4<true>(p.xf + (c < kChunks ? c : 0u) * 4);
-            }
-        }
-    }
-    Float4 xv[kMaxTrips];
-#pragma unroll
-    for (uint32_t t = 0; t < kMaxTrips; ++t) {
-        if (t * blockDim.x >= kChunks) break;   // workgroup-uniform: larger workgroups need fewer trips
-        const uint32_t c = t * blockDim.x + threadIdx.x;
-        const uint32_t cc = c < kChunks ? c : 0u;
-        xv[t] = vec ? load4<true>(p.xf + cc * 4) : load4<false>(p.xf + cc * 4);
-        if constexpr (NORM) nw[t] = load4<true>(p.norm_w + cc * 4);
-    }
-    asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
-    PairWeights<NSTEPS> a;
-    PairRows ra{};
-    if (live) {
-        ra = resolve_pair<SILU>(p, ps, first, row_bytes);
-        issue_pair<NSTEPS>(a, ra, lane);
-    }
-    asm volatile("" ::: "memory");   // ... and the weight loads ahead of the barriers
-    if constexpr (NORM) {
-        float partial = 0.0f;
-        if (threadIdx.x < kNormThreads) {
-#pragma unroll
-            for (uint32_t k = 0; k < kMaxTrips; ++k) {
-                const float q = chunk_squares(sq[k]);
-                partial += (k * kNormThreads + threadIdx.x < kChunks) ? q : 0.0f;
-            }
-        }
-        const float scale = rms_scale(first256_tree_sum(partial, red), nb * 32, p.eps);
-#pragma unroll
-        for (uint32_t t = 0; t < kMaxTrips; ++t) {
-            if (t * blockDim.x >= kChunks) break;
-            xv[t] = rms_apply(xv[t], scale, nw[t]);
-            const uint32_t c = t * blockDim.x + threadIdx.x;
-            if (p.normalized != nullptr && blockIdx.x == 0 && c < kChunks)
-                *reinterpret_cast<float4 *>(p.normalized + c * 4) = make_float4(xv[t].x, xv[t].y, xv[t].z, xv[t].w);
-        }
-    }
-#pragma unroll
-    for (uint32_t t = 0; t < kMaxTrips; ++t) {
-        if (t * blockDim.x >= kChunks) break;
-        const uint32_t c = t * blockDim.x + threadIdx.x;
-        float d;
-        const uint32_t packed = quantize4_q8_1(xv[t], d);   // all lanes take part in the exchanges
-        if (c < kChunks) {
-            lds_q[c] = packed;
-            if (c % 8 == 0) lds_d[c / 8] = half_bits_to_float(float_to_half_bits(d));
-        }
-    }
-    __syncthreads();
-    if (!live) return;
-    v4i xq[1][NSTEPS];
-    float dx[1][NSTEPS];
-#pragma unroll
-    for (int s = 0; s < NSTEPS; ++s) {
-        xq[0][s] = *reinterpret_cast<const v4i *>(&lds_q[s * 256 + lane * 4]);
-        dx[0][s] = lds_d[32 * s + (lane >> 1)];
-    }
-    run_pairs<1, NSTEPS, SILU, false>(p, ps, first, end, xq, dx, lane, a, ra);
 }
 
 // ---- rows of any length: a rolling pipeline over (pair, step) items -------------------------------
@@ -323,7 +155,8 @@ inline uint32_t ring_x_lds_bytes(uint32_t nb, uint32_t m) { return m * nb * (32 
 // XF32: fp32 activations, quantized into LDS by the whole workgroup before the first item is
 // consumed (the first loads of every wave are already in flight by then); otherwise one wave per
 // workgroup and Q8_1 blocks from global memory.
-// NORM (XF32, one row): the row is RMS-normalised before it is quantized, see gemv_pairs_f32_kernel.
+// NORM (XF32, one row): the row is RMS-normalised before it is quantized, with the arithmetic of the
+// stand-alone norm kernel (same bits); workgroup 0 also writes the normalised row.
 template <int M, bool SILU, bool XF32, bool NORM = false>
 __global__ __launch_bounds__(XF32 ? 512 : kWave) void gemv_pairs_ring_kernel(const GemvParams p, const PairSpace ps) {
     static_assert(!NORM || (XF32 && M == 1), "the fused norm handles one fp32 row");
@@ -470,7 +303,13 @@ __global__ __launch_bounds__(XF32 ? 512 : kWave) void gemv_pairs_ring_kernel(con
 // Measured against one wave per pair with the whole row's activations in registers (batch 1):
 // 8192 x 5120 fan-out 9.3 -> 8.7 us, SwiGLU 2 x 17408 x 5120 29.9 -> 28.7 us, 5120 x 5120 6.9 -> 6.6 us;
 // against one wave per pair with the activations read per step: 5120 x 17408 18.0 -> 16.7 us.
-template <int M, int NSTEPS, int WAVES, bool SILU = false>
+// XF32 (one fp32 activation row, one step per wave): a wave quantizes the 1024 floats of its step
+// itself -- a lane and its neighbour hold one 32-element block -- behind its first weight requests;
+// against workgroups of 8..16 waves that quantized the row into LDS and then owned whole pairs:
+// SwiGLU with the norm inside 36.3 -> 31.5 us, fan-out 11.4 -> 11.1, 5120 x 6144 9.3 -> 8.4.
+constexpr uint32_t kKsplitMaxPairs = 12;   // pairs a workgroup may take (its partial sums wait in LDS)
+
+template <int M, int NSTEPS, int WAVES, bool SILU = false, bool XF32 = false, bool NORM = false>
 // (waves per SIMD the registers are budgeted for: three at batch 2, which also serves the 17 KiB rows; five otherwise)
 __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_ksplit_kernel(const GemvParams p, const PairSpace ps) {
     constexpr uint32_t nb = NSTEPS * 32;
@@ -479,8 +318,11 @@ __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_kspl
     constexpr uint32_t kTail = (NSTEPS - S * WAVES) * 64 / WAVES;  // 16-byte pieces per wave of the steps left over
     static_assert((NSTEPS - S * WAVES) * 64 % WAVES == 0 && kTail % 2 == 0, "the left-over steps split evenly");
     constexpr int SL = S + (kTail ? 1 : 0);                        // register slots per wave
-    constexpr uint32_t kMaxPairs = 8;
-    __shared__ float part[kMaxPairs][WAVES][M][2];
+    static_assert(!XF32 || (M == 1 && SL == 1 && kTail == 0 && WAVES >= 4), "fp32 activations: one row, one step per wave, the norm's tree needs four waves");
+    static_assert(!NORM || XF32, "the norm applies to fp32 activations");
+    __shared__ float part[kKsplitMaxPairs][WAVES][M][2];
+    __shared__ float squares[NORM ? WAVES : 1][NORM ? kNormThreads : 1];
+    __shared__ float red[4];
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t w = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const bool odd = lane & 1u;
@@ -495,19 +337,31 @@ __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_kspl
 
     v4i xq[M][SL];
     uint16_t dxh[M][SL];
+    Float4 xv[XF32 ? 4 : 1], nw[NORM ? 4 : 1];   // XF32: the lane's 16 floats (half a block) of the wave's step
+    if constexpr (XF32) {
+        const uint32_t at = piece_of(0) * 16;
+        const bool vec = NORM || (reinterpret_cast<uintptr_t>(p.xf) % 16 == 0);   // the norm's entry points demand alignment
 #pragma unroll
-    for (int m = 0; m < M; ++m)
-#pragma unroll
-        for (int j = 0; j < SL; ++j) {
-            xq[m][j] = v4i{0, 0, 0, 0};
-            dxh[m][j] = 0;
-            if (live_in(j)) {
-                const uint32_t piece = piece_of(j);
-                const uint8_t *blk = p.y + static_cast<uint64_t>(m * nb + (piece >> 1)) * kQ81Bytes;
-                xq[m][j] = load_x16(blk + 4 + (piece & 1u) * 16);
-                dxh[m][j] = *reinterpret_cast<const uint16_t *>(blk);
-            }
+        for (int i = 0; i < 4; ++i) {
+            xv[i] = vec ? load4<true>(p.xf + at + 4 * i) : load4<false>(p.xf + at + 4 * i);
+            if constexpr (NORM) nw[i] = load4<true>(p.norm_w + at + 4 * i);
         }
+        asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
+    } else {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int j = 0; j < SL; ++j) {
+                xq[m][j] = v4i{0, 0, 0, 0};
+                dxh[m][j] = 0;
+                if (live_in(j)) {
+                    const uint32_t piece = piece_of(j);
+                    const uint8_t *blk = p.y + static_cast<uint64_t>(m * nb + (piece >> 1)) * kQ81Bytes;
+                    xq[m][j] = load_x16(blk + 4 + (piece & 1u) * 16);
+                    dxh[m][j] = *reinterpret_cast<const uint16_t *>(blk);
+                }
+            }
+    }
     v4i q0[SL], q1[SL];
     uint16_t d0[SL], d1[SL];
     auto issue = [&](int j, const PairRows &rows) {
@@ -521,10 +375,48 @@ __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_kspl
 #pragma unroll
     for (int j = 0; j < SL; ++j) issue(j, rows);
     float dx[M][SL];
+    if constexpr (XF32) {
+        asm volatile("" ::: "memory");   // ... and the weight loads ahead of the barriers
+        if constexpr (NORM) {
+            // Sum of squares in the stand-alone norm's order: there thread t adds chunks t, t + 256, ...;
+            // here wave u holds chunks 256 u + (0..255), so thread t adds squares[0..WAVES-1][t] ascending.
 #pragma unroll
-    for (int m = 0; m < M; ++m)
+            for (int i = 0; i < 4; ++i) squares[w][lane * 4 + i] = chunk_squares(xv[i]);
+            __syncthreads();
+            float partial = 0.0f;
+            if (threadIdx.x < kNormThreads) {
 #pragma unroll
-        for (int j = 0; j < SL; ++j) dx[m][j] = half_bits_to_float(dxh[m][j]);
+                for (int u = 0; u < WAVES; ++u) partial += squares[u][threadIdx.x];
+            }
+            const float scale = rms_scale(first256_tree_sum(partial, red), nb * 32, p.eps);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                xv[i] = rms_apply(xv[i], scale, nw[i]);
+                if (p.normalized != nullptr && blockIdx.x == 0)
+                    *reinterpret_cast<float4 *>(p.normalized + piece_of(0) * 16 + 4 * i) = make_float4(xv[i].x, xv[i].y, xv[i].z, xv[i].w);
+            }
+        }
+        // Q8_1 of the block this lane shares with its neighbour: the stand-alone quantizer's arithmetic
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(xv[i].x), fabsf(xv[i].y)), fmaxf(fabsf(xv[i].z), fabsf(xv[i].w))));
+        amax = fmaxf(amax, dpp_f32<kDppXor1>(amax));
+        const float d = amax / 127.0f;
+        int q[16];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rint_div4(xv[i], d, q[4 * i], q[4 * i + 1], q[4 * i + 2], q[4 * i + 3]);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) q[i] = amax == 0.0f ? 0 : q[i];
+        xq[0][0] = v4i{static_cast<int>(pack4(q[0], q[1], q[2], q[3])), static_cast<int>(pack4(q[4], q[5], q[6], q[7])),
+                       static_cast<int>(pack4(q[8], q[9], q[10], q[11])), static_cast<int>(pack4(q[12], q[13], q[14], q[15]))};
+        dx[0][0] = half_bits_to_float(float_to_half_bits(d));
+    } else {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int j = 0; j < SL; ++j) dx[m][j] = half_bits_to_float(dxh[m][j]);
+    }
 
     // one pair: REFILL = its slots are refilled with the next pair's bytes as they are consumed (every
     // pair but the last; a separate copy of the loop body, so that no branch sits between the loads
@@ -620,6 +512,45 @@ int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     return check_launch("gemv (row pairs, rows shared by the waves of a workgroup)");
 }
 
+// fp32 activations on rows of NSTEPS KiB: every workgroup quantizes (and normalises) the row itself,
+// each wave its own step, so a workgroup takes more pairs than with Q8_1 activations.
+template <int NSTEPS>
+int launch_ksplit_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
+    // Pairs per workgroup.  Staging costs a workgroup about as much as four pairs, so few, long
+    // workgroups: while all of them are resident at once (five waves per SIMD), a whole number per
+    // CU with at most four pairs each, or at most eight if four are too few; beyond, the fewest rounds of resident workgroups with an
+    // even share each, so that no short last round leaves most of the chip idle.  Measured at 5120
+    // columns with the norm inside (pairs: us by pairs per workgroup): 1024: 1 8.0, 2 6.5, 4 6.5,
+    // 8 8.4; 2048: 2 9.1, 4 8.0, 8 8.8; 4096: 4 11.1, 8 11.0; 6144: 4 15.8, 6 14.3, 8 13.7; 8192:
+    // 4 19.7, 8 17.0; 8704: 4 20.5, 8 20.6, 9 18.2.
+    const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+    const uint32_t resident = 20 / NSTEPS;   // workgroups per CU
+    if (ps.pairs <= cus * resident * 8) {
+        const uint32_t target = ps.pairs <= cus * resident * 4 ? 4 : 8;
+        const uint32_t per_cu = (ps.pairs + cus * target - 1) / (cus * target);
+        ps.ppw = (ps.pairs + cus * per_cu - 1) / (cus * per_cu);
+        if (ps.ppw < 2) ps.ppw = 2;
+    } else {
+        const uint32_t slots = cus * resident;
+        const uint32_t rounds = (ps.pairs + slots * kKsplitMaxPairs - 1) / (slots * kKsplitMaxPairs);
+        ps.ppw = (ps.pairs + slots * rounds - 1) / (slots * rounds);
+    }
+    const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
+    const bool silu = p.mode == kSiluMul;
+    if (p.norm_w != nullptr) {
+        if constexpr (NSTEPS <= 6) {
+            if (silu) gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, true, true, true><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
+            else gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, false, true, true><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
+            return check_launch("gemv (row pairs, fp32 activations, fused norm)");
+        } else {
+            return Q8MI_REJECTED;
+        }
+    }
+    if (silu) gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, true, true, false><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
+    else gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, false, true, false><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
+    return check_launch("gemv (row pairs, fp32 activations)");
+}
+
 template <int M>
 int launch_ring(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     ps.ppw = 2;   // measured at 17408 columns: 17.4 us against 18.0..18.8 with one pair per wave
@@ -672,21 +603,6 @@ int launch_ring_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     return launch(gemv_pairs_ring_kernel<M, false, true>);
 }
 
-template <int NSTEPS>
-int launch_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
-    uint32_t waves, grid;
-    if (p.norm_w != nullptr) {
-        f32_geometry(ps, 8, waves, grid);
-        if (p.mode == kSiluMul) gemv_pairs_f32_kernel<NSTEPS, true, true><<<grid, waves * kWave, 0, stream>>>(p, ps);
-        else gemv_pairs_f32_kernel<NSTEPS, false, true><<<grid, waves * kWave, 0, stream>>>(p, ps);
-        return check_launch("gemv (row pairs, fp32 activations, fused norm)");
-    }
-    f32_geometry(ps, 16, waves, grid);
-    if (p.mode == kSiluMul) gemv_pairs_f32_kernel<NSTEPS, true, false><<<grid, waves * kWave, 0, stream>>>(p, ps);
-    else gemv_pairs_f32_kernel<NSTEPS, false, false><<<grid, waves * kWave, 0, stream>>>(p, ps);
-    return check_launch("gemv (row pairs, fp32 activations)");
-}
-
 }  // namespace
 
 int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
@@ -707,9 +623,10 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
     if (p.xf != nullptr) {
         if (batch == 1) {
             switch (cols) {
-                case 4096: return launch_f32<4>(p, ps, stream);
-                case 5120: return launch_f32<5>(p, ps, stream);
-                case 6144: return launch_f32<6>(p, ps, stream);
+                case 4096: return launch_ksplit_f32<4>(p, ps, stream);
+                case 5120: return launch_ksplit_f32<5>(p, ps, stream);
+                case 6144: return launch_ksplit_f32<6>(p, ps, stream);
+                case 8192: return launch_ksplit_f32<8>(p, ps, stream);
                 default: return launch_ring_f32<1>(p, ps, stream);
             }
         }
@@ -723,8 +640,7 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
             case 4096: return launch_ksplit<1, 4, 4>(p, ps, stream);
             case 5120: return launch_ksplit<1, 5, 5>(p, ps, stream);
             case 6144: return launch_ksplit<1, 6, 6>(p, ps, stream);
-            // (8 KiB rows: 12.7 us on 8192 x 8192 against 13.1 below, but the fp32-activation form of that
-            // length runs the ring kernel, and the two forms give the same bits only on the same kernel)
+            case 8192: return launch_ksplit<1, 8, 8>(p, ps, stream);
             case 17408: return launch_ksplit<1, 17, 4>(p, ps, stream);   // two waves spill, eight: 17.1 us against 16.9
             default: return launch_ring<1>(p, ps, stream);
         }

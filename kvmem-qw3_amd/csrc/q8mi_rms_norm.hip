@@ -69,23 +69,26 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const NormParams
     const uint32_t chunks = (n + 3) / 4;
     const Float4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
 
-    Float4 held[kHeld];
+    // the norm weights of the held chunks are requested together with x: one memory round trip, not two
+    Float4 held[kHeld], wheld[kHeld];
     float partial = 0.0f;
 #pragma unroll
     for (uint32_t u = 0; u < kHeld; ++u) {
         const uint32_t c = u * kNormThreads + t;
         held[u] = c < chunks ? load_chunk<VEC>(x, c, n) : zero;
-        partial += chunk_squares(held[u]);   // + 0 for chunks past the end
+        wheld[u] = c < chunks ? load_chunk<VEC>(p.weight, c, n) : zero;
     }
+#pragma unroll
+    for (uint32_t u = 0; u < kHeld; ++u) partial += chunk_squares(held[u]);   // + 0 for chunks past the end
     for (uint32_t c = kHeld * kNormThreads + t; c < chunks; c += kNormThreads)
         partial += chunk_squares(load_chunk<VEC>(x, c, n));
     const float scale = rms_scale(block_tree_sum_256(partial, red), n, p.eps);
 
     // All lanes walk the same trips: the quantizer's lane exchanges need wave-uniform control flow
     // (cols % 32 == 0 there, so the eight lanes of a block are in or out together).
-    auto emit = [&](uint32_t c, const Float4 &v) {
+    auto emit = [&](uint32_t c, const Float4 &v, const Float4 &w) {
         const bool live = c < chunks;
-        const Float4 r = rms_apply(v, scale, live ? load_chunk<VEC>(p.weight, c, n) : zero);
+        const Float4 r = rms_apply(v, scale, w);
         if (live && p.out != nullptr) store_chunk<VEC>(p.out + static_cast<uint64_t>(j) * p.stride_out, c, n, r);
         if constexpr (QUANT) {
             float d;
@@ -103,11 +106,12 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const NormParams
     };
 #pragma unroll
     for (uint32_t u = 0; u < kHeld; ++u) {
-        if (u * kNormThreads < chunks) emit(u * kNormThreads + t, held[u]);   // uniform
+        if (u * kNormThreads < chunks) emit(u * kNormThreads + t, held[u], wheld[u]);   // uniform
     }
     for (uint32_t base = kHeld * kNormThreads; base < chunks; base += kNormThreads) {
         const uint32_t c = base + t;
-        emit(c, c < chunks ? load_chunk<VEC>(x, c, n) : zero);
+        const bool live = c < chunks;
+        emit(c, live ? load_chunk<VEC>(x, c, n) : zero, live ? load_chunk<VEC>(p.weight, c, n) : zero);
     }
 }
 
