@@ -318,8 +318,8 @@ __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_kspl
     constexpr uint32_t kTail = (NSTEPS - S * WAVES) * 64 / WAVES;  // 16-byte pieces per wave of the steps left over
     static_assert((NSTEPS - S * WAVES) * 64 % WAVES == 0 && kTail % 2 == 0, "the left-over steps split evenly");
     constexpr int SL = S + (kTail ? 1 : 0);                        // register slots per wave
-    static_assert(!XF32 || (M == 1 && SL == 1 && kTail == 0 && WAVES >= 4), "fp32 activations: one row, one step per wave, the norm's tree needs four waves");
-    static_assert(!NORM || XF32, "the norm applies to fp32 activations");
+    static_assert(!XF32 || (SL == 1 && kTail == 0), "fp32 activations: one step per wave");
+    static_assert(!NORM || (XF32 && M == 1 && WAVES >= 4), "the norm applies to one fp32 row, and its tree needs four waves");
     __shared__ float part[kKsplitMaxPairs][WAVES][M][2];
     __shared__ float squares[NORM ? WAVES : 1][NORM ? kNormThreads : 1];
     __shared__ float red[4];
@@ -337,15 +337,19 @@ __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_kspl
 
     v4i xq[M][SL];
     uint16_t dxh[M][SL];
-    Float4 xv[XF32 ? 4 : 1], nw[NORM ? 4 : 1];   // XF32: the lane's 16 floats (half a block) of the wave's step
+    Float4 xv[XF32 ? M : 1][XF32 ? 4 : 1], nw[NORM ? 4 : 1];   // XF32: the lane's 16 floats (half a block) of the wave's step
     if constexpr (XF32) {
         const uint32_t at = piece_of(0) * 16;
-        const bool vec = NORM || (reinterpret_cast<uintptr_t>(p.xf) % 16 == 0);   // the norm's entry points demand alignment
+        // (the norm's entry points demand alignment)
+        const bool vec = NORM || (reinterpret_cast<uintptr_t>(p.xf) % 16 == 0 && (M == 1 || p.x_stride % 4 == 0));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            xv[i] = vec ? load4<true>(p.xf + at + 4 * i) : load4<false>(p.xf + at + 4 * i);
-            if constexpr (NORM) nw[i] = load4<true>(p.norm_w + at + 4 * i);
-        }
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float *src = p.xf + static_cast<uint64_t>(m) * p.x_stride + at + 4 * i;
+                xv[m][i] = vec ? load4<true>(src) : load4<false>(src);
+                if constexpr (NORM) nw[i] = load4<true>(p.norm_w + at + 4 * i);
+            }
         asm volatile("" ::: "memory");   // the activation loads stay ahead of the weight loads
     } else {
 #pragma unroll
@@ -381,7 +385,7 @@ __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_kspl
             // Sum of squares in the stand-alone norm's order: there thread t adds chunks t, t + 256, ...;
             // here wave u holds chunks 256 u + (0..255), so thread t adds squares[0..WAVES-1][t] ascending.
 #pragma unroll
-            for (int i = 0; i < 4; ++i) squares[w][lane * 4 + i] = chunk_squares(xv[i]);
+            for (int i = 0; i < 4; ++i) squares[w][lane * 4 + i] = chunk_squares(xv[0][i]);
             __syncthreads();
             float partial = 0.0f;
             if (threadIdx.x < kNormThreads) {
@@ -391,26 +395,29 @@ __global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_kspl
             const float scale = rms_scale(first256_tree_sum(partial, red), nb * 32, p.eps);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                xv[i] = rms_apply(xv[i], scale, nw[i]);
+                xv[0][i] = rms_apply(xv[0][i], scale, nw[i]);
                 if (p.normalized != nullptr && blockIdx.x == 0)
-                    *reinterpret_cast<float4 *>(p.normalized + piece_of(0) * 16 + 4 * i) = make_float4(xv[i].x, xv[i].y, xv[i].z, xv[i].w);
+                    *reinterpret_cast<float4 *>(p.normalized + piece_of(0) * 16 + 4 * i) = make_float4(xv[0][i].x, xv[0][i].y, xv[0][i].z, xv[0][i].w);
             }
         }
         // Q8_1 of the block this lane shares with its neighbour: the stand-alone quantizer's arithmetic
-        float amax = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(xv[i].x), fabsf(xv[i].y)), fmaxf(fabsf(xv[i].z), fabsf(xv[i].w))));
-        amax = fmaxf(amax, dpp_f32<kDppXor1>(amax));
-        const float d = amax / 127.0f;
-        int q[16];
+        for (int m = 0; m < M; ++m) {
+            float amax = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) rint_div4(xv[i], d, q[4 * i], q[4 * i + 1], q[4 * i + 2], q[4 * i + 3]);
+            for (int i = 0; i < 4; ++i)
+                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(xv[m][i].x), fabsf(xv[m][i].y)), fmaxf(fabsf(xv[m][i].z), fabsf(xv[m][i].w))));
+            amax = fmaxf(amax, dpp_f32<kDppXor1>(amax));
+            const float d = amax / 127.0f;
+            int q[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) q[i] = amax == 0.0f ? 0 : q[i];
-        xq[0][0] = v4i{static_cast<int>(pack4(q[0], q[1], q[2], q[3])), static_cast<int>(pack4(q[4], q[5], q[6], q[7])),
-                       static_cast<int>(pack4(q[8], q[9], q[10], q[11])), static_cast<int>(pack4(q[12], q[13], q[14], q[15]))};
-        dx[0][0] = half_bits_to_float(float_to_half_bits(d));
+            for (int i = 0; i < 4; ++i) rint_div4(xv[m][i], d, q[4 * i], q[4 * i + 1], q[4 * i + 2], q[4 * i + 3]);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) q[i] = amax == 0.0f ? 0 : q[i];
+            xq[m][0] = v4i{static_cast<int>(pack4(q[0], q[1], q[2], q[3])), static_cast<int>(pack4(q[4], q[5], q[6], q[7])),
+                           static_cast<int>(pack4(q[8], q[9], q[10], q[11])), static_cast<int>(pack4(q[12], q[13], q[14], q[15]))};
+            dx[m][0] = half_bits_to_float(float_to_half_bits(d));
+        }
     } else {
 #pragma unroll
         for (int m = 0; m < M; ++m)
@@ -514,7 +521,7 @@ int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
 
 // fp32 activations on rows of NSTEPS KiB: every workgroup quantizes (and normalises) the row itself,
 // each wave its own step, so a workgroup takes more pairs than with Q8_1 activations.
-template <int NSTEPS>
+template <int M, int NSTEPS>
 int launch_ksplit_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     // Pairs per workgroup.  Staging costs a workgroup about as much as four pairs, so few, long
     // workgroups: while all of them are resident at once (five waves per SIMD), a whole number per
@@ -538,7 +545,7 @@ int launch_ksplit_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
     const bool silu = p.mode == kSiluMul;
     if (p.norm_w != nullptr) {
-        if constexpr (NSTEPS <= 6) {
+        if constexpr (M == 1 && NSTEPS <= 6) {
             if (silu) gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, true, true, true><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
             else gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, false, true, true><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
             return check_launch("gemv (row pairs, fp32 activations, fused norm)");
@@ -546,8 +553,8 @@ int launch_ksplit_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
             return Q8MI_REJECTED;
         }
     }
-    if (silu) gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, true, true, false><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
-    else gemv_pairs_ksplit_kernel<1, NSTEPS, NSTEPS, false, true, false><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
+    if (silu) gemv_pairs_ksplit_kernel<M, NSTEPS, NSTEPS, true, true, false><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
+    else gemv_pairs_ksplit_kernel<M, NSTEPS, NSTEPS, false, true, false><<<grid, NSTEPS * kWave, 0, stream>>>(p, ps);
     return check_launch("gemv (row pairs, fp32 activations)");
 }
 
@@ -607,7 +614,6 @@ int launch_ring_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
 
 int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
     if (batch == 0 || batch > kPairsMaxBatch || p.nb % 8 != 0) return Q8MI_REJECTED;
-    if (p.xf != nullptr && batch > 2) return Q8MI_REJECTED;   // the quantizer runs inside the kernel at batch 1 and 2 only
     if (p.norm_w != nullptr) {   // fused norm + quantizer: one row, at most kMaxNormCols columns
         constexpr uint32_t kMaxNormCols = 6144;
         if (batch != 1) return fail(Q8MI_REJECTED, "nqgemv: batch %u above 1 (normalise and quantize once, then use the GEMV)", batch);
@@ -621,16 +627,25 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
     if (ps.pairs == 0) return Q8MI_REJECTED;
     const uint32_t cols = p.nb * kQK;
     if (p.xf != nullptr) {
-        if (batch == 1) {
+        // The quantizer inside the kernel, batch 1 and 2.  (The shared-row kernel was measured up to
+        // batch 4 in this form, fused against quantizer launch + GEMV, us: 8192 x 5120 fan-out batch 1
+        // 9.4 / 10.9, batch 2 11.2 / 11.4, batch 3 13.8 / 12.0, batch 4 21.7 / 13.1; SwiGLU batch 2
+        // 35.6 / 32.6: every workgroup repeats the quantization, which stops paying at batch 2.)
+        auto f32_by_cols = [&](auto mtag) -> int {
+            constexpr int M = decltype(mtag)::value;
             switch (cols) {
-                case 4096: return launch_ksplit_f32<4>(p, ps, stream);
-                case 5120: return launch_ksplit_f32<5>(p, ps, stream);
-                case 6144: return launch_ksplit_f32<6>(p, ps, stream);
-                case 8192: return launch_ksplit_f32<8>(p, ps, stream);
-                default: return launch_ring_f32<1>(p, ps, stream);
+                case 4096: return launch_ksplit_f32<M, 4>(p, ps, stream);
+                case 5120: return launch_ksplit_f32<M, 5>(p, ps, stream);
+                case 6144: return launch_ksplit_f32<M, 6>(p, ps, stream);
+                case 8192: return launch_ksplit_f32<M, 8>(p, ps, stream);
+                default: return launch_ring_f32<M>(p, ps, stream);
             }
+        };
+        switch (batch) {
+            case 1: return f32_by_cols(std::integral_constant<int, 1>{});
+            case 2: return f32_by_cols(std::integral_constant<int, 2>{});
+            default: return Q8MI_REJECTED;
         }
-        return launch_ring_f32<2>(p, ps, stream);
     }
     if (reinterpret_cast<uintptr_t>(p.y) % 4 != 0) return Q8MI_REJECTED;
     // rows of 4, 5, 6, 8 and 17 KiB: shared by the waves of a workgroup, activations in registers;

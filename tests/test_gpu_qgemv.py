@@ -51,6 +51,9 @@ def test_qgemv_long_rows_against_oracle(gpu, oracle, rows, cols, batch):
 @pytest.mark.parametrize("rows,cols", [(5120, 5120), (300, 2304 // 256 * 256), (129, 6144), (640, 8192), (64, 256)])
 @pytest.mark.parametrize("batch", [1, 2, 3, 5, 8])
 def test_qgemv_equals_two_step(gpu, oracle, rows, cols, batch):
+    """The quantizer inside the GEMV, batch 1 and 2: the bits of quantizer + GEMV at batch 1 and, on
+    rows of 4, 5, 6 and 8 KiB (both forms run the kernel whose waves share the rows), at batch 2;
+    on other lengths at batch 2 each form is within the tolerance of the oracle.  Declined beyond."""
     L = gpu.lib()
     w = synth.q8_0_weight(rows, cols, seed=rows + cols)
     stride_x = cols + 8
@@ -64,6 +67,7 @@ def test_qgemv_equals_two_step(gpu, oracle, rows, cols, batch):
     one = hip.DeviceBuffer(4 * n).fill(0xee)
     ok(L.q8mi_gemv(dw.ptr, dy.ptr, two.ptr, rows, cols, batch, rows, NULL), "gemv")
     rc = L.q8mi_qgemv(dw.ptr, dx.ptr, stride_x, one.ptr, 0, rows, cols, batch, rows, NULL)
+    shared_rows = cols in (4096, 5120, 6144, 8192)
     if batch > 2:
         assert rc == q8mi.REJECTED, "the fused form serves batch 1 and 2 only"
         return
@@ -73,7 +77,7 @@ def test_qgemv_equals_two_step(gpu, oracle, rows, cols, batch):
         assert batch * steps * 2304 + 16 * 4096 > 160 * 1024, "a shape that fits LDS must not be declined"
         return
     ok(rc, "qgemv")
-    if batch == 2:
+    if batch == 2 and not shared_rows:
         hip.synchronize()
         y = dy.download(np.uint8, batch * (cols // 32) * 36)
         rc, ref = oracle.gemv(w, y, rows, cols, batch, threads=8)
@@ -95,11 +99,11 @@ def test_qgemv_equals_two_step(gpu, oracle, rows, cols, batch):
     assert np.array_equal(bits(a1, n), bits(a2, n))
 
 
-@pytest.mark.parametrize("batch", [1, 2])
-def test_qgemv_silu_and_fanout_equal_two_step(gpu, batch):
+@pytest.mark.parametrize("batch,rows,cols", [(1, 1000, 1024), (2, 8192, 1024), (1, 600, 5120), (2, 600, 5120)])
+def test_qgemv_silu_and_fanout_equal_two_step(gpu, batch, rows, cols):
     L = gpu.lib()
-    # rows enough that batch 2 stays on the row-pair kernels on both routes
-    rows, cols = (1000, 1024) if batch == 1 else (8192, 1024)
+    # 1024 columns at batch 2: rows enough that it stays on the row-pair kernels on both routes;
+    # 5120 columns: a row length whose rows the waves of a workgroup share on both routes
     wg, wu = synth.q8_0_weight(rows, cols, seed=1), synth.q8_0_weight(rows, cols, seed=2)
     wk = synth.q8_0_weight(130, cols, seed=3)
     x = synth.normal(batch, cols, seed=40 + batch)
@@ -110,7 +114,7 @@ def test_qgemv_silu_and_fanout_equal_two_step(gpu, batch):
     ok(L.q8mi_gemv_silu_mul(dg.ptr, du.ptr, dy.ptr, two.ptr, rows, cols, batch, rows, NULL), "silu")
     ok(L.q8mi_qgemv_silu_mul(dg.ptr, du.ptr, dx.ptr, cols, one.ptr, rows, cols, batch, rows, NULL), "qsilu")
     assert np.array_equal(bits(one, n), bits(two, n))
-    if batch == 2:
+    if batch == 2 and cols == 1024:
         return   # the fan-out below has too few row pairs for the row-pair kernels at batch 2
     outs2 = [hip.DeviceBuffer(4 * batch * r).fill(0xff) for r in (rows, 130, rows)]
     outs1 = [hip.DeviceBuffer(4 * batch * r).fill(0xee) for r in (rows, 130, rows)]
