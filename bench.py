@@ -554,7 +554,7 @@ def main():
         "resident_gbps": round(step_bytes / (ms_resident * 1e-3) / 1e9, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(),
-                     "kernel": "gemv_pairs_ksplit_kernel<1, 5, 5, true> (SwiGLU: gate+up 2 x 5120x17408, Q8_1 activations)",
+                     "kernel": "gemv_pairs_ksplit_kernel<1, 5, 5, true, false, false> (SwiGLU: gate+up 2 x 5120x17408, Q8_1 activations)",
                      "bytes_per_launch": silu_bytes, "launch_ms": round(back_ms, 5),
                      "launch_ms_mean": round(mean_ms, 5),
                      "launch_ms_median": round(med_ms, 5), "launch_ms_min": round(min_ms, 5),

@@ -97,13 +97,15 @@ int q8mi_gemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uint
 /* ---- GEMV with the Q8_1 quantizer fused in (batch 1..2) --------------------
  * The results of q8mi_quantize_q8_1 followed by the matching q8mi_gemv* call,
  * in one launch: every workgroup quantizes the fp32 activations
- * (x: [batch][stride_x_row] floats) into LDS with the quantizer's own code
- * before its waves stream their weight rows, so no Q8_1 scratch buffer and no
- * quantizer launch are needed.  The quantized values and the per-block
- * products are the same bits as in the two-step form.  At batch 1 so are the
- * outputs for rows of up to 8192 columns; longer rows, and batch 2 (where the
- * Q8_1 entry points may run another kernel), add the same products in another
- * order (inside the GEMV's tolerance).  This is what
+ * (x: [batch][stride_x_row] floats) itself with the quantizer's own arithmetic
+ * behind its first weight requests (rows of 4096 / 5120 / 6144 / 8192 columns:
+ * each wave the 1024 columns it works on, in registers; other lengths: into
+ * LDS), so no Q8_1 scratch buffer and no quantizer launch are needed.  The
+ * quantized values and the per-block products are the same bits as in the
+ * two-step form.  So are the outputs at batch 1 for rows of up to 8192 columns
+ * and at batch 2 for the four row lengths above; longer rows, and other lengths
+ * at batch 2 (where the Q8_1 entry points may run another kernel), add the same
+ * products in another order (inside the GEMV's tolerance).  This is what
  * the reference's operators do in two steps (src/kernels_cuda.cu:10764-10888,
  * 11244-11302, 12035-12069, 12227-12258: launch_quantize_q8_1 then the
  * launcher); the fusion itself has no counterpart in the reference.
