@@ -61,3 +61,25 @@ def test_decode_layer_at_model_shapes(gpu, oracle, layer, m):
     d, dmag = linear("down", yf)
     want = (h0 + o) + d
     assert_close_fp32(step.h.download(np.float32), want, np.abs(h0) + omag + dmag, f"residual stream, M={m}")
+
+
+def test_decode_layer_with_norms_both_forms_agree(gpu, layer):
+    """The M=1 layer with its two RMS norms, as bench.py times it: norm + quantizer inside the fan-out
+    and SwiGLU launches (5 launches) against norm + quantizer kernels of their own in front of the
+    Q8_1 GEMVs (7 launches).  Same bits in every output, at the model's shapes (17408 row pairs in
+    one launch: workgroups of several rounds)."""
+    dev_layer, _ = layer
+    step = bench.DecodeStep(gpu, hip, 1, seed=77)
+    hip.synchronize()
+    h0 = step.h.download(np.float32)
+    results = []
+    for one_launch in (True, False):
+        step.h.upload(h0)
+        for buf in (step.q, step.k, step.v, step.ffn, step.x):
+            buf.fill(0xee)
+        step.run_with_norms(dev_layer, one_launch)
+        hip.synchronize()
+        results.append([b.download(np.uint32).copy() for b in (step.q, step.k, step.v, step.ffn, step.x, step.h)])
+    for name, a, b in zip(("q", "k", "v", "ffn", "normalized x", "h"), *results):
+        assert np.array_equal(a, b), name
+    assert np.isfinite(results[0][3].view(np.float32)).all()

@@ -100,7 +100,7 @@ def test_rms_norm_rejections(gpu):
     ok(L.q8mi_rms_norm(b.ptr, b.ptr, b.ptr, 0, 64, 64, 64, EPS, NULL), "empty batch")
 
 
-@pytest.mark.parametrize("rows,cols", [(333, 6144), (5120, 5120), (100, 256), (77, 1024), (40, 2304)])
+@pytest.mark.parametrize("rows,cols", [(333, 6144), (5120, 5120), (201, 4096), (100, 256), (77, 1024), (40, 2304)])
 def test_nqgemv_equals_norm_then_qgemv(gpu, oracle, rows, cols):
     L = gpu.lib()
     w = synth.q8_0_weight(rows, cols, seed=rows + cols)
@@ -164,9 +164,8 @@ def test_nqgemv_fanout4_and_silu_mul(gpu, oracle):
         two = hip.DeviceBuffer(4 * r)
         ok(L.q8mi_qgemv(dws[i].ptr, nrm2.ptr, cols, two.ptr, 0, r, cols, 1, r, NULL), "qgemv")
         hip.synchronize()
-        # a fan-out cuts the concatenated rows into other work items than a single weight does, and
-        # the order of a row's block sums follows the cut: same tolerance, not the same bits
-        assert_close_fp32(outs[i].download(np.float32), two.download(np.float32), absum, f"slot {i} against qgemv")
+        # on this row length a row's sum does not depend on how the rows are cut into work items
+        assert np.array_equal(outs[i].download(np.uint32), two.download(np.uint32)), f"slot {i} against qgemv"
     # the same fan-out in two launches gives the same bits
     two = [hip.DeviceBuffer(4 * max(r, 1)).fill(0xdd) for r in rows]
     ok(L.q8mi_qgemv_fanout4(dws[0].ptr, dws[1].ptr, dws[2].ptr, dws[3].ptr, nrm2.ptr, cols, two[0].ptr, two[1].ptr,
