@@ -5,9 +5,9 @@
 // The weights are read exactly once from HBM and nothing else is large, so every kernel here is a
 // stream over the int8 plane of each row.  This file holds the entry points, the routing between
 // the kernel families, and two of the families:
-//   batch 1, and batch 2 on launches with row pairs to spare: independent waves that own whole
-//       row pairs (q8mi_gemv_pairs.hip)
-//   batch 2..16: the matrix-core kernel below (core in q8mi_gemv_mfma_core.hpp), one workgroup per
+//   batch 1..4 (by batch, row length and form: gemv_prefers_mfma in q8mi_gemv_core.hpp): many small
+//       workgroups that own whole row pairs, handed out by the dispatcher (q8mi_gemv_pairs.hip)
+//   batch 2..16 otherwise: the matrix-core kernel below (core in q8mi_gemv_mfma_core.hpp), one workgroup per
 //       CU whose waves split the items of its units and combine partial sums through LDS
 //   fallbacks: the dot-product kernel below (core in q8mi_gemv_core.hpp) with the same static
 //       split, for activations that fit LDS in no other layout, and a one-lane-per-block kernel

@@ -1,4 +1,4 @@
-// Q8_0 x Q8_1 GEMV for batch 1..2 as many small, independent workgroups (gfx950).
+// Q8_0 x Q8_1 GEMV for batch 1..4 as many small, independent workgroups (gfx950).
 // Reference semantics: src/mmvq_q8.cu:193-280 (plain), :295-399 (two weights), :414-519 (SwiGLU),
 // :528-606 (residual add), :976-1068 (fan-out); like the reference's kernel, a weight row is read
 // once and reused for every activation row (:221-243).

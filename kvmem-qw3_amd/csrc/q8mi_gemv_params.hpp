@@ -70,7 +70,7 @@ __device__ __forceinline__ void store_out(int mode, void *dst, uint64_t idx, flo
     }
 }
 
-// Row-pair kernels for batch 1..2 (q8mi_gemv_pairs.hip): Q8MI_REJECTED when the shape is not theirs,
+// Row-pair kernels for batch 1..4 (q8mi_gemv_pairs.hip): Q8MI_REJECTED when the shape is not theirs,
 // so that the caller goes on to the streaming kernels.
 int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream);
 
