@@ -277,40 +277,36 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
     }
 }
 
-__global__ __launch_bounds__(kMaxPartials) void lm_head_finalize_kernel(
+// One wave per verify row merges that row's partials (each lane a strided share, then a butterfly
+// over the lanes; the merge rule does not depend on the order); thread 0 then walks the drafts.
+constexpr int kFinalizeThreads = Q8MI_MAX_GEMV_BATCH * kWave;
+
+__global__ __launch_bounds__(kFinalizeThreads) void lm_head_finalize_kernel(
         const q8mi_argmax_pair *__restrict__ partial, uint32_t nparts, uint32_t batch, Drafts drafts_val,
         const int32_t *__restrict__ drafts_dev, int32_t eos, q8mi_argmax_pair *__restrict__ row_out,
         int32_t *__restrict__ accept_out) {
-    __shared__ float sv[kMaxPartials];
-    __shared__ int si[kMaxPartials];
     __shared__ int tokens[Q8MI_MAX_GEMV_BATCH];
-    const uint32_t tid = threadIdx.x;
-    for (uint32_t m = 0; m < batch; ++m) {
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, m = tid / kWave;
+    if (m < batch) {   // wave-uniform
         float v = -INFINITY;
         int i = -1;
-        if (tid < nparts) {
-            const q8mi_argmax_pair p = partial[static_cast<uint64_t>(m) * nparts + tid];
-            v = p.value;
-            i = p.index;
+        for (uint32_t k = lane; k < nparts; k += kWave) {
+            const q8mi_argmax_pair p = partial[static_cast<uint64_t>(m) * nparts + k];
+            if (beats(p.value, p.index, v, i)) { v = p.value; i = p.index; }
         }
-        sv[tid] = v;
-        si[tid] = i;
-        __syncthreads();
-        for (uint32_t stride = kMaxPartials / 2; stride > 0; stride >>= 1) {
-            if (tid < stride) {
-                const float ov = sv[tid + stride];
-                const int oi = si[tid + stride];
-                if (beats(ov, oi, sv[tid], si[tid])) { sv[tid] = ov; si[tid] = oi; }
-            }
-            __syncthreads();
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) {
+            const float ov = __shfl_xor(v, d, kWave);
+            const int oi = __shfl_xor(i, d, kWave);
+            if (beats(ov, oi, v, i)) { v = ov; i = oi; }
         }
-        if (tid == 0) {
-            row_out[m].value = sv[0];
-            row_out[m].index = si[0];
-            tokens[m] = si[0];
+        if (lane == 0) {
+            row_out[m].value = v;
+            row_out[m].index = i;
+            tokens[m] = i;
         }
-        __syncthreads();
     }
+    __syncthreads();
     if (tid == 0) {
         const uint32_t n_drafts = batch - 1;
         uint32_t accepted = 0;
@@ -449,7 +445,7 @@ static int lm_head_run(const uint8_t *weight, const void *y, uint32_t rows, uint
             for (uint32_t i = 0; i + 1 < batch; ++i) dv.v[i] = drafts[i];
         }
     }
-    lm_head_finalize_kernel<<<1, kMaxPartials, 0, s>>>(partial, grid, batch, dv, ddev, eos, row_out, accept_out);
+    lm_head_finalize_kernel<<<1, kFinalizeThreads, 0, s>>>(partial, grid, batch, dv, ddev, eos, row_out, accept_out);
     return check_launch("lm_head finalize");
 }
 
