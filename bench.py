@@ -572,7 +572,7 @@ def main():
         result["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "steps_per_graph": per_graph,
                                   "gbps": round(step_bytes / (ms_graph * 1e-3) / 1e9, 1)}
         sweep = {}
-        for m in (1, 2, 4, 6, 8):
+        for m in (1, 2, 3, 4, 6, 8):
             st = step if m == 1 else DecodeStep(q8mi, hip, m=m)
             b = st.algorithmic_bytes(layers[0].bytes)
             t = time_loop(hip, lambda i: st.run(layers[i % len(layers)]), max(args.steps // 2, 300), 50)

@@ -1,6 +1,6 @@
 """GPU parity at the model's own shapes: the decode GEMV set of one layer exactly as bench.py times
 it (QKV fan-out 5120 -> 6144 + 1024 + 1024, O 6144 -> 5120 with residual, gate/up 5120 -> 17408 SwiGLU,
-down 17408 -> 5120 with residual), at M = 1 (quantizer inside the launches), 2, 4, 6 and 8, against the
+down 17408 -> 5120 with residual), at M = 1 (quantizer inside the launches), 2, 3, 4, 6 and 8, against the
 CPU oracle."""
 import numpy as np
 import pytest
@@ -24,7 +24,7 @@ def layer(gpu):
     return dev_layer, host
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 6, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8])
 def test_decode_layer_at_model_shapes(gpu, oracle, layer, m):
     dev_layer, host = layer
     step = bench.DecodeStep(gpu, hip, m, seed=40 + m)
