@@ -55,6 +55,23 @@ def test_argmax_single_row(gpu, oracle, n):
         assert p["index"] == idx and p["value"].view(np.int32) == np.float32(v).view(np.int32)
 
 
+@pytest.mark.parametrize("n", [5, 1027, 70001])
+def test_argmax_single_row_off_a_16_byte_boundary(gpu, oracle, n):
+    """Rows on a 16-byte boundary are scanned four elements per load, others one by one: same result."""
+    rows = adversarial_rows(n, seed=n + 7)
+    L = q8mi.lib()
+    out2 = hip.DeviceBuffer(8)
+    for i, r in enumerate(rows):
+        for offset in (4, 8, 12):
+            shifted = hip.DeviceBuffer(4 * n + 16)
+            shifted.upload(r, offset)
+            ok(L.q8mi_argmax(shifted.ptr + offset, n, out2.ptr, NULL), "argmax")
+            hip.synchronize()
+            got = out2.download(np.int32)
+            v, idx = oracle.argmax_row(r)
+            assert got[0] == idx and got[1] == np.float32(v).view(np.int32), f"row {i}, offset {offset}"
+
+
 def test_argmax_empty_row(gpu):
     out2 = hip.DeviceBuffer(8)
     ok(q8mi.lib().q8mi_argmax(out2.ptr, 0, out2.ptr, NULL), "argmax")
