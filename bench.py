@@ -434,6 +434,17 @@ def bench_gemm_medium(q8mi, hip, synth, reps=30):
     return out
 
 
+def bench_batch_sweep(q8mi, hip, step, layers, steps):
+    """The layer's GEMV set at M = 1, 2, 3, 4, 6, 8 (quantizer launches included)."""
+    sweep = {}
+    for m in (1, 2, 3, 4, 6, 8):
+        st = step if m == 1 else DecodeStep(q8mi, hip, m=m)
+        b = st.algorithmic_bytes(layers[0].bytes)
+        t = time_loop(hip, lambda i: st.run(layers[i % len(layers)]), steps, 50)
+        sweep[f"m{m}"] = {"ms_per_step": round(t, 5), "gbps": round(b / (t * 1e-3) / 1e9, 1)}
+    return sweep
+
+
 def bench_lm_head(q8mi, hip, synth, reps=100):
     """Fused LM head (5120 x 248320) + argmax + accept at M = 1, 2, 4, 6, 8."""
     L, ok = q8mi.lib(), q8mi.ok
@@ -496,7 +507,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
     ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["gemm", "lm_head", "ceilings"], help="one secondary figure alone (for profiling runs)")
+    ap.add_argument("--only", choices=["gemm", "lm_head", "ceilings", "sweep"], help="one secondary figure alone (for profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's throughput; run with --gpus 1 "
@@ -519,6 +530,11 @@ def main():
         return
     if args.only == "lm_head":
         print(json.dumps({"lm_head_fused": bench_lm_head(q8mi, hip, synth)}))
+        return
+    if args.only == "sweep":
+        layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
+        print(json.dumps({"gemv_layer_gbps_by_m": bench_batch_sweep(q8mi, hip, DecodeStep(q8mi, hip, m=1), layers,
+                                                                     max(args.steps // 2, 300))}))
         return
     counter_calibration(synth, hip)
     layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
@@ -571,13 +587,7 @@ def main():
         ms_graph = time_graph_replays(hip, record, max(args.steps // per_graph, 10), 3) / per_graph
         result["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "steps_per_graph": per_graph,
                                   "gbps": round(step_bytes / (ms_graph * 1e-3) / 1e9, 1)}
-        sweep = {}
-        for m in (1, 2, 3, 4, 6, 8):
-            st = step if m == 1 else DecodeStep(q8mi, hip, m=m)
-            b = st.algorithmic_bytes(layers[0].bytes)
-            t = time_loop(hip, lambda i: st.run(layers[i % len(layers)]), max(args.steps // 2, 300), 50)
-            sweep[f"m{m}"] = {"ms_per_step": round(t, 5), "gbps": round(b / (t * 1e-3) / 1e9, 1)}
-        result["gemv_layer_gbps_by_m"] = sweep
+        result["gemv_layer_gbps_by_m"] = bench_batch_sweep(q8mi, hip, step, layers, max(args.steps // 2, 300))
         # the layer's two RMS norms in front of the fan-out and the SwiGLU: inside those launches, or on their own
         norms = {}
         for name, one in (("norms_inside_the_gemv_5_launches", True), ("norm_quantizer_kernels_7_launches", False)):
