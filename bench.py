@@ -2,16 +2,18 @@
 """Bench of the Q8_0 quantized-linear hot path on one MI355X.
 
 One "step" = one pass over the decode GEMV set of one 27B-style layer at M=1
-(config 1 of the benchmark definition), through the C ABI exactly as the executor would drive it:
+(config 1 of the benchmark definition), through the C ABI, every operator reading its own fp32
+input as in the model (the fan-out reads the attention norm's output, the SwiGLU the FFN norm's):
 
-    quantize_q8_1(x[5120])    the normed row, once for the two operators that read it
-    gemv_fanout4              Q 5120x6144, K 5120x1024, V 5120x1024
-    qgemv_add(a[6144])        O 6144x5120, residual add (quantizer inside the GEMV)
-    gemv_silu_mul             gate, up 5120x17408 each
+    qgemv_fanout4(x_attn[5120])   Q 5120x6144, K 5120x1024, V 5120x1024 (quantizer inside the GEMV)
+    qgemv_add(a[6144])            O 6144x5120, residual add (quantizer inside the GEMV)
+    quantize_q8_1(x_ffn[5120])
+    gemv_silu_mul                 gate, up 5120x17408 each
     quantize_q8_1(f[17408])
-    gemv_add                  down 17408x5120, residual add
+    gemv_add                      down 17408x5120, residual add
 
-for batch 2..8 the O projection is quantize_q8_1 + gemv_add as well (7 launches).
+(the faster of "quantizer inside" and "quantizer launch + GEMV" for each operator); for batch 2..8
+every operator is quantize_q8_1 + GEMV (8 launches).
 
 `value` is algorithmic bytes per step / time per step with all inputs resident
 in HBM, cycling through several distinct copies of the layer's weights so that
@@ -69,7 +71,8 @@ class DecodeStep:
         self.ok = q8mi.ok
         self.m = m
         f32 = lambda n: hip.DeviceBuffer(4 * n)
-        self.x = hip.to_device(synth.normal(m, HIDDEN, seed=seed))          # normed hidden state
+        self.x = hip.to_device(synth.normal(m, HIDDEN, seed=seed))          # attention norm's output
+        self.x_ffn = hip.to_device(synth.normal(m, HIDDEN, seed=seed + 3))  # FFN norm's output
         self.attn = hip.to_device(synth.normal(m, ATTN_OUT, seed=seed + 1))  # attention output
         self.h = hip.to_device(synth.normal(m, HIDDEN, seed=seed + 2))       # residual stream
         self.q, self.k, self.v = f32(m * QDIM), f32(m * KVDIM), f32(m * KVDIM)
@@ -79,31 +82,32 @@ class DecodeStep:
         self.y17408 = hip.DeviceBuffer(q81_bytes(m, FFN))
 
     def algorithmic_bytes(self, layer_bytes):
-        m = self.m
-        act = 2 * q81_bytes(m, HIDDEN) + q81_bytes(m, ATTN_OUT) + q81_bytes(m, FFN)
-        outs = 4 * m * (QDIM + 2 * KVDIM + HIDDEN + FFN + HIDDEN)
-        return layer_bytes + act + outs
+        return decode_step_bytes(self.m, layer_bytes)
 
     @property
     def launches(self):
-        return 6 if self.m == 1 else 7
+        return 6 if self.m == 1 else 8
 
     def run(self, layer, stream=None):
-        """The host layer's routing: the normed row is quantized once for the fan-out and the SwiGLU
-        (they read the same row); at M=1 the O projection quantizes its input inside the GEMV (one
-        launch instead of two), every other operator reads Q8_1 blocks."""
+        """Every operator on its own fp32 input.  At M=1 the fan-out and the O projection quantize
+        inside the GEMV (one launch instead of two); the SwiGLU and the down projection, and every
+        operator at M >= 2, read Q8_1 blocks from a quantizer launch of their own."""
         L, m, w = self.L, self.m, layer.w
         ok = self.ok
-        ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize x")
-        ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.y5120.ptr,
-                               self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
-                               HIDDEN, m, QDIM, KVDIM, KVDIM, 0, stream), "fanout4")
         if m == 1:
+            ok(L.q8mi_qgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.x.ptr, HIDDEN,
+                                    self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
+                                    HIDDEN, m, QDIM, KVDIM, KVDIM, 0, stream), "qfanout4")
             ok(L.q8mi_qgemv_add(w["o"].ptr, self.attn.ptr, ATTN_OUT, self.h.ptr, 0, HIDDEN, ATTN_OUT, m, HIDDEN,
                                 stream), "qo")
         else:
+            ok(L.q8mi_quantize_q8_1(self.x.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize x")
+            ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, self.y5120.ptr,
+                                   self.q.ptr, self.k.ptr, self.v.ptr, None, QDIM, KVDIM, KVDIM, 0,
+                                   HIDDEN, m, QDIM, KVDIM, KVDIM, 0, stream), "fanout4")
             ok(L.q8mi_quantize_q8_1(self.attn.ptr, self.y6144.ptr, m, ATTN_OUT, ATTN_OUT, stream), "quantize attn")
             ok(L.q8mi_gemv_add(w["o"].ptr, self.y6144.ptr, self.h.ptr, HIDDEN, ATTN_OUT, m, HIDDEN, stream), "o")
+        ok(L.q8mi_quantize_q8_1(self.x_ffn.ptr, self.y5120.ptr, m, HIDDEN, HIDDEN, stream), "quantize x_ffn")
         self.run_silu(layer, stream)
         ok(L.q8mi_quantize_q8_1(self.ffn.ptr, self.y17408.ptr, m, FFN, FFN, stream), "quantize ffn")
         ok(L.q8mi_gemv_add(w["down"].ptr, self.y17408.ptr, self.h.ptr, HIDDEN, FFN, m, HIDDEN, stream), "down")
@@ -257,8 +261,10 @@ def cpu_baseline(seconds=12.0):
     one, n1 = run(1, seconds / 2)
     many, nm = run(cores, seconds / 2)
     return {"value": round(many, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "host_cpu_count": os.cpu_count(),
             "sample": f"oracle q8o_gemv, config 0 (5120x5120, M=1), {nm} calls row-parallel on {cores} threads "
-                      f"(~{seconds / 2:.0f} s); single core: {one:.3f} GB/s over {n1} calls",
+                      f"of the {os.cpu_count()} the host reports (~{seconds / 2:.0f} s); single core: {one:.3f} GB/s "
+                      f"over {n1} calls",
             "value_1core": round(one, 3)}
 
 
@@ -326,15 +332,15 @@ def bench_launches_m1(q8mi, hip, synth, step, layers, reps=300):
 
     def fan(i):
         w = layers[i % nl].w
-        ok(L.q8mi_gemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, step.y5120.ptr, step.q.ptr, step.k.ptr,
-                               step.v.ptr, None, QDIM, KVDIM, KVDIM, 0, HIDDEN, m, QDIM, KVDIM, KVDIM, 0, None), "fanout4")
+        ok(L.q8mi_qgemv_fanout4(w["q"].ptr, w["k"].ptr, w["v"].ptr, None, step.x.ptr, HIDDEN, step.q.ptr, step.k.ptr,
+                                step.v.ptr, None, QDIM, KVDIM, KVDIM, 0, HIDDEN, m, QDIM, KVDIM, KVDIM, 0, None), "qfanout4")
     ops = [
-        ("quantize_q8_1 x (5120 floats)", 0,
-         lambda i: ok(L.q8mi_quantize_q8_1(step.x.ptr, step.y5120.ptr, m, HIDDEN, HIDDEN, None), "quantize")),
-        ("gemv_fanout4 q/k/v 8192x5120", w_bytes(QDIM + 2 * KVDIM, HIDDEN), fan),
+        ("qgemv_fanout4 q/k/v 8192x5120 (fp32 in)", w_bytes(QDIM + 2 * KVDIM, HIDDEN), fan),
         ("qgemv_add o 5120x6144 (fp32 in)", w_bytes(HIDDEN, ATTN_OUT),
          lambda i: ok(L.q8mi_qgemv_add(layers[i % nl].w["o"].ptr, step.attn.ptr, ATTN_OUT, step.h.ptr, 0, HIDDEN,
                                        ATTN_OUT, m, HIDDEN, None), "qo")),
+        ("quantize_q8_1 x_ffn (5120 floats)", 0,
+         lambda i: ok(L.q8mi_quantize_q8_1(step.x_ffn.ptr, step.y5120.ptr, m, HIDDEN, HIDDEN, None), "quantize")),
         ("gemv_silu_mul gate/up 2x17408x5120", 2 * w_bytes(FFN, HIDDEN), lambda i: step.run_silu(layers[i % nl])),
         ("quantize_q8_1 ffn (17408 floats)", 0,
          lambda i: ok(L.q8mi_quantize_q8_1(step.ffn.ptr, step.y17408.ptr, m, FFN, FFN, None), "quantize")),
@@ -434,6 +440,169 @@ def bench_gemm_medium(q8mi, hip, synth, reps=30):
     return out
 
 
+def split_to_gguf(split, rows, cols):
+    """Split-plane rows ([fp16 d x nb][int8 x 32 nb]) back to interleaved 34-byte GGUF blocks:
+    what DeviceBackend::weight_q8_0 takes."""
+    nb = cols // 32
+    rows_v = np.asarray(split, np.uint8).reshape(rows, nb * 34)
+    d = rows_v[:, :2 * nb].reshape(rows, nb, 2)
+    q = rows_v[:, 2 * nb:].reshape(rows, nb, 32)
+    return np.ascontiguousarray(np.concatenate([d, q], axis=2)).reshape(-1)
+
+
+class BackendSteps:
+    """The layer's operators driven through qw3::HipQ8Backend (the C++ mirror of the reference's
+    DeviceBackend) in the executors' call order: tests/cpp/backend_steps.cpp behind ctypes."""
+
+    SHAPES = (("q", QDIM, HIDDEN), ("k", KVDIM, HIDDEN), ("v", KVDIM, HIDDEN), ("o", HIDDEN, ATTN_OUT),
+              ("gate", FFN, HIDDEN), ("up", FFN, HIDDEN), ("down", HIDDEN, FFN))
+
+    def __init__(self, synth, n_layers):
+        path = os.path.join(ROOT, "tests", "cpp", "libbackend_steps.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: run __graft_entry__.build()")
+        B = C.CDLL(path)
+        B.bsteps_create.restype = C.c_void_p
+        B.bsteps_create.argtypes = [C.c_uint32] * 5
+        B.bsteps_destroy.argtypes = [C.c_void_p]
+        B.bsteps_error.restype = C.c_char_p
+        B.bsteps_error.argtypes = [C.c_void_p]
+        B.bsteps_add_layer.argtypes = [C.c_void_p] * 8
+        B.bsteps_set_head.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32]
+        B.bsteps_prepare.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p]
+        B.bsteps_time_layers.restype = C.c_double
+        B.bsteps_time_layers.argtypes = [C.c_void_p, C.c_int, C.c_uint32, C.c_uint32]
+        B.bsteps_time_head.restype = C.c_double
+        B.bsteps_time_head.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        self.B, self.synth = B, synth
+        self.h = B.bsteps_create(HIDDEN, QDIM, KVDIM, ATTN_OUT, FFN)
+        for s in range(n_layers):
+            blocks = [split_to_gguf(synth.q8_0_weight(r, c, seed=(s + 1) * 16 + i, sigma=0.02), r, c)
+                      for i, (_, r, c) in enumerate(self.SHAPES)]
+            if B.bsteps_add_layer(self.h, *[b.ctypes.data_as(C.c_void_p) for b in blocks]) < 0:
+                raise RuntimeError("backend steps: weight upload failed")
+
+    def prepare(self, m):
+        h, mid = self.synth.normal(m, HIDDEN, seed=71), self.synth.normal(m, ATTN_OUT, seed=72)
+        if self.B.bsteps_prepare(self.h, m, h.ctypes.data_as(C.c_void_p), mid.ctypes.data_as(C.c_void_p)) != 0:
+            raise RuntimeError("backend steps: tensor set-up failed")
+
+    def time_layers(self, order, steps, warmup):
+        ms = self.B.bsteps_time_layers(self.h, order, steps, warmup)
+        if ms < 0:
+            raise RuntimeError("backend steps: " + (self.B.bsteps_error(self.h) or b"").decode())
+        return ms
+
+    def set_head(self):
+        blocks = split_to_gguf(self.synth.q8_0_weight(VOCAB, HIDDEN, seed=4242), VOCAB, HIDDEN)
+        if self.B.bsteps_set_head(self.h, blocks.ctypes.data_as(C.c_void_p), VOCAB) != 0:
+            raise RuntimeError("backend steps: LM head upload failed")
+
+    def time_head(self, calls, warmup):
+        ms = self.B.bsteps_time_head(self.h, calls, warmup, None, None)
+        if ms < 0:
+            raise RuntimeError("backend steps: " + (self.B.bsteps_error(self.h) or b"").decode())
+        return ms
+
+    def close(self):
+        self.B.bsteps_destroy(self.h)
+
+
+def bench_backend_layers(synth, n_layers, steps, layer_bytes, with_head=True):
+    """Microseconds per layer step through HipQ8Backend: decode (M=1) in the executor's order, and
+    M = 2, 4, 6, 8 in the executor's batched order (matmul + add_n) and the continuous-batching
+    verifier's (matmul_add in place); the two RMS norms of the layer are part of each step.  Also the
+    verify tail (final norm + fused LM head, host read of the accept result included)."""
+    bs = BackendSteps(synth, n_layers)
+    out = {}
+    try:
+        bs.prepare(1)
+        t = bs.time_layers(-1, steps, 50)
+        b1 = decode_step_bytes(1, layer_bytes)
+        out["decode_m1"] = {"us_per_layer": round(t * 1e3, 2), "gbps": round(b1 / (t * 1e-3) / 1e9, 1)}
+        for m in (2, 4, 6, 8):
+            bs.prepare(m)
+            row = {}
+            for name, order in (("executor_order", 0), ("matmul_add_order", 1)):
+                t = bs.time_layers(order, steps, 50)
+                row[name] = {"us_per_layer": round(t * 1e3, 2),
+                             "gbps": round(decode_step_bytes(m, layer_bytes) / (t * 1e-3) / 1e9, 1)}
+            out[f"verify_m{m}"] = row
+        if with_head:
+            bs.set_head()
+            head = {}
+            for m in (1, 2, 4, 6, 8):
+                bs.prepare(m)
+                t = bs.time_head(60, 20)
+                nbytes = w_bytes(VOCAB, HIDDEN) + q81_bytes(m, HIDDEN) + 8 * m
+                head[f"m{m}"] = {"ms": round(t, 4), "gbps": round(nbytes / (t * 1e-3) / 1e9, 1)}
+            out["norm_plus_lm_head_verify"] = head
+    finally:
+        bs.close()
+    return out
+
+
+def decode_step_bytes(m, layer_bytes):
+    """Algorithmic bytes of one layer's GEMV set at batch m: the weights once, the Q8_1 blocks of the
+    four activation rows, the fp32 outputs."""
+    act = 2 * q81_bytes(m, HIDDEN) + q81_bytes(m, ATTN_OUT) + q81_bytes(m, FFN)
+    outs = 4 * m * (QDIM + 2 * KVDIM + HIDDEN + FFN + HIDDEN)
+    return layer_bytes + act + outs
+
+
+def bench_prefill_ffn(q8mi, hip, synth, m=2048, reps=12):
+    """The FFN block of a prefill chunk of m rows as a sequence, repeated back to back: D4 quantizer,
+    gate/up SwiGLU, D4 quantizer, down projection + residual.  `separate`: the launches the
+    reference's executor runs (two GEMMs + silu_mul, GEMM + add); `fused`: one tile launch per
+    operator where the library has one (q8mi_gemm_silu_mul; q8mi_gemm_add unless it declines the shape)."""
+    L, ok = q8mi.lib(), q8mi.ok
+    wg = hip.to_device(synth.q8_0_weight(FFN, HIDDEN, seed=501))
+    wu = hip.to_device(synth.q8_0_weight(FFN, HIDDEN, seed=502))
+    wd = hip.to_device(synth.q8_0_weight(HIDDEN, FFN, seed=503))
+    x = hip.to_device(synth.normal(m, HIDDEN, seed=504))
+    h = hip.to_device(synth.normal(m, HIDDEN, seed=505))
+    yx = hip.DeviceBuffer(L.q8mi_q8_1_d4_scratch_bytes(m, HIDDEN))
+    yf = hip.DeviceBuffer(L.q8mi_q8_1_d4_scratch_bytes(m, FFN))
+    gate, up, mid = (hip.DeviceBuffer(4 * m * FFN) for _ in range(3))
+    tmp = hip.DeviceBuffer(4 * m * HIDDEN)
+    add_fuses = L.q8mi_gemm_add(wd.ptr, yf.ptr, h.ptr, h.ptr, HIDDEN, FFN, m, HIDDEN, None) == q8mi.OK
+
+    def down_separate():
+        ok(L.q8mi_gemm(wd.ptr, yf.ptr, tmp.ptr, HIDDEN, FFN, m, HIDDEN, None), "gemm down")
+        ok(L.q8mi_add(h.ptr, h.ptr, tmp.ptr, m * HIDDEN, 0, None), "add")
+
+    def separate(i):
+        ok(L.q8mi_quantize_q8_1_d4(x.ptr, yx.ptr, m, HIDDEN, HIDDEN, None), "quantize x")
+        ok(L.q8mi_gemm(wg.ptr, yx.ptr, gate.ptr, FFN, HIDDEN, m, FFN, None), "gemm gate")
+        ok(L.q8mi_gemm(wu.ptr, yx.ptr, up.ptr, FFN, HIDDEN, m, FFN, None), "gemm up")
+        ok(L.q8mi_silu_mul(mid.ptr, gate.ptr, up.ptr, m * FFN, None), "silu_mul")
+        ok(L.q8mi_quantize_q8_1_d4(mid.ptr, yf.ptr, m, FFN, FFN, None), "quantize mid")
+        down_separate()
+
+    def fused(i):
+        ok(L.q8mi_quantize_q8_1_d4(x.ptr, yx.ptr, m, HIDDEN, HIDDEN, None), "quantize x")
+        ok(L.q8mi_gemm_silu_mul(wg.ptr, wu.ptr, yx.ptr, mid.ptr, FFN, HIDDEN, m, FFN, None), "gemm_silu_mul")
+        ok(L.q8mi_quantize_q8_1_d4(mid.ptr, yf.ptr, m, FFN, FFN, None), "quantize mid")
+        if add_fuses:
+            ok(L.q8mi_gemm_add(wd.ptr, yf.ptr, h.ptr, h.ptr, HIDDEN, FFN, m, HIDDEN, None), "gemm_add")
+        else:
+            down_separate()
+
+    # alternate the two forms so that both see the same clocks: sustained matrix work runs the chip at its power limit
+    t_sep, t_fus = [], []
+    for _ in range(3):
+        t_sep.append(time_loop(hip, separate, reps, 2))
+        t_fus.append(time_loop(hip, fused, reps, 2))
+    ops = 2.0 * m * FFN * HIDDEN * 3
+    for b in (wg, wu, wd, x, h, yx, yf, gate, up, mid, tmp):
+        b.free()
+    t_s, t_f = min(t_sep), min(t_fus)
+    return {"m": m, "separate_launches_ms": round(t_s, 4), "fused_stores_ms": round(t_f, 4),
+            "separate_tops": round(ops / (t_s * 1e-3) / 1e12, 1), "fused_tops": round(ops / (t_f * 1e-3) / 1e12, 1),
+            "down_plus_residual_in_one_launch": add_fuses, "all_rounds_ms": {"separate": [round(t, 4) for t in t_sep],
+                                                                             "fused": [round(t, 4) for t in t_fus]}}
+
+
 def bench_batch_sweep(q8mi, hip, step, layers, steps):
     """The layer's GEMV set at M = 1, 2, 3, 4, 6, 8 (quantizer launches included)."""
     sweep = {}
@@ -507,7 +676,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
     ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["gemm", "lm_head", "ceilings", "sweep"], help="one secondary figure alone (for profiling runs)")
+    ap.add_argument("--only", choices=["gemm", "lm_head", "ceilings", "sweep", "backend", "prefill_ffn"], help="one secondary figure alone (for profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's throughput; run with --gpus 1 "
@@ -530,6 +699,14 @@ def main():
         return
     if args.only == "lm_head":
         print(json.dumps({"lm_head_fused": bench_lm_head(q8mi, hip, synth)}))
+        return
+    if args.only == "backend":
+        lb = sum(w_bytes(r, c) for _, r, c in BackendSteps.SHAPES)
+        print(json.dumps({"through_hip_q8_backend": bench_backend_layers(synth, args.copies, max(args.steps // 2, 300), lb)}))
+        return
+    if args.only == "prefill_ffn":
+        print(json.dumps({"prefill_ffn_block": {f"m{m}": bench_prefill_ffn(q8mi, hip, synth, m=m, reps=r)
+                                                for m, r in ((2048, 12), (8192, 4))}}))
         return
     if args.only == "sweep":
         layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
@@ -595,6 +772,8 @@ def main():
             norms[name] = {"ms_per_step": round(t, 5), "gbps": round(step_bytes / (t * 1e-3) / 1e9, 1)}
         result["layer_with_rms_norms_m1"] = norms
         result["launches_m1"] = bench_launches_m1(q8mi, hip, synth, step, layers)
+        # the same layer through the C++ operator layer, in the executors' call order
+        result["through_hip_q8_backend"] = bench_backend_layers(synth, len(layers), max(args.steps // 2, 300), layers[0].bytes)
     for l in layers[1:]:
         for b in l.w.values():
             b.free()
@@ -614,6 +793,7 @@ def main():
                                    "ops_per_launch": 2 * 2048 * FFN * HIDDEN, "launch_ms": g["gemm_ms"],
                                    "frac_of_measured_rescale_ceiling": g["frac_of_rescale_ceiling"]}
         result["gemm_medium_batches"] = bench_gemm_medium(q8mi, hip, synth)
+        result["prefill_ffn_block"] = {f"m{m}": bench_prefill_ffn(q8mi, hip, synth, m=m, reps=r) for m, r in ((2048, 12), (8192, 4))}
         result["lm_head_fused"] = bench_lm_head(q8mi, hip, synth)
     if not (args.quick or args.no_cpu):
         result["cpu_baseline"] = cpu_baseline()

@@ -196,6 +196,43 @@ int q8mi_gemm(const uint8_t *weight, const void *y, float *dst, uint32_t rows, u
 int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *dst, uint32_t rows,
                      uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
 
+/* The batched forms of the executor's fused operators, one launch each where the reference's CUDA
+ * backend runs its tile GEMM into a temporary and a second kernel over the batch x rows outputs.
+ * All three take D4 activations and serve rows >= 128, cols % 256 == 0 (every model shape);
+ * anything else, and the shapes named below, is Q8MI_REJECTED (nothing enqueued) and the caller
+ * runs the two-step form.
+ *
+ * q8mi_gemm_add: dst[j][r] = residual[j][r] + (W x)[j][r]; residual rows are stride_dst_row floats
+ * apart like dst's and residual may be dst.  Replaces launch_mmq_q8_0 into matmul_tmp followed by
+ * add_kernel (q8_0_matmul_add, include/qw3/device_backend.hpp:529-540, src/kernels_cuda.cu:11919-11957,
+ * 1644-1652); same bits as q8mi_gemm + q8mi_add wherever q8mi_gemm does not sum from two halves of K.
+ * Rejected: batch <= 16 out of place (in place the matrix-core GEMV adds as q8mi_gemv_add does), and
+ * shapes q8mi_gemm serves by adding two halves of K into a zeroed dst (a partly filled last round of
+ * 128 x 128 tiles, or at most one 32-row tile per CU at batch <= 32): a sum that arrives in halves
+ * cannot meet the residual in an order that repeats, and on those shapes q8mi_gemm + q8mi_add is the
+ * faster route anyway. */
+int q8mi_gemm_add(const uint8_t *weight, const void *y_d4, const float *residual, float *dst, uint32_t rows,
+                  uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
+/* q8mi_gemm with bf16 outputs (round to nearest even in the store): replaces launch_mmq_q8_0 into an
+ * fp32 workspace followed by convert_q8_output_bf16 (src/kernels_cuda.cu:14509-14530).  Rejected:
+ * batch <= 16 (a weight stream: quantize to Q8_1 and use q8mi_gemv_bf16) and the two-halves shapes above. */
+int q8mi_gemm_bf16(const uint8_t *weight, const void *y_d4, uint16_t *dst, uint32_t rows, uint32_t cols,
+                   uint32_t batch, uint32_t stride_dst_row, void *stream);
+/* dst[j][r] = silu((Wg x)[j][r]) * (Wu x)[j][r], silu(g) = g / (1 + exp(-g)): the batched SwiGLU the
+ * operator interface asks for (q8_0_matmul_silu_mul, include/qw3/device_backend.hpp:330-336).  The
+ * reference's CUDA backend declines it for Q8_0 (src/kernels_cuda.cu:12323-12333) and the executor
+ * then runs launch_mmq_q8_0 twice and silu_mul_kernel (src/qwen_executor.cpp:6669-6685,
+ * src/kernels_cuda.cu:1894-1911): five passes over batch x rows floats that this call replaces by
+ * one write.  Every tile holds gate rows and the matching up rows, so both sums of an output meet in
+ * one lane.  Any batch: the matrix-core GEMV up to 16 rows where one pass covers them, 32 + 32-row
+ * ring tiles for medium batches, 64 + 64-row main tiles from about 0.4 tiles per workgroup slot. */
+int q8mi_gemm_silu_mul(const uint8_t *weight_gate, const uint8_t *weight_up, const void *y_d4, float *dst,
+                       uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
+
+/* replaces silu_mul_kernel, src/kernels_cuda.cu:1894-1911, as launched by silu_mul and silu_mul_n
+ * (:14880-14900): out[i] = silu(gate[i]) * up[i] for i < n (fp32).  out may be gate or up. */
+int q8mi_silu_mul(float *out, const float *gate, const float *up, uint64_t n, void *stream);
+
 /* replaces fp32_to_bf16_kernel as used by convert_q8_output_bf16,
  * src/kernels_cuda.cu:14523-14530: out[i] = bf16(in[i]), round to nearest even. */
 int q8mi_f32_to_bf16(const float *in, uint16_t *out, uint64_t n, void *stream);

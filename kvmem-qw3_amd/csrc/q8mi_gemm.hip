@@ -41,8 +41,9 @@ namespace q8mi {
 int gemv_any_batch(const uint8_t *w, const void *y_q8_1, float *dst, uint32_t rows, uint32_t cols,
                    uint32_t batch, uint32_t stride_dst_row, hipStream_t stream);
 // Matrix-core GEMV on D4 activations (q8mi_gemv.hip): small batches, else Q8MI_REJECTED.
-int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, uint32_t cols, uint32_t batch,
-                 uint32_t stride_dst_row, hipStream_t stream);
+// w_up != nullptr: the SwiGLU form (dst = silu(w x) * (w_up x)); add: dst += w x instead of a store.
+int gemv_mfma_d4(const uint8_t *w, const uint8_t *w_up, const void *y_d4, float *dst, uint32_t rows, uint32_t cols,
+                 uint32_t batch, uint32_t stride_dst_row, bool add, hipStream_t stream);
 
 namespace {
 
@@ -54,6 +55,28 @@ constexpr int kStageBytes = kTileRows * kRec + kTileCols * kRec + 4 * kTileCols 
 constexpr int kLdsBytes = 2 * kStageBytes;                                             // 77824
 constexpr uint32_t kMagicBits = 0x4B400000u;  // 1.5 * 2^23
 constexpr float kMagic = 12582912.0f;
+
+// What a tile does with its sums.  Store / bf16 store / residual add differ only after the K loop
+// and are a wave-uniform run-time switch there; the SwiGLU form stages the rows of two weights
+// and is a template parameter of the kernels (SILU).
+enum : uint32_t {
+    kEpiStore = 0,       // dst[j][r] = sum                              (fp32)
+    kEpiStoreBf16 = 1,   // dst[j][r] = bf16(sum), round to nearest even (what f32_to_bf16 would store)
+    kEpiAdd = 2,         // dst[j][r] = residual[j][r] + sum             (fp32; residual may be dst)
+};
+struct TileOut {
+    void *dst;
+    const float *residual;   // kEpiAdd only; rows stride_dst apart like dst
+    uint32_t stride_dst;
+    uint32_t epi;
+};
+
+__device__ __forceinline__ void emit(const TileOut &o, uint64_t idx, float v) {
+    if (o.epi == kEpiStoreBf16) static_cast<uint16_t *>(o.dst)[idx] = float_to_bf16_bits(v);
+    else if (o.epi == kEpiAdd) static_cast<float *>(o.dst)[idx] = o.residual[idx] + v;
+    else static_cast<float *>(o.dst)[idx] = v;
+}
+__device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.0f + __expf(-g))) * u; }
 
 struct Prefetch {
     v4i wq[4];   // 4 x 16 B of weight quants
@@ -339,16 +362,21 @@ __device__ __forceinline__ void stage_scales(uint8_t *stage, const Scales &sc, u
     }
 }
 
-template <bool CHECK, int RB>
+// SILU: the tile's first RB / 2 blocks of 32 LDS rows hold rows of the gate weight `w`, the other
+// RB / 2 the same rows of the up weight `w2`; a lane's sums for gate row r and up row r then sit in
+// the same lane (acc[rb] and acc[rb + RB / 2]) and the store writes silu(gate) * up, so a tile
+// yields 16 * RB output rows and `rows` counts the rows of one weight.
+template <bool CHECK, int RB, bool SILU>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
-        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
-        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles,
-        uint32_t split_from) {
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ w2, const uint8_t *__restrict__ y, const TileOut out,
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t row_tiles, uint32_t col_tiles, uint32_t split_from) {
     using T = DmaTile<RB>;
+    constexpr uint32_t kOut = SILU ? T::kRows / 2 : T::kRows;   // output rows of a tile
     extern __shared__ __align__(16) uint8_t smem[];
     const uint32_t tid = threadIdx.x, lane = tid % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
+    const uint32_t stride_dst = out.stride_dst;
     // Tiles from split_from on are computed by two workgroups, one per half of K, which add their
     // sums into a zeroed dst (see launch_dma): the tiles of a last, partly filled round.
     uint32_t id = blockIdx.x, k_half = 0;
@@ -362,7 +390,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
     const uint32_t xcd = id % 8u, seq = id / 8u;
     const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
     if (rt >= row_tiles) return;   // uniform for the workgroup
-    const uint32_t row0 = rt * T::kRows, col0 = ct * kTileCols;
+    const uint32_t row0 = rt * kOut, col0 = ct * kTileCols;
     const uint32_t nsb = nb / 4;
     const uint32_t sb0 = (split && k_half) ? nsb / 2 : 0u;
     const uint32_t sb1 = (split && !k_half) ? nsb / 2 : nsb;
@@ -380,21 +408,25 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
     LaneOffsets<RB> lo;
 #pragma unroll
     for (int i = 0; i < RB; ++i) {
-        const uint32_t r = (wave * RB + i) * 8 + lane / 8;
-        uint32_t gr = r;
-        if (CHECK) gr = row0 + r < rows ? r : rows - 1 - row0;   // rows past the end re-read the last row
+        const uint32_t r = (wave * RB + i) * 8 + lane / 8;   // LDS row of the tile
+        uint32_t gr = r % kOut;                               // weight row, counted from the tile's first
+        if (CHECK) gr = row0 + gr < rows ? gr : rows - 1 - row0;   // rows past the end re-read the last row
         lo.wq[i] = gr * static_cast<uint32_t>(row_bytes) + ((lane & 7u) ^ swz(r)) * 16;
     }
     lo.yr = lane * 16;
     {
-        uint32_t gr = tid & (T::kRows - 1);
+        uint32_t gr = (tid & (T::kRows - 1)) % kOut;
         if (CHECK) gr = row0 + gr < rows ? gr : rows - 1 - row0;
         lo.sc = gr * static_cast<uint32_t>(row_bytes);
         lo.ysc = (tid & 127u) * kRec;
     }
     const uint64_t y_step = static_cast<uint64_t>(batch) * kRec;
-    const uint8_t *wd_base = uniform_ptr(w + row0 * row_bytes + sb0 * 8u);   // scale plane of the tile's first row
-    const uint8_t *wq_base = wd_base + 2 * nb - sb0 * 8u + sb0 * 128u;       // its quant plane
+    // Which weight a wave stages is wave-uniform: quants, waves 0 .. 3 take LDS rows 32 wave ..; scales,
+    // thread t < 128 takes LDS row t (wave 0: rows 0 .. 63, wave 1: rows 64 .. 127).
+    const uint8_t *wq_src = (SILU && wave >= 2) ? w2 : w;
+    const uint8_t *wd_src = (SILU && wave == 1) ? w2 : w;
+    const uint8_t *wd_base = uniform_ptr(wd_src + row0 * row_bytes + sb0 * 8u);             // scale plane of the tile's first row
+    const uint8_t *wq_base = uniform_ptr(wq_src + row0 * row_bytes + 2 * nb + sb0 * 128u);  // quant plane
     const uint8_t *y_base = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec + sb0 * y_step);
     // last 16-byte offset from y_base that is still inside the activation buffer (used when CHECK)
     uint64_t y_room = static_cast<uint64_t>(nsb - sb0) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
@@ -457,8 +489,22 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
         __syncthreads();
     }
     // D[i][n]: n = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (activation row)
+    if constexpr (SILU) {
+#pragma unroll
+        for (int rb = 0; rb < RB / 2; ++rb) {
+            const uint32_t r = row0 + rb * 32 + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t j = col0 + wave * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
+                if (!CHECK || (r < rows && j < batch))
+                    static_cast<float *>(out.dst)[static_cast<uint64_t>(j) * stride_dst + r] = silu_mul(acc[rb][v], acc[rb + RB / 2][v]);
+            }
+        }
+        return;
+    }
     if (split) {
         // two addends onto zero: the sum does not depend on which half arrives first
+        float *dst = static_cast<float *>(out.dst);
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
             const uint32_t r = row0 + rb * 32 + l32;
@@ -477,7 +523,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_d4_dma_kernel(
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t j = col0 + wave * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
-            if (!CHECK || (r < rows && j < batch)) dst[static_cast<uint64_t>(j) * stride_dst + r] = acc[rb][v];
+            if (!CHECK || (r < rows && j < batch)) emit(out, static_cast<uint64_t>(j) * stride_dst + r, acc[rb][v]);
         }
     }
 }
@@ -554,14 +600,20 @@ __device__ __forceinline__ void wait_ring(uint32_t steps) {
     }
 }
 
-template <int CB, int W, int NS, bool KSPLIT, int RB = 1>
+// SILU (RB even): the first RB / 2 blocks of 32 LDS rows hold rows of the gate weight `w`, the others
+// the same rows of the up weight `w2`; the tile yields 16 * RB rows of silu(gate) * up and `rows`
+// counts the rows of one weight.
+template <int CB, int W, int NS, bool KSPLIT, int RB = 1, bool SILU = false>
 __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
-        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, float *__restrict__ dst,
-        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t stride_dst, uint32_t row_tiles, uint32_t col_tiles) {
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ w2, const uint8_t *__restrict__ y, const TileOut out,
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t row_tiles, uint32_t col_tiles) {
     constexpr bool ksplit = KSPLIT;
-    static_assert(!KSPLIT || RB == 1, "only the narrowest tile is cut along K");
+    static_assert(!KSPLIT || (RB == 1 && !SILU), "only the narrowest tile is cut along K");
+    static_assert(!SILU || RB % 2 == 0, "a SwiGLU tile holds as many gate rows as up rows");
     using T = RingTile<CB, W, RB>;
     constexpr uint32_t S = T::kShares;
+    constexpr uint32_t kOut = SILU ? T::kRows / 2 : T::kRows;   // output rows of a tile
+    const uint32_t stride_dst = out.stride_dst;
     extern __shared__ __align__(16) uint8_t smem[];
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -573,7 +625,7 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     const uint32_t xcd = id % 8u, seq = id / 8u;
     const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
     if (rt >= row_tiles) return;   // uniform for the workgroup
-    const uint32_t row0 = rt * T::kRows, col0 = ct * T::kCols;
+    const uint32_t row0 = rt * kOut, col0 = ct * T::kCols;
     const uint32_t nsb_all = nb / 4;
     const uint32_t sb0 = (ksplit && k_half) ? nsb_all / 2 : 0u;                   // first super-block of this workgroup
     const uint32_t nsb = ((ksplit && !k_half) ? nsb_all / 2 : nsb_all) - sb0;     // and how many it covers
@@ -582,7 +634,10 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     // The pieces of a step this wave loads: kind and LDS position are wave-uniform, the per-lane
     // source offsets do not change over the K loop.  Weight rows past the end re-read the last row,
     // activation rows past the end of the batch the last activation row (never stored).
-    auto clamp_row = [&](uint32_t r) { return row0 + r < rows ? r : rows - 1 - row0; };
+    auto clamp_row = [&](uint32_t r) {   // LDS row of the tile -> weight row, counted from the tile's first
+        r %= kOut;
+        return row0 + r < rows ? r : rows - 1 - row0;
+    };
     uint32_t lane_off[T::kLoads];
 #pragma unroll
     for (int i = 0; i < T::kLoads; ++i) {
@@ -604,6 +659,7 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
         }
     }
     const uint8_t *wd_base0 = uniform_ptr(w + row0 * row_bytes);
+    const uint8_t *wd_base1 = SILU ? uniform_ptr(w2 + row0 * row_bytes) : wd_base0;   // the up weight's rows
     const uint8_t *y_base0 = uniform_ptr(y + static_cast<uint64_t>(col0) * kRec);
     const uint64_t y_step = static_cast<uint64_t>(batch) * kRec;
     const uint64_t y_room0 = static_cast<uint64_t>(nsb_all) * batch * kRec - static_cast<uint64_t>(col0) * kRec - 16;
@@ -612,8 +668,7 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
     auto issue = [&](uint32_t step) {   // step counts from this workgroup's first super-block
         const uint32_t stage_off = smem_off + (step % NS) * T::kStage;
         const uint32_t gstep = sb0 + step;
-        const uint8_t *wd_base = wd_base0 + static_cast<uint64_t>(gstep) * 8;
-        const uint8_t *wq_base = wd_base0 + 2 * nb + static_cast<uint64_t>(gstep) * 128;
+        const uint64_t wd_step = static_cast<uint64_t>(gstep) * 8, wq_step = 2 * nb + static_cast<uint64_t>(gstep) * 128;
         const uint8_t *y_base = y_base0 + gstep * y_step;
         const uint64_t room = y_room0 - gstep * y_step;
         const uint32_t y_limit = static_cast<uint32_t>(room < 0xffffffffull ? room : 0xffffffffull);
@@ -622,14 +677,15 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
             uint32_t item = wave + W * i;
             item = item < T::kItems ? item : T::kItems - 1;
             if (item < T::kWItems) {
-                dma16(wq_base, lane_off[i], stage_off + item * 1024);
+                dma16((SILU && item >= T::kWItems / 2 ? wd_base1 : wd_base0) + wq_step, lane_off[i], stage_off + item * 1024);
             } else if (item < T::kWItems + T::kYChunks) {
                 const uint32_t off = lane_off[i] <= y_limit ? lane_off[i] : y_limit;   // never past the buffer
                 dma16(y_base, off, stage_off + T::kOffYr + (item - T::kWItems) * 1024);
             } else if (item < T::kWItems + T::kYChunks + T::kDyItems) {
                 dma4(y_base, lane_off[i], stage_off + T::kOffDy + (item - T::kWItems - T::kYChunks) * 256);
             } else {
-                dma4(wd_base, lane_off[i], stage_off + T::kOffWsc + (item - T::kWItems - T::kYChunks - T::kDyItems) * 256);
+                const uint32_t blk32 = item - T::kWItems - T::kYChunks - T::kDyItems;   // block of 32 LDS rows
+                dma4((SILU && blk32 >= RB / 2 ? wd_base1 : wd_base0) + wd_step, lane_off[i], stage_off + T::kOffWsc + blk32 * 256);
             }
         }
     };
@@ -688,16 +744,24 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
         const uint32_t r_out = row0 + rb * 32 + l32;
         const uint32_t j = col0 + grp * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
         if (r_out < rows && j < batch) {
-            float *out = &dst[static_cast<uint64_t>(j) * stride_dst + r_out];
-            if constexpr (KSPLIT) unsafeAtomicAdd(out, value);   // two addends onto zero: order-independent
-            else *out = value;
+            const uint64_t idx = static_cast<uint64_t>(j) * stride_dst + r_out;
+            if constexpr (KSPLIT) unsafeAtomicAdd(static_cast<float *>(out.dst) + idx, value);   // two addends onto zero: order-independent
+            else if constexpr (SILU) static_cast<float *>(out.dst)[idx] = value;
+            else emit(out, idx, value);
         }
     };
     if constexpr (S == 1) {
+        if constexpr (SILU) {
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
+            for (int rb = 0; rb < RB / 2; ++rb)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) store(rb, v, acc[rb][v]);
+                for (int v = 0; v < 16; ++v) store(rb, v, silu_mul(acc[rb][v], acc[rb + RB / 2][v]));
+        } else {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) store(rb, v, acc[rb][v]);
+        }
     } else {
         // every load has landed and every wave is past its last read of the stages: reuse them
         float *part = reinterpret_cast<float *>(smem);
@@ -707,16 +771,18 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
             for (int v = 0; v < 16; ++v) part[((wave * RB + rb) * 16 + v) * kWave + lane] = acc[rb][v];
         __syncthreads();
         constexpr int kMine = 16 / S;   // outputs of each patch this wave finishes
+        auto total_of = [&](int rb, int v) {
+            auto p = [&](uint32_t s) { return part[(((s * CB + grp) * RB + rb) * 16 + v) * kWave + lane]; };
+            if constexpr (S == 2) return p(0) + p(1);
+            else return (p(0) + p(1)) + (p(2) + p(3));
+        };
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
+        for (int rb = 0; rb < (SILU ? RB / 2 : RB); ++rb)
 #pragma unroll
             for (int k = 0; k < kMine; ++k) {
                 const int v = share * kMine + k;
-                auto p = [&](uint32_t s) { return part[(((s * CB + grp) * RB + rb) * 16 + v) * kWave + lane]; };
-                float total;
-                if constexpr (S == 2) total = p(0) + p(1);
-                else total = (p(0) + p(1)) + (p(2) + p(3));
-                store(rb, v, total);
+                if constexpr (SILU) store(rb, v, silu_mul(total_of(rb, v), total_of(rb + RB / 2, v)));
+                else store(rb, v, total_of(rb, v));
             }
     }
 }
@@ -755,51 +821,122 @@ int launch_variant(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows
     return check_launch("gemm");
 }
 
-template <bool CHECK, int RB>
-int launch_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
-               uint32_t stride, hipStream_t stream) {
+// A last round of main tiles that fills at most half of the chip's slots (two workgroups per CU)
+// leaves the other CUs idle for most of a tile's time: those tiles are cut in two along K and both
+// halves add into a zeroed dst.  Measured on MI355X at M=2048: K=17408, N=5120 (640 tiles on 512
+// slots) and K=5120, N=17408 (2176 tiles).  Only on whole groups of eight row tiles (every
+// workgroup id is a tile then) and at least four super-blocks of K.  Returns the number of tiles
+// cut this way (0: none).  Only plain fp32 stores can be split: a sum that arrives in two halves
+// cannot be rounded to bf16 or added to a residual in an order that repeats.
+uint64_t split_round_tiles(uint32_t rows, uint32_t nb, uint32_t batch) {
+    const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
+    const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
+    if (row_tiles % 8 != 0 || nb / 4 < 4) return 0;
+    const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
+    const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
+    const uint64_t left = tiles % slots;
+    return (tiles >= slots && left != 0 && left * 2 <= slots) ? left : 0;
+}
+
+// A call of the tile kernels: one weight (or gate + up for the SwiGLU form) and what to do with the sums.
+struct TileCall {
+    const uint8_t *w;
+    const uint8_t *w2;   // the up weight of the SwiGLU form, else unused
+    const uint8_t *y;
+    TileOut out;
+};
+
+template <bool CHECK, int RB, bool SILU>
+int launch_dma(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, bool may_split, hipStream_t stream) {
     using T = DmaTile<RB>;
     static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
     if (!granted) {
         if (T::kLds > 64 * 1024 &&
-            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_dma_kernel<CHECK, RB>),
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_dma_kernel<CHECK, RB, SILU>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, T::kLds) != hipSuccess) {
             (void)hipGetLastError();
             return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", T::kLds);
         }
         granted = true;
     }
-    const uint32_t row_tiles = (rows + T::kRows - 1) / T::kRows;
+    constexpr uint32_t kOut = SILU ? T::kRows / 2 : T::kRows;
+    const uint32_t row_tiles = (rows + kOut - 1) / kOut;
     const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
     uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
     if (grid64 > 0x7ffffff0ull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
-    // A last round that fills at most half of the chip's slots (two workgroups per CU) leaves the
-    // other CUs idle for most of a tile's time: those tiles are cut in two along K and both halves
-    // add into a zeroed dst.  Measured on MI355X at M=2048: K=17408, N=5120 (640 tiles on 512 slots)
-    // and K=5120, N=17408 (2176 tiles).  Only main tiles on whole groups of eight row tiles (every
-    // id is a tile then) and at least four super-blocks of K.
     uint32_t split_from = 0xffffffffu;
-    if (RB == 4 && row_tiles % 8 == 0 && nb / 4 >= 4) {
-        const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
-        const uint64_t left = grid64 % slots;
-        if (grid64 >= slots && left != 0 && left * 2 <= slots) {
+    if (may_split) {
+        const uint64_t left = split_round_tiles(rows, nb, batch);
+        if (left != 0) {
             split_from = static_cast<uint32_t>(grid64 - left);
             gemm_zero_split_tiles_kernel<RB><<<static_cast<uint32_t>(left), kGemmThreads, 0, stream>>>(
-                dst, rows, batch, stride, row_tiles, col_tiles, split_from);
+                static_cast<float *>(c.out.dst), rows, batch, c.out.stride_dst, row_tiles, col_tiles, split_from);
             grid64 += left;
         }
     }
-    gemm_d4_dma_kernel<CHECK, RB><<<static_cast<uint32_t>(grid64), kGemmThreads, T::kLds, stream>>>(
-        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles, split_from);
+    gemm_d4_dma_kernel<CHECK, RB, SILU><<<static_cast<uint32_t>(grid64), kGemmThreads, T::kLds, stream>>>(
+        c.w, c.w2, c.y, c.out, rows, nb, batch, row_tiles, col_tiles, split_from);
     return check_launch("gemm");
 }
 
-template <int RB>
-int launch_dma_rows(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
-                    uint32_t stride, hipStream_t stream) {
-    const bool check = (rows % (32 * RB) != 0) || (batch % kTileCols != 0);
-    return check ? launch_dma<true, RB>(w, y, dst, rows, nb, batch, stride, stream)
-                 : launch_dma<false, RB>(w, y, dst, rows, nb, batch, stride, stream);
+template <bool SILU>
+int launch_dma_rows(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, bool may_split, hipStream_t stream) {
+    const bool check = (rows % (SILU ? 64u : 128u) != 0) || (batch % kTileCols != 0);
+    return check ? launch_dma<true, 4, SILU>(c, rows, nb, batch, may_split, stream)
+                 : launch_dma<false, 4, SILU>(c, rows, nb, batch, may_split, stream);
+}
+
+template <int CB, int W, int NS, bool KSPLIT, int RB, bool SILU>
+int launch_ring_inst(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, uint32_t row_tiles,
+                     uint32_t col_tiles, uint32_t grid, hipStream_t stream) {
+    using T = RingTile<CB, W, RB>;
+    constexpr int lds = NS * T::kStage;
+    static_assert(lds >= W * RB * 16 * kWave * 4, "the stages are reused for the partial sums of the waves");
+    static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
+    if (!granted) {
+        if (lds > 64 * 1024 &&
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS, KSPLIT, RB, SILU>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", lds);
+        }
+        granted = true;
+    }
+    gemm_d4_ring_kernel<CB, W, NS, KSPLIT, RB, SILU><<<grid, kWave * W, lds, stream>>>(
+        c.w, c.w2, c.y, c.out, rows, nb, batch, row_tiles, col_tiles);
+    return check_launch("gemm");
+}
+
+// With at most one tile per CU the launch lasts as long as one workgroup's chain of K steps
+// (a step is bound by its serial latency, not by bandwidth or arithmetic): two workgroups per
+// tile, one per half of K, halve that chain; they add into a dst zeroed by one more small
+// kernel.  Two addends onto zero, so results repeat bit for bit.  Only the narrowest tile
+// (up to 32 activation rows, four waves): measured on MI355X 19.2 -> 15.5 us at 5120 x 5120 and
+// 58.6 -> 44.6 us at K = 17408, batch 32; the wider tiles already split K over their waves
+// and gain nothing (64 rows) or lose (128 rows, sixteen waves: 29 -> 35 us).
+bool ring_splits_k(uint32_t rows, uint32_t nb, uint32_t batch) {
+    return batch <= 32 && static_cast<uint64_t>((rows + 31u) / 32u) <= static_cast<uint32_t>(device_cu_count()) &&
+           nb / 4 >= 8;
+}
+
+template <int CB, int W, int NS, int RB = 1, bool SILU = false>
+int launch_ring(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, hipStream_t stream) {
+    using T = RingTile<CB, W, RB>;
+    constexpr uint32_t kOut = SILU ? T::kRows / 2 : T::kRows;
+    const uint32_t row_tiles = (rows + kOut - 1) / kOut;
+    const uint32_t col_tiles = (batch + T::kCols - 1) / T::kCols;
+    const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
+    if (grid64 > 0x3fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    if constexpr (CB == 1 && RB == 1 && !SILU) {
+        if (c.out.epi == kEpiStore && ring_splits_k(rows, nb, batch)) {
+            gemm_zero_dst_kernel<<<dim3((rows + 1023u) / 1024u, batch), 256, 0, stream>>>(
+                static_cast<float *>(c.out.dst), rows, c.out.stride_dst);
+            return launch_ring_inst<CB, W, NS, true, RB, false>(c, rows, nb, batch, row_tiles, col_tiles,
+                                                                static_cast<uint32_t>(grid64 * 2), stream);
+        }
+    }
+    return launch_ring_inst<CB, W, NS, false, RB, SILU>(c, rows, nb, batch, row_tiles, col_tiles,
+                                                        static_cast<uint32_t>(grid64), stream);
 }
 
 // Tile choice.  Workgroups are scheduled dynamically and a lone workgroup on a CU runs nearly
@@ -807,75 +944,37 @@ int launch_dma_rows(const uint8_t *w, const uint8_t *y, float *dst, uint32_t row
 // little: problems with at least 0.4 main tiles per resident slot (two per CU) use main tiles
 // throughout (measured crossover on MI355X: between 160 and 256 main tiles); smaller ones use the
 // ring-staged 32-row tiles.
-template <int CB, int W, int NS, bool KSPLIT, int RB = 1>
-int launch_ring_inst(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
-                     uint32_t stride, uint32_t row_tiles, uint32_t col_tiles, uint32_t grid, hipStream_t stream) {
-    using T = RingTile<CB, W, RB>;
-    constexpr int lds = NS * T::kStage;
-    static_assert(lds >= W * RB * 16 * kWave * 4, "the stages are reused for the partial sums of the waves");
-    static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
-    if (!granted) {
-        if (lds > 64 * 1024 &&
-            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_kernel<CB, W, NS, KSPLIT, RB>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", lds);
-        }
-        granted = true;
-    }
-    gemm_d4_ring_kernel<CB, W, NS, KSPLIT, RB><<<grid, kWave * W, lds, stream>>>(
-        w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles);
-    return check_launch("gemm");
-}
-
-template <int CB, int W, int NS, int RB = 1>
-int launch_ring(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
-                uint32_t stride, hipStream_t stream) {
-    using T = RingTile<CB, W, RB>;
-    const uint32_t row_tiles = (rows + T::kRows - 1) / T::kRows;
-    const uint32_t col_tiles = (batch + T::kCols - 1) / T::kCols;
-    const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
-    if (grid64 > 0x3fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
-    // With at most one tile per CU the launch lasts as long as one workgroup's chain of K steps
-    // (a step is bound by its serial latency, not by bandwidth or arithmetic): two workgroups per
-    // tile, one per half of K, halve that chain; they add into a dst zeroed by one more small
-    // kernel.  Two addends onto zero, so results repeat bit for bit.  Only the narrowest tile
-    // (up to 32 activation rows, four waves): measured on MI355X 19.2 -> 15.5 us at 5120 x 5120 and
-    // 58.6 -> 44.6 us at K = 17408, batch 32; the wider tiles already split K over their waves
-    // and gain nothing (64 rows) or lose (128 rows, sixteen waves: 29 -> 35 us).
-    if constexpr (CB == 1 && RB == 1) {
-        if (static_cast<uint64_t>(row_tiles) * col_tiles <= static_cast<uint32_t>(device_cu_count()) &&
-            nb / 4 >= 8 && batch <= 65535u) {
-            gemm_zero_dst_kernel<<<dim3((rows + 1023u) / 1024u, batch), 256, 0, stream>>>(dst, rows, stride);
-            return launch_ring_inst<CB, W, NS, true>(w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles,
-                                                     static_cast<uint32_t>(grid64 * 2), stream);
-        }
-    }
-    return launch_ring_inst<CB, W, NS, false, RB>(w, y, dst, rows, nb, batch, stride, row_tiles, col_tiles,
-                                                  static_cast<uint32_t>(grid64), stream);
-}
-
-int launch_gemm_dma(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, uint32_t nb, uint32_t batch,
-                    uint32_t stride, hipStream_t stream) {
+bool uses_main_tiles(uint32_t rows, uint32_t batch) {
     const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
-    const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
-    const uint32_t col_tiles = (batch + kTileCols - 1) / kTileCols;
-    const uint64_t tiles = static_cast<uint64_t>(row_tiles) * col_tiles;
-    if (tiles * 5 >= slots * 2) return launch_dma_rows<4>(w, y, dst, rows, nb, batch, stride, stream);
+    const uint64_t tiles = static_cast<uint64_t>((rows + kTileRows - 1) / kTileRows) * ((batch + kTileCols - 1) / kTileCols);
+    return tiles * 5 >= slots * 2;
+}
+
+int launch_gemm_dma(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, hipStream_t stream) {
+    if (uses_main_tiles(rows, batch)) return launch_dma_rows<false>(c, rows, nb, batch, c.out.epi == kEpiStore, stream);
     // too few main tiles to fill the chip: 32-row tiles behind a ring of stages, as wide as the batch needs
     // Batches of 33..64 rows on matrices tall enough for more than 1.5 32-row tiles per CU take 64-row
     // tiles: half as many workgroups re-read the activation records of a step (measured at
     // 17408 x 5120, batch 64: 59 -> 51 us).  The 32- and 128-row-wide tiles lose with 64 rows (54
     // against 43 us, 88 against 77 us): their rings then leave room for one workgroup per CU only.
     if (batch > 32 && batch <= 64 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * static_cast<uint32_t>(device_cu_count()))
-        return launch_ring<2, kRingWaves2, kRing2, 2>(w, y, dst, rows, nb, batch, stride, stream);
-    if (batch <= 32) return launch_ring<1, 4, kRing1>(w, y, dst, rows, nb, batch, stride, stream);
-    if (batch <= 64) return launch_ring<2, kRingWaves2, kRing2>(w, y, dst, rows, nb, batch, stride, stream);
+        return launch_ring<2, kRingWaves2, kRing2, 2>(c, rows, nb, batch, stream);
+    if (batch <= 32) return launch_ring<1, 4, kRing1>(c, rows, nb, batch, stream);
+    if (batch <= 64) return launch_ring<2, kRingWaves2, kRing2>(c, rows, nb, batch, stream);
     // at most one tile per CU: sixteen waves (four K shares per group) instead of eight
     const uint64_t ring_tiles = static_cast<uint64_t>((rows + 31u) / 32u) * ((batch + 127u) / 128u);
     if (ring_tiles <= static_cast<uint32_t>(device_cu_count()))
-        return launch_ring<4, 16, kRing4>(w, y, dst, rows, nb, batch, stride, stream);
-    return launch_ring<4, kRingWaves4, kRing4>(w, y, dst, rows, nb, batch, stride, stream);
+        return launch_ring<4, 16, kRing4>(c, rows, nb, batch, stream);
+    return launch_ring<4, kRingWaves4, kRing4>(c, rows, nb, batch, stream);
+}
+
+// SwiGLU form: gate and up rows side by side in every tile.  Main tiles (64 gate + 64 up rows) when
+// the two GEMMs it replaces would use main tiles, else 64-row ring tiles (32 + 32).
+int launch_gemm_silu(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, hipStream_t stream) {
+    if (uses_main_tiles(2 * rows, batch)) return launch_dma_rows<true>(c, rows, nb, batch, false, stream);
+    if (batch <= 32) return launch_ring<1, 4, kRing1, 2, true>(c, rows, nb, batch, stream);
+    if (batch <= 64) return launch_ring<2, kRingWaves2, kRing2, 2, true>(c, rows, nb, batch, stream);
+    return launch_ring<4, kRingWaves4, kRing4, 2, true>(c, rows, nb, batch, stream);
 }
 
 int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, uint32_t cols,
@@ -883,7 +982,7 @@ int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, u
     // small batches: the weight-streaming matrix-core GEMV, which reads the weights at HBM speed
     // instead of padding the batch to a 32-wide tile (it declines what the ring tiles serve better)
     if (batch <= 16 && (cols / kQK) % 8 == 0) {
-        const int rc = gemv_mfma_d4(w, y, dst, rows, cols, batch, stride, stream);
+        const int rc = gemv_mfma_d4(w, nullptr, y, dst, rows, cols, batch, stride, false, stream);
         if (rc != Q8MI_REJECTED) return rc;
     }
     const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
@@ -896,9 +995,19 @@ int launch_gemm_d4(const uint8_t *w, const void *y, float *dst, uint32_t rows, u
     const uint32_t nb = cols / kQK;
     const bool a16 = nb % 8 == 0;
     const auto *yb = static_cast<const uint8_t *>(y);
-    if (a16) return launch_gemm_dma(w, yb, dst, rows, nb, batch, stride, stream);
+    if (a16) return launch_gemm_dma(TileCall{w, nullptr, yb, TileOut{dst, nullptr, stride, kEpiStore}}, rows, nb, batch, stream);
     return check ? launch_variant<true, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream)
                  : launch_variant<false, false>(w, yb, dst, rows, nb, batch, stride, row_tiles, col_tiles, grid, stream);
+}
+
+// The shapes the fused-epilogue entry points serve: D4 activations on the direct-to-LDS tiles.
+int fused_gate(const char *what, const void *weight, uint32_t rows, uint32_t cols, uint32_t batch) {
+    if (cols == 0 || cols % 128 != 0) return fail(Q8MI_REJECTED, "%s: cols %u not a multiple of 128", what, cols);
+    if (batch == 0 || rows == 0) return fail(Q8MI_REJECTED, "%s: empty shape", what);
+    if (rows < 128) return fail(Q8MI_REJECTED, "%s: %u rows (fewer than 128: the activations would be Q8_1)", what, rows);
+    if ((cols / kQK) % 8 != 0) return fail(Q8MI_REJECTED, "%s: cols %u not a multiple of 256", what, cols);
+    if (reinterpret_cast<uintptr_t>(weight) % 16 != 0) return fail(Q8MI_REJECTED, "%s: weight pointer not 16-byte aligned", what);
+    return Q8MI_OK;
 }
 
 }  // namespace
@@ -928,4 +1037,58 @@ extern "C" int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *
     if (reinterpret_cast<uintptr_t>(weight) % 16 != 0)
         return fail(Q8MI_REJECTED, "gemm_medium: weight pointer not 16-byte aligned");
     return launch_gemm_d4(weight, y_d4, dst, rows, cols, batch, stride_dst_row, as_stream(stream));
+}
+
+// Shapes whose plain GEMM cuts its last round of main tiles in two along K keep that route (the
+// caller runs q8mi_gemm and the second step): there it is the faster one.
+static bool plain_gemm_splits(uint32_t rows, uint32_t cols, uint32_t batch) {
+    return uses_main_tiles(rows, batch) && split_round_tiles(rows, cols / kQK, batch) != 0;
+}
+
+extern "C" int q8mi_gemm_add(const uint8_t *weight, const void *y_d4, const float *residual, float *dst, uint32_t rows,
+                             uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream) {
+    if (int rc = fused_gate("gemm_add", weight, rows, cols, batch)) return rc;
+    if (residual == nullptr || dst == nullptr) return fail(Q8MI_REJECTED, "gemm_add: null pointer");
+    if (batch <= 16) {   // a weight stream: the matrix-core GEMV adds in place
+        if (residual != dst) return fail(Q8MI_REJECTED, "gemm_add: batch %u is served in place only", batch);
+        const int rc = gemv_mfma_d4(weight, nullptr, y_d4, dst, rows, cols, batch, stride_dst_row, true, as_stream(stream));
+        if (rc != Q8MI_REJECTED) return rc;
+    }
+    if (batch <= 32 && ring_splits_k(rows, cols / kQK, batch))
+        return fail(Q8MI_REJECTED, "gemm_add: this shape is summed from two halves of K (use q8mi_gemm, then q8mi_add)");
+    if (plain_gemm_splits(rows, cols, batch))
+        return fail(Q8MI_REJECTED, "gemm_add: the last round of this shape is summed from two halves of K (use q8mi_gemm, then q8mi_add)");
+    return launch_gemm_dma(TileCall{weight, nullptr, static_cast<const uint8_t *>(y_d4),
+                                    TileOut{dst, residual, stride_dst_row, kEpiAdd}},
+                           rows, cols / kQK, batch, as_stream(stream));
+}
+
+extern "C" int q8mi_gemm_bf16(const uint8_t *weight, const void *y_d4, uint16_t *dst, uint32_t rows, uint32_t cols,
+                              uint32_t batch, uint32_t stride_dst_row, void *stream) {
+    if (int rc = fused_gate("gemm_bf16", weight, rows, cols, batch)) return rc;
+    if (dst == nullptr) return fail(Q8MI_REJECTED, "gemm_bf16: null pointer");
+    if (batch <= 16) return fail(Q8MI_REJECTED, "gemm_bf16: batch %u is a weight stream (use the GEMV family)", batch);
+    if (batch <= 32 && ring_splits_k(rows, cols / kQK, batch))
+        return fail(Q8MI_REJECTED, "gemm_bf16: this shape is summed from two halves of K (use q8mi_gemm, then q8mi_f32_to_bf16)");
+    if (plain_gemm_splits(rows, cols, batch))
+        return fail(Q8MI_REJECTED, "gemm_bf16: the last round of this shape is summed from two halves of K (use q8mi_gemm, then q8mi_f32_to_bf16)");
+    return launch_gemm_dma(TileCall{weight, nullptr, static_cast<const uint8_t *>(y_d4),
+                                    TileOut{dst, nullptr, stride_dst_row, kEpiStoreBf16}},
+                           rows, cols / kQK, batch, as_stream(stream));
+}
+
+extern "C" int q8mi_gemm_silu_mul(const uint8_t *weight_gate, const uint8_t *weight_up, const void *y_d4, float *dst,
+                                  uint32_t rows, uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream) {
+    if (int rc = fused_gate("gemm_silu_mul", weight_gate, rows, cols, batch)) return rc;
+    if (reinterpret_cast<uintptr_t>(weight_up) % 16 != 0 || weight_up == nullptr)
+        return fail(Q8MI_REJECTED, "gemm_silu_mul: up weight pointer null or not 16-byte aligned");
+    if (dst == nullptr) return fail(Q8MI_REJECTED, "gemm_silu_mul: null pointer");
+    if (batch <= 16) {
+        const int rc = gemv_mfma_d4(weight_gate, weight_up, y_d4, dst, rows, cols, batch, stride_dst_row, false,
+                                    as_stream(stream));
+        if (rc != Q8MI_REJECTED) return rc;
+    }
+    return launch_gemm_silu(TileCall{weight_gate, weight_up, static_cast<const uint8_t *>(y_d4),
+                                     TileOut{dst, nullptr, stride_dst_row, kEpiStore}},
+                            rows, cols / kQK, batch, as_stream(stream));
 }

@@ -440,10 +440,11 @@ int run_single(const char *what, int mode, const uint8_t *w, const XSource &y, v
 // passes of the short slices (measured against the 32-row ring tiles of the GEMM: 14.7..17.2 us
 // against 19 us at 5120 x 5120 and 9..16 rows, but 26..32 us in two passes at 17..32 rows;
 // 49 against 58 us at 5120 x 17408 and 8 rows).  Q8MI_REJECTED otherwise (the caller then uses
-// tiles).
-int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, uint32_t cols, uint32_t batch,
-                 uint32_t stride_dst_row, hipStream_t stream) {
+// tiles).  w_up: the SwiGLU form (dst = silu(w x) * (w_up x)); add: dst += w x.
+int gemv_mfma_d4(const uint8_t *w, const uint8_t *w_up, const void *y_d4, float *dst, uint32_t rows, uint32_t cols,
+                 uint32_t batch, uint32_t stride_dst_row, bool add, hipStream_t stream) {
     const uint32_t nb = cols / kQK;
+    const bool silu = w_up != nullptr;
     if (nb % 8 != 0 || batch == 0) return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): cols %u not served", cols);
     // D4 scales are fp32 values: only the fp32 scale table keeps them exact
     uint32_t fit = 0;
@@ -455,19 +456,30 @@ int gemv_mfma_d4(const uint8_t *w, const void *y_d4, float *dst, uint32_t rows, 
     // ... unless the GEMM's 32-row tiles come at most one per CU: those are then cut in two along K
     // (launch_ring) and beat two passes (measured at 17408 columns and 5..8 rows: 43 against 46..48 us
     // on 5120 weight rows, 49 against 65..67 us on 8192)
-    if (batch > fit && (rows + 31u) / 32u <= static_cast<uint32_t>(device_cu_count()) && nb / 4 >= 8)
+    if (batch > fit && !silu && !add && (rows + 31u) / 32u <= static_cast<uint32_t>(device_cu_count()) && nb / 4 >= 8)
         return fail(Q8MI_REJECTED, "gemv (matrix-core, D4): batch %u at %u columns is served by split tiles", batch, cols);
     const auto *y = static_cast<const uint8_t *>(y_d4);
     for (uint32_t j0 = 0; j0 < batch; j0 += fit) {
         const uint32_t m = batch - j0 < fit ? batch - j0 : fit;
         GemvParams p = single(w, XSource{y + static_cast<uint64_t>(j0) * kD4Bytes, nullptr, batch},
-                              dst + static_cast<uint64_t>(j0) * stride_dst_row, rows, cols, stride_dst_row, kStoreF32);
+                              dst + static_cast<uint64_t>(j0) * stride_dst_row, rows, cols, stride_dst_row,
+                              silu ? kSiluMul : add ? kAddF32 : kStoreF32);
+        p.w[1] = silu ? w_up : p.w[1];
         int rc;
-        switch ((m + 3) / 4) {
-            case 1: rc = launch_mfma<1, false, false, true>(p, m, stream); break;
-            case 2: rc = launch_mfma<2, false, false, true>(p, m, stream); break;
-            case 3: rc = launch_mfma<3, false, false, true>(p, m, stream); break;
-            default: rc = launch_mfma<4, false, false, true>(p, m, stream); break;
+        if (silu) {
+            switch ((m + 3) / 4) {
+                case 1: rc = launch_mfma<1, true, false, true>(p, m, stream); break;
+                case 2: rc = launch_mfma<2, true, false, true>(p, m, stream); break;
+                case 3: rc = launch_mfma<3, true, false, true>(p, m, stream); break;
+                default: rc = launch_mfma<4, true, false, true>(p, m, stream); break;
+            }
+        } else {
+            switch ((m + 3) / 4) {
+                case 1: rc = launch_mfma<1, false, false, true>(p, m, stream); break;
+                case 2: rc = launch_mfma<2, false, false, true>(p, m, stream); break;
+                case 3: rc = launch_mfma<3, false, false, true>(p, m, stream); break;
+                default: rc = launch_mfma<4, false, false, true>(p, m, stream); break;
+            }
         }
         if (rc != Q8MI_OK) return rc;
     }

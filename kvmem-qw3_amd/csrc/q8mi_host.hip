@@ -108,6 +108,20 @@ __global__ __launch_bounds__(256) void add_kernel(void *__restrict__ out_v, cons
     }
 }
 
+// ---- elementwise SwiGLU: out = silu(gate) * up, silu(g) = g / (1 + exp(-g)) --------------------
+// Four elements per thread when the three pointers are 16-byte aligned.
+__global__ __launch_bounds__(256) void silu_mul_kernel(float *out, const float *gate, const float *up, uint64_t n, bool vec) {
+    const uint64_t i0 = (static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+    if (i0 >= n) return;
+    auto f = [](float g, float u) { return (g / (1.0f + __expf(-g))) * u; };
+    if (vec && i0 + 4 <= n) {
+        const float4 g = *reinterpret_cast<const float4 *>(gate + i0), u = *reinterpret_cast<const float4 *>(up + i0);
+        *reinterpret_cast<float4 *>(out + i0) = make_float4(f(g.x, u.x), f(g.y, u.y), f(g.z, u.z), f(g.w, u.w));
+    } else {
+        for (uint64_t i = i0; i < n && i < i0 + 4; ++i) out[i] = f(gate[i], up[i]);
+    }
+}
+
 }  // namespace
 }  // namespace q8mi
 
@@ -169,4 +183,14 @@ extern "C" int q8mi_add(void *out, const void *a, const void *b, uint64_t n, int
     else
         add_kernel<false><<<static_cast<uint32_t>(grid), 256, 0, as_stream(stream)>>>(out, a, b, n, vec);
     return check_launch("add");
+}
+
+extern "C" int q8mi_silu_mul(float *out, const float *gate, const float *up, uint64_t n, void *stream) {
+    if (n == 0) return Q8MI_OK;
+    if (out == nullptr || gate == nullptr || up == nullptr) return fail(Q8MI_REJECTED, "silu_mul: null pointer");
+    const uint64_t grid = ((n + 3) / 4 + 255) / 256;
+    if (grid > 0x7fffffffull) return fail(Q8MI_REJECTED, "silu_mul: too many elements for one launch");
+    const bool vec = (reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up)) % 16 == 0;
+    silu_mul_kernel<<<static_cast<uint32_t>(grid), 256, 0, as_stream(stream)>>>(out, gate, up, n, vec);
+    return check_launch("silu_mul");
 }

@@ -19,6 +19,14 @@
 //   * strided batch > 8 (in_stride != cols or out_stride != rows), which the
 //     reference serves with a legacy kernel outside this path, runs as GEMV
 //     slices of eight rows.
+//   * q8_0_matmul_silu_mul is served for Q8_0 (the reference declines it and the executor
+//     falls back to two matmuls and silu_mul_n); q8_0_matmul_add above eight rows and bf16
+//     outputs of q8_0_matmul take the tile kernel's fused store where it has one.
+//   * a norm and the projections that read its output share work: rms_norm / rms_norm_batch of
+//     up to eight rows also leave the rows' Q8_1 blocks in the scratch, and the operator called
+//     next reads them instead of quantizing again; a one-row rms_norm is held back one call and
+//     runs inside the GEMV when that call is a batch-1 projection of its output (PendingNorm
+//     in the header).  Same bits either way.
 #include "hip_q8_backend.hpp"
 
 #include <cstdio>
@@ -101,11 +109,15 @@ HipQ8Backend::~HipQ8Backend() {
 
 DeviceStatus HipQ8Backend::end() { return synchronize(); }
 
-DeviceStatus HipQ8Backend::synchronize() { return hip_status(hipStreamSynchronize(stream_), "hip synchronize"); }
+DeviceStatus HipQ8Backend::synchronize() {
+    if (auto st = flush_norm(); !st.ok) return st;
+    return hip_status(hipStreamSynchronize(stream_), "hip synchronize");
+}
 
 // ---- graph capture (src/kernels_cuda.cu:9958-9980) -------------------------------
 bool HipQ8Backend::begin_capture() {
     if (capturing_) return false;
+    if (!flush_norm().ok) return false;   // a norm from before the capture runs before it
     if (hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal) != hipSuccess) {
         (void)hipGetLastError();
         return false;
@@ -116,10 +128,12 @@ bool HipQ8Backend::begin_capture() {
 
 DeviceStatus HipQ8Backend::end_capture() {
     if (!capturing_) return {false, "end_capture without begin_capture"};
+    const DeviceStatus flushed = flush_norm();   // a norm still held back belongs to the graph
     capturing_ = false;
     if (graph_exec_) { (void)hipGraphExecDestroy(graph_exec_); graph_exec_ = nullptr; }
     if (graph_) { (void)hipGraphDestroy(graph_); graph_ = nullptr; }
     if (auto st = hip_status(hipStreamEndCapture(stream_, &graph_), "hip end capture"); !st.ok) return st;
+    if (!flushed.ok) return flushed;
     return hip_status(hipGraphInstantiate(&graph_exec_, graph_, nullptr, nullptr, 0), "hip graph instantiate");
 }
 
@@ -129,11 +143,14 @@ DeviceStatus HipQ8Backend::replay_graph() {
 }
 
 // ---- tensors / weights -------------------------------------------------------------
+// (A new tensor may reuse the address of a freed one: whatever the scratch holds for that address is stale.)
 std::unique_ptr<DeviceTensor> HipQ8Backend::tensor_f32(uint64_t count, const char *) {
+    forget_quantized();
     return make_tensor(count, 4, DeviceTensorDType::F32);
 }
 
 std::unique_ptr<DeviceTensor> HipQ8Backend::tensor_bf16(uint64_t count, const char *) {
+    forget_quantized();
     return make_tensor(count, 2, DeviceTensorDType::BF16);
 }
 
@@ -174,6 +191,8 @@ DeviceStatus HipQ8Backend::copy_bytes_from_host(DeviceTensor &x, uint64_t byte_o
                                                 uint64_t bytes) {
     auto &t = T(x);
     if (byte_offset + bytes > t.count * t.elem_size) return {false, "copy_bytes_from_host out of range"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    forget_quantized();
     if (auto st = hip_status(hipMemcpyAsync(static_cast<uint8_t *>(t.ptr) + byte_offset, host, bytes,
                                             hipMemcpyHostToDevice, stream_), "copy_bytes_from_host"); !st.ok)
         return st;
@@ -184,6 +203,7 @@ DeviceStatus HipQ8Backend::copy_bytes_to_host(const DeviceTensor &x, void *host,
                                               uint64_t bytes) {
     const auto &t = T(x);
     if (byte_offset + bytes > t.count * t.elem_size) return {false, "copy_bytes_to_host out of range"};
+    if (auto st = flush_norm(); !st.ok) return st;
     if (auto st = hip_status(hipMemcpyAsync(host, static_cast<const uint8_t *>(t.ptr) + byte_offset, bytes,
                                             hipMemcpyDeviceToHost, stream_), "copy_bytes_to_host"); !st.ok)
         return st;
@@ -199,6 +219,8 @@ DeviceStatus HipQ8Backend::zero_tensor(DeviceTensor &x) {
     auto &t = T(x);
     // memset nodes are kept out of captured graphs
     if (capturing_) return {false, "zero_tensor is not available during graph capture"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    forget_quantized();
     return hip_status(hipMemsetAsync(t.ptr, 0, t.count * t.elem_size, stream_), "zero_tensor");
 }
 
@@ -207,6 +229,7 @@ DeviceStatus HipQ8Backend::zero_tensor(DeviceTensor &x) {
 DeviceStatus HipQ8Backend::ensure(Scratch &s, size_t need, const char *what) {
     if (need <= s.capacity) return {};
     if (capturing_) return {false, "scratch would grow during graph capture: run the op eagerly once first"};
+    if (&s == &q8_1_) forget_quantized();
     if (s.ptr) {
         (void)hipStreamSynchronize(stream_);
         (void)hipFree(s.ptr);
@@ -226,19 +249,49 @@ DeviceStatus HipQ8Backend::failed(const char *where) {
     return {false, g_msg};
 }
 
+// The Q8_1 blocks of `batch` rows at x, in the scratch: quantized now, unless the norm that wrote
+// those rows has left them there already.
 DeviceStatus HipQ8Backend::quantize_q8_1(const float *x, uint32_t batch, uint32_t cols, uint32_t stride) {
+    if (quantized_.src == x && quantized_.batch == batch && quantized_.cols == cols && quantized_.stride == stride)
+        return {};
+    forget_quantized();
     if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(batch, cols), "q8_1 scratch alloc"); !st.ok) return st;
     if (!ported::launch_quantize_q8_1(x, q8_1_.ptr, batch, cols, stride, stream_))
         return failed("quantize_q8_1");
     return {};
 }
 
+// Runs the norm that rms_norm_batch held back, with the quantizer in the same pass.
+DeviceStatus HipQ8Backend::flush_norm() {
+    if (!pending_.active) return {};
+    const PendingNorm n = pending_;
+    pending_.active = false;
+    forget_quantized();
+    if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(1, n.cols), "q8_1 scratch alloc"); !st.ok) return st;
+    if (q8mi_rms_norm_quantize_q8_1(n.x, n.weight, n.out, q8_1_.ptr, 1, n.cols, n.cols, n.cols, n.eps, stream_) != Q8MI_OK)
+        return failed("rms_norm_quantize_q8_1");
+    quantized_ = QuantizedRows{n.out, 1, n.cols, n.cols};
+    return launch_status("hip rms_norm");
+}
+
+// Whether a batch-1 projection of x (cols floats) whose first output is out0 can run the held-back
+// norm inside its own launch: x is that norm's output, and the launch writes neither the norm's
+// input (every workgroup reads it) nor its output (workgroup 0 writes it).
+bool HipQ8Backend::absorbs_norm(const float *x, uint32_t cols, const void *out0) const {
+    return pending_.active && x == pending_.out && cols == pending_.cols && out0 != pending_.x && out0 != pending_.out;
+}
+
 // Batch 1 on rows of up to 8192 columns: one launch that quantizes the activations inside the GEMV
 // (measured on MI355X: 10.2 against 3.3 + 9.3 us for the QKV fan-out, 9.3 against 3.3 + 7.8 us for the O
 // projection).  Longer rows (the down projection's 17408 columns) and batches above 1 are faster
 // with the stand-alone quantizer in front (3.5 + 18.0 against 23.7 us).  The fused entry point may
-// still decline a shape; the two-step form below then runs.
-static bool fuse_quantizer(uint32_t batch, uint32_t cols) { return batch == 1 && cols % 256 == 0 && cols <= 8192; }
+// still decline a shape; the two-step form below then runs.  Rows whose Q8_1 blocks a norm has
+// already left in the scratch take the two-step form without its first step.
+bool HipQ8Backend::fuse_quantizer(const float *x, uint32_t batch, uint32_t cols, uint32_t stride) const {
+    if (quantized_.src == x && quantized_.batch == batch && quantized_.cols == cols && quantized_.stride == stride)
+        return false;
+    return batch == 1 && cols % 256 == 0 && cols <= 8192;
+}
 
 // dispatch_q8_matvec, src/kernels_cuda.cu:14617-14658: any batch as GEMV slices of <= 8 rows
 DeviceStatus HipQ8Backend::gemv_route(float *out, const DeviceWeight &weight, const float *x, uint32_t batch,
@@ -247,7 +300,7 @@ DeviceStatus HipQ8Backend::gemv_route(float *out, const DeviceWeight &weight, co
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
     const uint32_t xs = (batch == 1 && in_stride == 0) ? cols : in_stride;
     const uint32_t os = (batch == 1 && out_stride == 0) ? rows : out_stride;
-    if (fuse_quantizer(batch, cols) &&
+    if (fuse_quantizer(x, batch, cols, xs) &&
         q8mi_qgemv(w.ptr, x, xs, out, 0, rows, cols, 1, os, stream_) == Q8MI_OK)
         return launch_status("hip q8_0_matvec fused");
     for (uint32_t j0 = 0; j0 < batch; j0 += 8) {
@@ -260,6 +313,13 @@ DeviceStatus HipQ8Backend::gemv_route(float *out, const DeviceWeight &weight, co
     return launch_status("hip q8_0_matvec");
 }
 
+// D4 records of `batch` rows of x in the scratch (src/kernels_cuda.cu:14493-14507)
+DeviceStatus HipQ8Backend::quantize_d4(const float *x, uint32_t batch, uint32_t cols, uint32_t stride) {
+    if (auto st = ensure(d4_, ported::q8_1_mmq_scratch_bytes(batch, cols), "q8_1_mmq scratch alloc"); !st.ok) return st;
+    if (!ported::launch_quantize_mmq_q8_1(x, d4_.ptr, batch, cols, stride, stream_)) return failed("quantize_mmq_q8_1");
+    return {};
+}
+
 // ---- decode-side ops --------------------------------------------------------------------
 // src/kernels_cuda.cu:10764-10888
 DeviceStatus HipQ8Backend::q8_0_matvec(DeviceTensor &out, const DeviceWeight &weight, const DeviceTensor &x) {
@@ -267,16 +327,29 @@ DeviceStatus HipQ8Backend::q8_0_matvec(DeviceTensor &out, const DeviceWeight &we
     auto &o = T(out);
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "q8_0_matvec: weight is not Q8_0"};
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
+    const float *xin = T(x).f32();
+    if (absorbs_norm(xin, cols, o.ptr)) {   // norm, quantizer and GEMV in one launch
+        const int rc = q8mi_nqgemv(w.ptr, pending_.x, pending_.weight, pending_.eps, pending_.out, o.ptr,
+                                   o.is_bf16() ? 1 : 0, rows, cols, 1, stream_);
+        if (rc == Q8MI_OK) {
+            pending_.active = false;
+            wrote(o.ptr);
+            return launch_status("hip rms_norm + q8_0_matvec");
+        }
+        if (rc != Q8MI_REJECTED) return failed("nqgemv");
+    }
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
     if (o.is_bf16()) {
-        if (fuse_quantizer(1, cols) &&
-            q8mi_qgemv(w.ptr, T(x).f32(), cols, o.bf16(), 1, rows, cols, 1, rows, stream_) == Q8MI_OK)
+        if (fuse_quantizer(xin, 1, cols, cols) &&
+            q8mi_qgemv(w.ptr, xin, cols, o.bf16(), 1, rows, cols, 1, rows, stream_) == Q8MI_OK)
             return launch_status("hip q8_0_matvec bf16 fused");
-        if (auto st = quantize_q8_1(T(x).f32(), 1, cols, cols); !st.ok) return st;
+        if (auto st = quantize_q8_1(xin, 1, cols, cols); !st.ok) return st;
         if (!ported::launch_mmvq_q8_0_bf16(w.ptr, q8_1_.ptr, o.bf16(), rows, cols, 1, rows, stream_))
             return failed("mmvq_q8_0_bf16");
         return launch_status("hip q8_0_matvec bf16");
     }
-    return gemv_route(o.f32(), weight, T(x).f32(), 1, 0, 0);
+    return gemv_route(o.f32(), weight, xin, 1, 0, 0);
 }
 
 // src/kernels_cuda.cu:12035-12069
@@ -284,11 +357,14 @@ DeviceStatus HipQ8Backend::q8_0_matvec_add(DeviceTensor &accum, const DeviceWeig
     const auto &w = W(weight);
     auto &o = T(accum);
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "q8_0_matvec_add: weight is not Q8_0"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
-    if (fuse_quantizer(1, cols) &&
-        q8mi_qgemv_add(w.ptr, T(x).f32(), cols, o.ptr, o.is_bf16() ? 1 : 0, rows, cols, 1, rows, stream_) == Q8MI_OK)
+    const float *xin = T(x).f32();
+    if (fuse_quantizer(xin, 1, cols, cols) &&
+        q8mi_qgemv_add(w.ptr, xin, cols, o.ptr, o.is_bf16() ? 1 : 0, rows, cols, 1, rows, stream_) == Q8MI_OK)
         return launch_status("hip q8_0_matvec_add fused");
-    if (auto st = quantize_q8_1(T(x).f32(), 1, cols, cols); !st.ok) return st;
+    if (auto st = quantize_q8_1(xin, 1, cols, cols); !st.ok) return st;
     const bool ok = o.is_bf16()
         ? ported::launch_mmvq_q8_0_add_bf16(w.ptr, q8_1_.ptr, o.bf16(), rows, cols, 1, rows, stream_)
         : ported::launch_mmvq_q8_0_add(w.ptr, q8_1_.ptr, o.f32(), rows, cols, 1, rows, stream_);
@@ -299,19 +375,9 @@ DeviceStatus HipQ8Backend::q8_0_matvec_add(DeviceTensor &accum, const DeviceWeig
 // src/kernels_cuda.cu:12227-12258
 DeviceStatus HipQ8Backend::q8_0_matvec_silu_mul(DeviceTensor &out, const DeviceWeight &weight_gate,
                                                 const DeviceWeight &weight_up, const DeviceTensor &x) {
-    const auto &g = W(weight_gate), &u = W(weight_up);
-    if (g.format != DeviceWeightFormat::Q8_0 || u.format != DeviceWeightFormat::Q8_0)
-        return {false, "q8_0_matvec_silu_mul: weights are not Q8_0"};
-    if (g.rows != u.rows || g.cols != u.cols) return {false, "q8_0_matvec_silu_mul: gate/up shapes differ"};
-    if (T(out).is_bf16()) return {false, "q8_0_matvec_silu_mul: bf16 output not supported"};
-    const uint32_t cols = static_cast<uint32_t>(g.cols), rows = static_cast<uint32_t>(g.rows);
-    if (fuse_quantizer(1, cols) &&
-        q8mi_qgemv_silu_mul(g.ptr, u.ptr, T(x).f32(), cols, T(out).f32(), rows, cols, 1, rows, stream_) == Q8MI_OK)
-        return launch_status("hip q8_0_matvec_silu_mul fused");
-    if (auto st = quantize_q8_1(T(x).f32(), 1, cols, cols); !st.ok) return st;
-    if (!ported::launch_mmvq_q8_0_silu_mul(g.ptr, u.ptr, q8_1_.ptr, T(out).f32(), rows, cols, 1, rows, stream_))
-        return failed("mmvq_q8_0_silu_mul");
-    return launch_status("hip q8_0_matvec_silu_mul");
+    const auto &g = W(weight_gate);
+    return q8_0_matmul_silu_mul(out, weight_gate, weight_up, x, 1, static_cast<uint32_t>(g.cols),
+                                static_cast<uint32_t>(g.rows));
 }
 
 // src/kernels_cuda.cu:11244-11302: quantize once, then as few launches as possible
@@ -330,8 +396,22 @@ DeviceStatus HipQ8Backend::q8_0_matmul(DeviceTensor &out, const DeviceWeight &we
     auto &o = T(out);
     if (batch == 0) return {};
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "q8_0_matmul: weight is not Q8_0"};
+    if (batch == 1 && (in_stride == 0 || in_stride == w.cols) && (out_stride == 0 || out_stride == w.rows))
+        return q8_0_matvec(out, weight, x);
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
     const uint64_t out_count = static_cast<uint64_t>(batch) * (out_stride ? out_stride : rows);
+    const float *xin = T(x).f32();
+    const bool contiguous = in_stride == cols && out_stride == rows;
+    const bool tiles = batch > 8 && contiguous && cols % 32 == 0;
+    const bool d4 = rows >= 128 && cols % 128 == 0;   // layout rule of src/kernels_cuda.cu:14545-14552
+    if (tiles && d4 && o.is_bf16()) {   // the tile kernel rounds to bf16 in its store where it can
+        if (auto st = quantize_d4(xin, batch, cols, cols); !st.ok) return st;
+        const int rc = q8mi_gemm_bf16(w.ptr, d4_.ptr, o.bf16(), rows, cols, batch, rows, stream_);
+        if (rc == Q8MI_OK) return launch_status("hip q8_0_matmul mmq bf16");
+        if (rc != Q8MI_REJECTED) return failed("gemm_bf16");
+    }
     float *dst = o.f32();
     if (o.is_bf16()) {   // compute in fp32, convert at the end (src/kernels_cuda.cu:14509-14530)
         if (auto st = ensure(out_f32_, out_count * 4, "q8 fp32 output workspace"); !st.ok) return st;
@@ -342,15 +422,11 @@ DeviceStatus HipQ8Backend::q8_0_matmul(DeviceTensor &out, const DeviceWeight &we
         if (q8mi_f32_to_bf16(dst, o.bf16(), out_count, stream_) != Q8MI_OK) return failed("f32_to_bf16");
         return launch_status("hip q8 fp32->bf16 output");
     };
-    const float *xin = T(x).f32();
-    const bool contiguous = in_stride == cols && out_stride == rows;
-    if (batch > 8 && contiguous && cols % 32 == 0) {
-        const bool d4 = rows >= 128 && cols % 128 == 0;   // layout rule of src/kernels_cuda.cu:14545-14552
+    if (tiles) {
         if (d4) {
-            if (auto st = ensure(d4_, ported::q8_1_mmq_scratch_bytes(batch, cols), "q8_1_mmq scratch alloc"); !st.ok)
-                return st;
-            if (!ported::launch_quantize_mmq_q8_1(xin, d4_.ptr, batch, cols, cols, stream_))
-                return failed("quantize_mmq_q8_1");
+            if (!o.is_bf16()) {   // (quantized above otherwise)
+                if (auto st = quantize_d4(xin, batch, cols, cols); !st.ok) return st;
+            }
             const bool medium = batch >= 12 && batch <= 64;   // vmed range, src/kernels_cuda.cu:14566
             const bool ok = medium
                 ? ported::launch_mmq_q8_0_medium(w.ptr, d4_.ptr, dst, rows, cols, batch, rows, stream_)
@@ -366,98 +442,12 @@ DeviceStatus HipQ8Backend::q8_0_matmul(DeviceTensor &out, const DeviceWeight &we
     return finish(gemv_route(dst, weight, xin, batch, in_stride, out_stride));
 }
 
-// src/kernels_cuda.cu:11551-11613
-DeviceStatus HipQ8Backend::q8_0_matmul_fanout(DeviceTensor *const *outs, const DeviceWeight *const *weights,
-                                              const uint32_t *out_strides, uint32_t n, const DeviceTensor &x,
-                                              uint32_t batch, uint32_t in_stride) {
-    if (n == 0 || batch == 0) return {};
-    const uint32_t cols = static_cast<uint32_t>(W(*weights[0]).cols);
-    bool fast = batch <= 8 && in_stride == cols && cols % 32 == 0;
-    for (uint32_t i = 0; i < n && fast; ++i) {
-        const auto &w = W(*weights[i]);
-        fast = w.format == DeviceWeightFormat::Q8_0 && w.cols == cols && !T(*outs[i]).is_bf16();
-    }
-    if (!fast) {   // base-class behaviour: one q8_0_matmul per weight
-        for (uint32_t i = 0; i < n; ++i) {
-            if (auto st = q8_0_matmul(*outs[i], *weights[i], x, batch, in_stride, out_strides[i]); !st.ok) return st;
-        }
-        return {};
-    }
-    const bool fused = fuse_quantizer(batch, cols);
-    if (!fused) {
-        if (auto st = quantize_q8_1(T(x).f32(), batch, cols, in_stride); !st.ok) return st;
-    }
-    for (uint32_t i0 = 0; i0 < n; i0 += 4) {
-        const uint8_t *wp[4] = {nullptr, nullptr, nullptr, nullptr};
-        float *op[4] = {nullptr, nullptr, nullptr, nullptr};
-        uint32_t r[4] = {0, 0, 0, 0}, s[4] = {0, 0, 0, 0};
-        for (uint32_t i = i0; i < n && i < i0 + 4; ++i) {
-            wp[i - i0] = W(*weights[i]).ptr;
-            op[i - i0] = T(*outs[i]).f32();
-            r[i - i0] = static_cast<uint32_t>(W(*weights[i]).rows);
-            s[i - i0] = out_strides[i];
-        }
-        if (fused) {
-            if (q8mi_qgemv_fanout4(wp[0], wp[1], wp[2], wp[3], T(x).f32(), in_stride, op[0], op[1], op[2], op[3], r[0],
-                                   r[1], r[2], r[3], cols, batch, s[0], s[1], s[2], s[3], stream_) != Q8MI_OK)
-                return failed("qgemv_fanout4");
-            continue;
-        }
-        if (!ported::launch_mmvq_q8_0_fanout4_batch(wp[0], wp[1], wp[2], wp[3], q8_1_.ptr, op[0], op[1], op[2], op[3],
-                                                    r[0], r[1], r[2], r[3], cols, batch, s[0], s[1], s[2], s[3],
-                                                    stream_))
-            return failed("mmvq_q8_0_fanout4_batch");
-    }
-    return launch_status("hip q8_0_matmul_fanout");
-}
-
-// ---- RMS norm ------------------------------------------------------------------------------
-// src/kernels_cuda.cu:14748-14779
-DeviceStatus HipQ8Backend::rms_norm(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight, float eps) {
-    return rms_norm_batch(out, x, weight, 1, static_cast<uint32_t>(T(x).count), eps);
-}
-
-// src/kernels_cuda.cu:14781-14816
-DeviceStatus HipQ8Backend::rms_norm_batch(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight,
-                                          uint32_t batch, uint32_t n, float eps) {
-    if (batch == 0) return {};
-    const auto &w = W(weight);
-    if (T(out).is_bf16()) return {false, "hip rms_norm_batch BF16 output is not implemented"};
-    if (T(x).is_bf16()) return {false, "hip rms_norm_batch BF16 input is outside the Q8_0 path"};
-    if (w.format != DeviceWeightFormat::F32 || w.cols < n) return {false, "rms_norm_batch: norm weight is not fp32 [n]"};
-    if (T(x).count < static_cast<uint64_t>(batch) * n || T(out).count < static_cast<uint64_t>(batch) * n)
-        return {false, "rms_norm_batch: tensor smaller than batch * n"};
-    if (q8mi_rms_norm(T(x).f32(), reinterpret_cast<const float *>(w.ptr), T(out).f32(), batch, n, n, n, eps,
-                      stream_) != Q8MI_OK)
-        return failed("rms_norm");
-    return launch_status("hip rms_norm_batch");
-}
-
-// include/qw3/device_backend.hpp:421-444
-DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized, DeviceTensor *const *outs,
-                                                       const DeviceWeight *const *weights, const uint32_t *out_strides,
-                                                       uint32_t fanout, const DeviceTensor &x,
-                                                       const DeviceWeight &norm_weight, uint32_t batch,
-                                                       uint32_t in_stride, float eps) {
-    if (fanout == 0 || batch == 0) return {};
-    const auto &nw = W(norm_weight);
-    const uint32_t cols = in_stride;
-    bool fast = batch <= 8 && cols % 32 == 0 && !T(x).is_bf16() && !T(normalized).is_bf16() &&
-                nw.format == DeviceWeightFormat::F32 && nw.cols == cols &&
-                T(x).count >= static_cast<uint64_t>(batch) * cols &&
-                T(normalized).count >= static_cast<uint64_t>(batch) * cols;
-    for (uint32_t i = 0; i < fanout && fast; ++i) {
-        const auto &w = W(*weights[i]);
-        fast = w.format == DeviceWeightFormat::Q8_0 && w.cols == cols && !T(*outs[i]).is_bf16() &&
-               out_strides[i] >= w.rows && T(*outs[i]).count >= static_cast<uint64_t>(batch) * out_strides[i];
-    }
-    if (!fast) {   // base-class behaviour
-        if (auto st = rms_norm_batch(normalized, x, norm_weight, batch, in_stride, eps); !st.ok) return st;
-        return q8_0_matmul_fanout(outs, weights, out_strides, fanout, normalized, batch, in_stride);
-    }
-    const float *xin = T(x).f32();
-    const float *nwp = reinterpret_cast<const float *>(nw.ptr);
-    float *nrm = T(normalized).f32();
+// norm (already applied or to be applied inside the first launch) + projections of up to eight rows:
+// shared by rms_norm_q8_0_matmul_fanout and by a fan-out that follows a held-back one-row norm.
+// xin: the rows before the norm; nrm: where the normalised rows go.
+DeviceStatus HipQ8Backend::fanout_normed(float *nrm, const float *xin, const float *nwp, float eps,
+                                         DeviceTensor *const *outs, const DeviceWeight *const *weights,
+                                         const uint32_t *out_strides, uint32_t fanout, uint32_t batch, uint32_t cols) {
     auto group = [&](uint32_t i0, const uint8_t *(&wp)[4], float *(&op)[4], uint32_t (&r)[4], uint32_t (&s)[4]) {
         for (uint32_t k = 0; k < 4; ++k) { wp[k] = nullptr; op[k] = nullptr; r[k] = 0; s[k] = 0; }
         for (uint32_t i = i0; i < fanout && i < i0 + 4; ++i) {
@@ -472,13 +462,18 @@ DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized,
     uint32_t r[4], s[4];
     uint32_t first = 0;
     bool quantized = false;
+    forget_quantized();
     if (batch == 1 && nrm != xin) {   // the first four weights: norm + quantizer inside the GEMV, which also leaves
                                       // `normalized` (not in place: every workgroup reads x)
         group(0, wp, op, r, s);
-        const int rc = q8mi_nqgemv_fanout4(wp[0], wp[1], wp[2], wp[3], xin, nwp, eps, nrm, op[0], op[1], op[2], op[3],
-                                           r[0], r[1], r[2], r[3], cols, 1, stream_);
-        if (rc == Q8MI_OK) first = 4;
-        else if (rc != Q8MI_REJECTED) return failed("nqgemv_fanout4");
+        bool dense = true;            // the one-launch form writes dense rows
+        for (uint32_t k = 0; k < 4; ++k) dense = dense && (r[k] == 0 || s[k] == r[k]);
+        if (dense) {
+            const int rc = q8mi_nqgemv_fanout4(wp[0], wp[1], wp[2], wp[3], xin, nwp, eps, nrm, op[0], op[1], op[2], op[3],
+                                               r[0], r[1], r[2], r[3], cols, 1, stream_);
+            if (rc == Q8MI_OK) first = 4;
+            else if (rc != Q8MI_REJECTED) return failed("nqgemv_fanout4");
+        }
     }
     if (first == 0) {
         if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(batch, cols), "q8_1 scratch alloc"); !st.ok) return st;
@@ -499,7 +494,134 @@ DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized,
                                                     stream_))
             return failed("mmvq_q8_0_fanout4_batch");
     }
+    if (quantized) quantized_ = QuantizedRows{nrm, batch, cols, cols};   // the next projection of these rows reads the blocks
+    for (uint32_t i = 0; i < fanout; ++i) wrote(T(*outs[i]).ptr);
     return launch_status("hip rms_norm_q8_0_matmul_fanout");
+}
+
+// src/kernels_cuda.cu:11551-11613
+DeviceStatus HipQ8Backend::q8_0_matmul_fanout(DeviceTensor *const *outs, const DeviceWeight *const *weights,
+                                              const uint32_t *out_strides, uint32_t n, const DeviceTensor &x,
+                                              uint32_t batch, uint32_t in_stride) {
+    if (n == 0 || batch == 0) return {};
+    const uint32_t cols = static_cast<uint32_t>(W(*weights[0]).cols);
+    bool fast = batch <= 8 && in_stride == cols && cols % 32 == 0;
+    for (uint32_t i = 0; i < n && fast; ++i) {
+        const auto &w = W(*weights[i]);
+        fast = w.format == DeviceWeightFormat::Q8_0 && w.cols == cols && !T(*outs[i]).is_bf16();
+    }
+    const float *xin = T(x).f32();
+    if (fast && batch == 1 && pending_.active) {   // a held-back norm of x: inside the first launch
+        bool absorb = true;
+        for (uint32_t i = 0; i < n; ++i) absorb = absorb && absorbs_norm(xin, cols, T(*outs[i]).ptr);
+        if (absorb) {
+            const PendingNorm pn = pending_;
+            pending_.active = false;
+            return fanout_normed(pn.out, pn.x, pn.weight, pn.eps, outs, weights, out_strides, n, 1, cols);
+        }
+    }
+    if (auto st = flush_norm(); !st.ok) return st;
+    if (!fast) {   // base-class behaviour: one q8_0_matmul per weight
+        for (uint32_t i = 0; i < n; ++i) {
+            if (auto st = q8_0_matmul(*outs[i], *weights[i], x, batch, in_stride, out_strides[i]); !st.ok) return st;
+        }
+        return {};
+    }
+    const bool fused = fuse_quantizer(xin, batch, cols, in_stride);
+    if (!fused) {
+        if (auto st = quantize_q8_1(xin, batch, cols, in_stride); !st.ok) return st;
+    }
+    for (uint32_t i0 = 0; i0 < n; i0 += 4) {
+        const uint8_t *wp[4] = {nullptr, nullptr, nullptr, nullptr};
+        float *op[4] = {nullptr, nullptr, nullptr, nullptr};
+        uint32_t r[4] = {0, 0, 0, 0}, s[4] = {0, 0, 0, 0};
+        for (uint32_t i = i0; i < n && i < i0 + 4; ++i) {
+            wp[i - i0] = W(*weights[i]).ptr;
+            op[i - i0] = T(*outs[i]).f32();
+            r[i - i0] = static_cast<uint32_t>(W(*weights[i]).rows);
+            s[i - i0] = out_strides[i];
+        }
+        if (fused) {
+            if (q8mi_qgemv_fanout4(wp[0], wp[1], wp[2], wp[3], xin, in_stride, op[0], op[1], op[2], op[3], r[0],
+                                   r[1], r[2], r[3], cols, batch, s[0], s[1], s[2], s[3], stream_) != Q8MI_OK)
+                return failed("qgemv_fanout4");
+            continue;
+        }
+        if (!ported::launch_mmvq_q8_0_fanout4_batch(wp[0], wp[1], wp[2], wp[3], q8_1_.ptr, op[0], op[1], op[2], op[3],
+                                                    r[0], r[1], r[2], r[3], cols, batch, s[0], s[1], s[2], s[3],
+                                                    stream_))
+            return failed("mmvq_q8_0_fanout4_batch");
+    }
+    for (uint32_t i = 0; i < n; ++i) wrote(T(*outs[i]).ptr);
+    return launch_status("hip q8_0_matmul_fanout");
+}
+
+// ---- RMS norm ------------------------------------------------------------------------------
+// src/kernels_cuda.cu:14748-14779
+DeviceStatus HipQ8Backend::rms_norm(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight, float eps) {
+    return rms_norm_batch(out, x, weight, 1, static_cast<uint32_t>(T(x).count), eps);
+}
+
+// src/kernels_cuda.cu:14781-14816.  Up to eight rows (what a GEMV takes) also leave their Q8_1 blocks
+// in the scratch for the projection that follows; one row of a length the fused GEMVs serve is held
+// back for that projection's own launch (flush_norm runs it if something else comes first).
+DeviceStatus HipQ8Backend::rms_norm_batch(DeviceTensor &out, const DeviceTensor &x, const DeviceWeight &weight,
+                                          uint32_t batch, uint32_t n, float eps) {
+    if (batch == 0) return {};
+    const auto &w = W(weight);
+    if (T(out).is_bf16()) return {false, "hip rms_norm_batch BF16 output is not implemented"};
+    if (T(x).is_bf16()) return {false, "hip rms_norm_batch BF16 input is outside the Q8_0 path"};
+    if (w.format != DeviceWeightFormat::F32 || w.cols < n) return {false, "rms_norm_batch: norm weight is not fp32 [n]"};
+    if (T(x).count < static_cast<uint64_t>(batch) * n || T(out).count < static_cast<uint64_t>(batch) * n)
+        return {false, "rms_norm_batch: tensor smaller than batch * n"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(T(out).ptr);
+    const float *xin = T(x).f32();
+    const float *nwp = reinterpret_cast<const float *>(w.ptr);
+    float *nrm = T(out).f32();
+    auto aligned16 = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (batch == 1 && n % 256 == 0 && n <= 6144 && nrm != xin && aligned16(xin) && aligned16(nwp) && aligned16(nrm)) {
+        pending_ = PendingNorm{true, xin, nwp, nrm, n, eps};
+        return {};
+    }
+    if (batch <= 8 && n % 32 == 0) {
+        forget_quantized();
+        if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(batch, n), "q8_1 scratch alloc"); !st.ok) return st;
+        if (q8mi_rms_norm_quantize_q8_1(xin, nwp, nrm, q8_1_.ptr, batch, n, n, n, eps, stream_) != Q8MI_OK)
+            return failed("rms_norm_quantize_q8_1");
+        quantized_ = QuantizedRows{nrm, batch, n, n};
+        return launch_status("hip rms_norm_batch");
+    }
+    if (q8mi_rms_norm(xin, nwp, nrm, batch, n, n, n, eps, stream_) != Q8MI_OK) return failed("rms_norm");
+    return launch_status("hip rms_norm_batch");
+}
+
+// include/qw3/device_backend.hpp:421-444
+DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized, DeviceTensor *const *outs,
+                                                       const DeviceWeight *const *weights, const uint32_t *out_strides,
+                                                       uint32_t fanout, const DeviceTensor &x,
+                                                       const DeviceWeight &norm_weight, uint32_t batch,
+                                                       uint32_t in_stride, float eps) {
+    if (fanout == 0 || batch == 0) return {};
+    if (auto st = flush_norm(); !st.ok) return st;
+    const auto &nw = W(norm_weight);
+    const uint32_t cols = in_stride;
+    bool fast = batch <= 8 && cols % 32 == 0 && !T(x).is_bf16() && !T(normalized).is_bf16() &&
+                nw.format == DeviceWeightFormat::F32 && nw.cols == cols &&
+                T(x).count >= static_cast<uint64_t>(batch) * cols &&
+                T(normalized).count >= static_cast<uint64_t>(batch) * cols;
+    for (uint32_t i = 0; i < fanout && fast; ++i) {
+        const auto &w = W(*weights[i]);
+        fast = w.format == DeviceWeightFormat::Q8_0 && w.cols == cols && !T(*outs[i]).is_bf16() &&
+               out_strides[i] >= w.rows && T(*outs[i]).count >= static_cast<uint64_t>(batch) * out_strides[i];
+    }
+    if (!fast) {   // base-class behaviour
+        if (auto st = rms_norm_batch(normalized, x, norm_weight, batch, in_stride, eps); !st.ok) return st;
+        return q8_0_matmul_fanout(outs, weights, out_strides, fanout, normalized, batch, in_stride);
+    }
+    wrote(T(normalized).ptr);
+    return fanout_normed(T(normalized).f32(), T(x).f32(), reinterpret_cast<const float *>(nw.ptr), eps, outs, weights,
+                         out_strides, fanout, batch, cols);
 }
 
 // src/kernels_cuda.cu:14818-14862: elementwise out = a + b over the first `count` elements; the
@@ -517,25 +639,64 @@ DeviceStatus HipQ8Backend::add_n(DeviceTensor &out, const DeviceTensor &a, const
         if (!aa.is_bf16()) return {false, "hip add_n BF16 output with FP32 lhs"};
         if (!bb.is_bf16()) return {false, "hip add_n BF16 output with FP32 rhs"};
     }
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
     if (q8mi_add(o.ptr, aa.ptr, bb.ptr, count, o.is_bf16() ? 1 : 0, stream_) != Q8MI_OK) return failed("add");
     return launch_status("hip add");
 }
 
-// src/kernels_cuda.cu:11919-11957: in-place residual add for batch <= 8, else matmul + add
+// src/kernels_cuda.cu:14880-14900
+DeviceStatus HipQ8Backend::silu_mul(DeviceTensor &out, const DeviceTensor &gate, const DeviceTensor &up) {
+    return silu_mul_n(out, gate, up, out.count);
+}
+
+DeviceStatus HipQ8Backend::silu_mul_n(DeviceTensor &out, const DeviceTensor &gate, const DeviceTensor &up,
+                                      uint64_t count) {
+    auto &o = T(out);
+    const auto &g = T(gate), &u = T(up);
+    if (count > o.count || count > g.count || count > u.count) return {false, "hip silu_mul_n count exceeds tensor size"};
+    if (o.is_bf16() || g.is_bf16() || u.is_bf16()) return {false, "hip silu_mul_n: fp32 tensors only"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
+    if (q8mi_silu_mul(o.f32(), g.f32(), u.f32(), count, stream_) != Q8MI_OK) return failed("silu_mul");
+    return launch_status("hip silu_mul");
+}
+
+// src/kernels_cuda.cu:11919-11957: in-place residual add for batch <= 8; above, the tile kernel
+// adds the residual in its store where it can, else matmul + add
 DeviceStatus HipQ8Backend::q8_0_matmul_add(DeviceTensor &out, const DeviceTensor &residual, DeviceTensor &matmul_tmp,
                                            const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
                                            uint32_t in_stride, uint32_t out_stride) {
     const auto &w = W(weight);
     auto &o = T(out);
     const uint32_t cols = static_cast<uint32_t>(w.cols), rows = static_cast<uint32_t>(w.rows);
-    const bool fast = o.ptr == T(residual).ptr && w.format == DeviceWeightFormat::Q8_0 && cols % 32 == 0 &&
-                      batch >= 1 && batch <= 8 && in_stride == cols &&
-                      o.count >= static_cast<uint64_t>(batch) * out_stride;
+    const bool shapes_ok = w.format == DeviceWeightFormat::Q8_0 && cols % 32 == 0 && batch >= 1 && in_stride == cols &&
+                           o.count >= static_cast<uint64_t>(batch) * out_stride;
+    const bool fast = shapes_ok && o.ptr == T(residual).ptr && batch <= 8;
+    if (auto st = flush_norm(); !st.ok) return st;
     if (!fast) {
+        if (shapes_ok && batch > 8 && out_stride == rows && rows >= 128 && cols % 256 == 0 && !o.is_bf16() &&
+            !T(residual).is_bf16() && !T(matmul_tmp).is_bf16() &&
+            T(residual).count >= static_cast<uint64_t>(batch) * out_stride &&
+            T(matmul_tmp).count >= static_cast<uint64_t>(batch) * out_stride) {
+            wrote(o.ptr);
+            wrote(T(matmul_tmp).ptr);
+            if (auto st = quantize_d4(T(x).f32(), batch, cols, cols); !st.ok) return st;
+            const int rc = q8mi_gemm_add(w.ptr, d4_.ptr, T(residual).f32(), o.f32(), rows, cols, batch, rows, stream_);
+            if (rc == Q8MI_OK) return launch_status("hip q8_0_matmul_add mmq");
+            if (rc != Q8MI_REJECTED) return failed("gemm_add");
+            // a shape the tile kernel sums from two halves of K: the same records, then the add
+            if (!ported::launch_mmq_q8_0(w.ptr, d4_.ptr, T(matmul_tmp).f32(), rows, cols, batch, rows, stream_))
+                return failed("mmq_q8_0");
+            if (q8mi_add(o.ptr, T(residual).ptr, T(matmul_tmp).ptr, static_cast<uint64_t>(batch) * rows, 0, stream_) != Q8MI_OK)
+                return failed("add");
+            return launch_status("hip q8_0_matmul_add mmq + add");
+        }
         // include/qw3/device_backend.hpp:529-540: the matmul into the temporary, then out = residual + tmp
         if (auto st = q8_0_matmul(matmul_tmp, weight, x, batch, in_stride, out_stride); !st.ok) return st;
         return add(out, residual, matmul_tmp);
     }
+    wrote(o.ptr);
     if (auto st = quantize_q8_1(T(x).f32(), batch, cols, in_stride); !st.ok) return st;
     const bool ok = o.is_bf16()
         ? ported::launch_mmvq_q8_0_add_bf16(w.ptr, q8_1_.ptr, o.bf16(), rows, cols, batch, out_stride, stream_)
@@ -544,15 +705,61 @@ DeviceStatus HipQ8Backend::q8_0_matmul_add(DeviceTensor &out, const DeviceTensor
     return launch_status("hip q8_0_matmul_add");
 }
 
-// src/kernels_cuda.cu:12323-12333: not fused for Q8_0; the executor runs two matmuls + silu_mul_n
-DeviceStatus HipQ8Backend::q8_0_matmul_silu_mul(DeviceTensor &, const DeviceWeight &, const DeviceWeight &,
-                                                const DeviceTensor &, uint32_t, uint32_t, uint32_t) {
-    return {false, "q8_0_matmul_silu_mul not implemented for Q8_0 weights"};
+// include/qw3/device_backend.hpp:330-336 (batch 1: src/kernels_cuda.cu:12227-12258).  One GEMV launch
+// for up to eight rows; above, D4 records once and one launch of the dual-weight tiles; shapes
+// neither serves run as GEMV slices of eight rows.
+DeviceStatus HipQ8Backend::q8_0_matmul_silu_mul(DeviceTensor &out, const DeviceWeight &weight_gate,
+                                                const DeviceWeight &weight_up, const DeviceTensor &x,
+                                                uint32_t batch, uint32_t in_stride, uint32_t out_stride) {
+    const auto &g = W(weight_gate), &u = W(weight_up);
+    auto &o = T(out);
+    if (batch == 0) return {};
+    if (g.format != DeviceWeightFormat::Q8_0 || u.format != DeviceWeightFormat::Q8_0)
+        return {false, "q8_0_matmul_silu_mul: weights are not Q8_0"};
+    if (g.rows != u.rows || g.cols != u.cols) return {false, "q8_0_matmul_silu_mul: gate/up shapes differ"};
+    if (o.is_bf16() || T(x).is_bf16()) return {false, "q8_0_matmul_silu_mul: fp32 tensors only"};
+    const uint32_t cols = static_cast<uint32_t>(g.cols), rows = static_cast<uint32_t>(g.rows);
+    if (cols % 32 != 0) return {false, "q8_0_matmul_silu_mul: cols not a multiple of 32"};
+    if (in_stride < cols || out_stride < rows) return {false, "q8_0_matmul_silu_mul: stride shorter than a row"};
+    if (T(x).count < static_cast<uint64_t>(batch - 1) * in_stride + cols ||
+        o.count < static_cast<uint64_t>(batch - 1) * out_stride + rows)
+        return {false, "q8_0_matmul_silu_mul: tensor smaller than the batch"};
+    const float *xin = T(x).f32();
+    if (batch == 1 && absorbs_norm(xin, cols, o.ptr)) {   // norm, quantizer and SwiGLU GEMV in one launch
+        const int rc = q8mi_nqgemv_silu_mul(g.ptr, u.ptr, pending_.x, pending_.weight, pending_.eps, pending_.out,
+                                            o.f32(), rows, cols, 1, stream_);
+        if (rc == Q8MI_OK) {
+            pending_.active = false;
+            wrote(o.ptr);
+            return launch_status("hip rms_norm + q8_0_matvec_silu_mul");
+        }
+        if (rc != Q8MI_REJECTED) return failed("nqgemv_silu_mul");
+    }
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
+    if (fuse_quantizer(xin, batch, cols, in_stride) &&
+        q8mi_qgemv_silu_mul(g.ptr, u.ptr, xin, in_stride, o.f32(), rows, cols, 1, out_stride, stream_) == Q8MI_OK)
+        return launch_status("hip q8_0_matvec_silu_mul fused");
+    if (batch > 8 && rows >= 128 && cols % 256 == 0) {
+        if (auto st = quantize_d4(xin, batch, cols, in_stride); !st.ok) return st;
+        const int rc = q8mi_gemm_silu_mul(g.ptr, u.ptr, d4_.ptr, o.f32(), rows, cols, batch, out_stride, stream_);
+        if (rc == Q8MI_OK) return launch_status("hip q8_0_matmul_silu_mul mmq");
+        if (rc != Q8MI_REJECTED) return failed("gemm_silu_mul");
+    }
+    for (uint32_t j0 = 0; j0 < batch; j0 += 8) {
+        const uint32_t m = batch - j0 < 8 ? batch - j0 : 8;
+        if (auto st = quantize_q8_1(xin + static_cast<uint64_t>(j0) * in_stride, m, cols, in_stride); !st.ok) return st;
+        if (!ported::launch_mmvq_q8_0_silu_mul(g.ptr, u.ptr, q8_1_.ptr, o.f32() + static_cast<uint64_t>(j0) * out_stride,
+                                               rows, cols, m, out_stride, stream_))
+            return failed("mmvq_q8_0_silu_mul");
+    }
+    return launch_status("hip q8_0_matmul_silu_mul");
 }
 
 // ---- argmax (src/kernels_cuda.cu:20733-20850) ------------------------------------------------
 DeviceStatus HipQ8Backend::argmax_launch(const DeviceTensor &x) {
     const auto &t = T(x);
+    if (auto st = flush_norm(); !st.ok) return st;
     if (!argmax_dev_) {
         if (capturing_) return {false, "argmax buffers must exist before capture"};
         if (auto st = hip_status(hipMalloc(reinterpret_cast<void **>(&argmax_dev_), 8), "argmax alloc"); !st.ok)
@@ -601,6 +808,7 @@ std::unique_ptr<DeviceArgmaxBuffer> HipQ8Backend::argmax_buffer(uint64_t count) 
 DeviceStatus HipQ8Backend::argmax_to_buffer(const DeviceTensor &x, DeviceArgmaxBuffer &out, uint32_t index) {
     auto &dst = static_cast<HipArgmaxBuffer &>(out);
     if (index >= dst.count) return {false, "argmax_to_buffer index oob"};
+    if (auto st = flush_norm(); !st.ok) return st;
     if (q8mi_argmax_to_pair(T(x).f32(), T(x).count, dst.ptr, index, stream_) != Q8MI_OK)
         return failed("argmax_to_pair");
     return launch_status("hip argmax_to_buffer");
@@ -612,6 +820,8 @@ DeviceStatus HipQ8Backend::q8_0_get_row(DeviceTensor &out, const DeviceWeight &w
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "row lookup requires Q8_0 weight"};
     if (o.count < w.cols) return {false, "q8_0_get_row: output smaller than a row"};
     if (row >= w.rows) return {false, "q8_0_get_row: row outside the matrix"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
     if (q8mi_get_row(w.ptr, row, w.rows, w.cols, o.ptr, o.is_bf16() ? 1 : 0, stream_) != Q8MI_OK)
         return failed("get_row");
     return launch_status("hip q8_0_get_row");
@@ -626,6 +836,8 @@ DeviceStatus HipQ8Backend::q8_0_get_row_from_argmax(DeviceTensor &out, const Dev
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "argmax row lookup requires Q8_0 weight"};
     if (o.is_bf16()) return {false, "q8_0_get_row_from_argmax: fp32 output only"};
     if (o.count < w.cols) return {false, "q8_0_get_row_from_argmax: output smaller than a row"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
     if (q8mi_get_row_from_argmax(w.ptr, a.ptr, index, w.rows, w.cols, o.f32(), stream_) != Q8MI_OK)
         return failed("get_row_from_argmax");
     return launch_status("hip q8_0_get_row_from_argmax");
@@ -638,6 +850,8 @@ DeviceStatus HipQ8Backend::q8_0_get_rows_batch(DeviceTensor &out, const DeviceWe
     auto &o = T(out);
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "batched row lookup requires Q8_0 weight"};
     if (o.count < static_cast<uint64_t>(batch) * w.cols) return {false, "q8_0_get_rows_batch: output too small"};
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(o.ptr);
     // grow-only device copy of the ids (src/kernels_cuda.cu:10722-10727)
     if (auto st = ensure(row_ids_, batch * sizeof(uint64_t), "row id buffer"); !st.ok) return st;
     if (auto st = hip_status(hipMemcpyAsync(row_ids_.ptr, rows, batch * sizeof(uint64_t), hipMemcpyHostToDevice,
@@ -667,6 +881,7 @@ DeviceStatus HipQ8Backend::argmax_batch(const DeviceTensor &x, uint32_t batch, u
     const auto &t = T(x);
     out.assign(batch, DeviceArgmax{});
     if (batch == 0) return {};
+    if (auto st = flush_norm(); !st.ok) return st;
     const uint32_t blocks_per_row = (row_stride + 255) / 256;
     if (row_stride == 0 || blocks_per_row > 1024 || t.count < static_cast<uint64_t>(batch) * row_stride) {
         // the reference's host scan (include/qw3/device_backend.hpp:2477-2497)
@@ -706,6 +921,7 @@ DeviceStatus HipQ8Backend::lm_head_verify(const DeviceWeight &w_out, const Devic
     const auto &w = W(w_out);
     if (w.format != DeviceWeightFormat::Q8_0) return {false, "lm_head_verify: weight is not Q8_0"};
     if (batch == 0 || batch > 8 || n_drafts + 1 != batch) return {false, "lm_head_verify: batch must be drafts + 1, <= 8"};
+    if (auto st = flush_norm(); !st.ok) return st;
     const uint32_t cols = static_cast<uint32_t>(w.cols), vocab = static_cast<uint32_t>(w.rows);
     if (auto st = ensure(lm_head_, q8mi_lm_head_scratch_bytes(vocab, cols, batch), "lm head scratch alloc"); !st.ok)
         return st;

@@ -115,9 +115,17 @@ public:
     DeviceStatus q8_0_matmul_add(DeviceTensor &out, const DeviceTensor &residual, DeviceTensor &matmul_tmp,
                                  const DeviceWeight &weight, const DeviceTensor &x, uint32_t batch,
                                  uint32_t in_stride, uint32_t out_stride);
+    // out[j][r] = silu(gate row r . x[j]) * (up row r . x[j]) for `batch` rows of x
+    // (include/qw3/device_backend.hpp:330-336): one GEMV launch up to eight rows, one tile launch
+    // above (the reference's CUDA backend declines Q8_0 here and the executor runs two matmuls and
+    // silu_mul_n, src/kernels_cuda.cu:12323-12333, src/qwen_executor.cpp:6669-6685)
     DeviceStatus q8_0_matmul_silu_mul(DeviceTensor &out, const DeviceWeight &weight_gate,
                                       const DeviceWeight &weight_up, const DeviceTensor &x, uint32_t batch,
                                       uint32_t in_stride, uint32_t out_stride);
+    // elementwise out = silu(gate) * up over the whole of `out` / its first `count` elements
+    // (include/qw3/device_backend.hpp:652-663, src/kernels_cuda.cu:14880-14900); fp32 tensors
+    DeviceStatus silu_mul(DeviceTensor &out, const DeviceTensor &gate, const DeviceTensor &up);
+    DeviceStatus silu_mul_n(DeviceTensor &out, const DeviceTensor &gate, const DeviceTensor &up, uint64_t count);
 
     // RMS norm in front of the projections.  rms_norm normalises the whole tensor as one row
     // (src/kernels_cuda.cu:14748-14779), rms_norm_batch `batch` dense rows of n (:14781-14816).
@@ -235,14 +243,46 @@ private:
         void *ptr = nullptr;
         size_t capacity = 0;
     };
+    // A one-row rms_norm whose launch is held back until the next call: when that call is a
+    // batch-1 projection of the normalised row, norm, quantizer and GEMV run as one launch (which
+    // also writes the normalised row); any other call runs the norm first.  Nothing a caller can
+    // observe depends on which of the two happened.
+    struct PendingNorm {
+        bool active = false;
+        const float *x = nullptr;
+        const float *weight = nullptr;
+        float *out = nullptr;
+        uint32_t cols = 0;
+        float eps = 0.0f;
+    };
+    // What the Q8_1 scratch holds: the blocks of `batch` rows of `cols` floats at `src`, written by
+    // the norm that produced those rows.  Valid only until the next call that writes a tensor or
+    // the scratch: the projections that follow a norm read them instead of quantizing again.
+    struct QuantizedRows {
+        const float *src = nullptr;
+        uint32_t batch = 0, cols = 0, stride = 0;
+    };
+    DeviceStatus flush_norm();
+    void forget_quantized() { quantized_ = QuantizedRows{}; }
+    bool absorbs_norm(const float *x, uint32_t cols, const void *out0) const;
     DeviceStatus ensure(Scratch &s, size_t need, const char *what);
     DeviceStatus launch_status(const char *where);
     DeviceStatus failed(const char *where);
+    void wrote(const void *tensor) {   // a call that writes `tensor`: its rows' blocks in the scratch are stale
+        if (tensor == quantized_.src) forget_quantized();
+    }
+    bool fuse_quantizer(const float *x, uint32_t batch, uint32_t cols, uint32_t stride) const;
     DeviceStatus quantize_q8_1(const float *x, uint32_t batch, uint32_t cols, uint32_t stride);
+    DeviceStatus quantize_d4(const float *x, uint32_t batch, uint32_t cols, uint32_t stride);
+    DeviceStatus fanout_normed(float *nrm, const float *xin, const float *nwp, float eps, DeviceTensor *const *outs,
+                               const DeviceWeight *const *weights, const uint32_t *out_strides, uint32_t fanout,
+                               uint32_t batch, uint32_t cols);
     DeviceStatus gemv_route(float *out, const DeviceWeight &w, const float *x, uint32_t batch, uint32_t in_stride,
                             uint32_t out_stride);
 
     hipStream_t stream_ = nullptr;
+    PendingNorm pending_;
+    QuantizedRows quantized_;
     Scratch q8_1_, d4_, argmax_partial_, argmax_result_, lm_head_, lm_rows_, out_f32_, row_ids_;
     int32_t *argmax_dev_ = nullptr;    // {token, logit bits}
     int32_t *argmax_host_ = nullptr;   // pinned mirror

@@ -8,8 +8,7 @@ import ctypes as C
 import os
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-# Q8MI_LIB points at another build of the same library (tuning variants)
-LIB_PATH = os.environ.get("Q8MI_LIB") or os.path.join(PKG_DIR, "libq8mi.so")
+LIB_PATH = os.path.join(PKG_DIR, "libq8mi.so")
 
 OK, REJECTED, LAUNCH_ERROR = 0, 1, 2
 QK = 32
@@ -46,6 +45,10 @@ SIGNATURES = {
     "q8mi_quantize_q8_1_d4": (_int, [_vp, _vp, _u32, _u32, _u32, _vp]),
     "q8mi_gemm": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_gemm_medium": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_gemm_add": (_int, [_u8p, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_gemm_bf16": (_int, [_u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_gemm_silu_mul": (_int, [_u8p, _u8p, _vp, _vp, _u32, _u32, _u32, _u32, _vp]),
+    "q8mi_silu_mul": (_int, [_vp, _vp, _vp, _u64, _vp]),
     "q8mi_f32_to_bf16": (_int, [_vp, _vp, _u64, _vp]),
     "q8mi_add": (_int, [_vp, _vp, _vp, _u64, _int, _vp]),
     "q8mi_get_row": (_int, [_u8p, _u64, _u64, _u64, _vp, _int, _vp]),

@@ -91,11 +91,14 @@ void oracle_linear(const HostWeight &w, const float *x, uint32_t batch, uint32_t
     }
 }
 
-void oracle_gemm_d4(const HostWeight &w, const float *x, uint32_t batch, std::vector<float> &ref) {
+void oracle_gemm_d4(const HostWeight &w, const float *x, uint32_t batch, std::vector<float> &ref, uint32_t in_stride = 0,
+                    uint32_t out_stride = 0) {
+    in_stride = in_stride ? in_stride : w.cols;
+    out_stride = out_stride ? out_stride : w.rows;
     std::vector<uint8_t> y(static_cast<size_t>(w.cols / 128) * batch * 144);
-    q8o_quantize_q8_1_d4(x, batch, w.cols, w.cols, y.data());
-    ref.assign(static_cast<size_t>(batch) * w.rows, 0.0f);
-    q8o_gemm_d4(w.split.data(), y.data(), ref.data(), w.rows, w.cols, batch, w.rows, 8);
+    q8o_quantize_q8_1_d4(x, batch, w.cols, in_stride, y.data());
+    ref.assign(static_cast<size_t>(batch) * out_stride, 0.0f);
+    q8o_gemm_d4(w.split.data(), y.data(), ref.data(), w.rows, w.cols, batch, out_stride, 8);
 }
 
 // |got - ref| <= 1e-5 |ref| + 1e-6 * sum|terms|: the allowance for a different
@@ -382,9 +385,11 @@ void case_matmul(qw3::HipQ8Backend &b) {
         }
         // forms the backend declines, as the reference does
         auto other = b.tensor_f32(static_cast<size_t>(nb) * wa.rows, "other");
-        ok = !b.q8_0_matmul_silu_mul(*other, *da, *da, *dx, nb, cols, wa.rows).ok;
+        ok = !b.q8_0_matmul_silu_mul(*other, *da, *db, *dx, nb, cols, wa.rows).ok;   // gate / up heights differ
+        ok = ok && !b.q8_0_matmul_silu_mul(*other, *da, *da, *dx, nb, cols - 1, wa.rows).ok;   // stride shorter than a row
         ok = ok && b.weight_q8_0(wa.gguf.data(), 4, 40, "bad") == nullptr;
         ok = ok && !b.add_n(*other, *other, *other, other->count + 1).ok;
+        ok = ok && !b.silu_mul_n(*other, *other, *other, other->count + 1).ok;
         report("declined_forms", ok);
     }
 }
@@ -445,6 +450,192 @@ void case_matmul_add_batched(qw3::HipQ8Backend &b) {
         }
         ok = ok && far == 0 && off * 100 < got.size();
         report("matmul_add_bf16_batch64", ok, "differing " + std::to_string(off) + ", beyond one step " + std::to_string(far));
+    }
+}
+
+// silu(g) * u for sums g, u that are each within the GEMV / GEMM tolerance (tg, tu) of their
+// references: the derivative bound |silu'| <= 1.1 and a few ulp of the fast exponential.
+bool close_swiglu(const std::vector<float> &got, const std::vector<float> &gref, const std::vector<float> &gmag,
+                  const std::vector<float> &uref, const std::vector<float> &umag, uint32_t batch, uint32_t rows,
+                  uint32_t stride, std::string &detail) {
+    for (uint32_t j = 0; j < batch; ++j)
+        for (uint32_t r = 0; r < rows; ++r) {
+            const size_t i = static_cast<size_t>(j) * stride + r;
+            const double g = gref[i], u = uref[i];
+            const double want = g / (1.0 + std::exp(-g)) * u;
+            const double tg = 1e-5 * std::fabs(g) + 1e-6 * gmag[i], tu = 1e-5 * std::fabs(u) + 1e-6 * umag[i];
+            const double tol = 1.1 * tg * std::fabs(u) + tu * std::fabs(g) + 1e-6 * std::fabs(want) + 1e-30;
+            if (!(std::fabs(got[i] - want) <= tol)) {
+                char buf[160];
+                std::snprintf(buf, sizeof(buf), "[%u,%u] got %.9g want %.9g tol %.3g", j, r, got[i], want, tol);
+                detail = buf;
+                return false;
+            }
+        }
+    return true;
+}
+
+// q8_0_matmul_silu_mul (include/qw3/device_backend.hpp:330-336) for Q8_0 at every batch regime: GEMV
+// (2, 8, strided), matrix-core GEMV on D4 records (9, 16), ring tiles (20, 40, 64, 300) and main tiles
+// (512 x 3328 rows, and ragged 500 x 3300), against the oracle's two products (Q8_1 rows up to eight,
+// D4 records above: the quantizer each route uses) combined in double; and silu_mul / silu_mul_n.
+void case_silu_mul(qw3::HipQ8Backend &b) {
+    std::string d;
+    auto run = [&](uint32_t rows, uint32_t cols, uint32_t batch, uint32_t in_stride, uint32_t out_stride, uint64_t seed) {
+        d.clear();
+        const HostWeight wg = make_weight(rows, cols, seed), wu = make_weight(rows, cols, seed + 1);
+        auto dg = b.weight_q8_0(wg.gguf.data(), rows, cols, "g");
+        auto du = b.weight_q8_0(wu.gguf.data(), rows, cols, "u");
+        const auto x = normal_vec(static_cast<size_t>(batch) * in_stride, seed + 2);
+        auto dx = upload_f32(b, x);
+        auto out = b.tensor_f32(static_cast<size_t>(batch) * out_stride, "o");
+        bool ok = dg && du && require(b.zero_tensor(*out), "zero");
+        ok = ok && require(b.q8_0_matmul_silu_mul(*out, *dg, *du, *dx, batch, in_stride, out_stride), "matmul_silu_mul");
+        std::vector<float> gref, gmag, uref, umag;
+        oracle_linear(wg, x.data(), batch, in_stride, out_stride, gref, gmag);
+        oracle_linear(wu, x.data(), batch, in_stride, out_stride, uref, umag);
+        if (batch > 8 && rows >= 128 && cols % 256 == 0) {   // D4 records
+            oracle_gemm_d4(wg, x.data(), batch, gref, in_stride, out_stride);
+            oracle_gemm_d4(wu, x.data(), batch, uref, in_stride, out_stride);
+        }
+        const auto got = download_f32(b, *out);
+        ok = ok && close_swiglu(got, gref, gmag, uref, umag, batch, rows, out_stride, d);
+        for (uint32_t j = 0; j < batch && ok; ++j)     // the gap between rows stays untouched
+            for (uint32_t r = rows; r < out_stride; ++r)
+                if (got[static_cast<size_t>(j) * out_stride + r] != 0.0f) { ok = false; d = "wrote into the stride gap"; }
+        char name[96];
+        std::snprintf(name, sizeof(name), "matmul_silu_mul_%ux%u_batch%u%s", rows, cols, batch,
+                      (in_stride != cols || out_stride != rows) ? "_strided" : "");
+        report(name, ok, d);
+    };
+    for (uint32_t batch : {1u, 2u, 8u, 9u, 16u, 20u, 40u, 64u, 300u}) run(384, 1024, batch, 1024, 384, 500 + batch);
+    run(384, 1024, 5, 1024 + 32, 384 + 8, 520);       // strided GEMV route
+    run(384, 1024, 19, 1024 + 32, 384 + 8, 521);      // strided above eight rows: the tiles take strides
+    run(200, 480, 12, 480, 200, 522);                 // cols % 128 != 0: GEMV slices
+    run(3328, 512, 512, 512, 3328, 523);              // 64 + 64-row main tiles
+    run(3300, 512, 500, 512, 3300, 524);              // the same with ragged edges
+
+    // elementwise silu_mul / silu_mul_n on a length that is not a multiple of four
+    {
+        const size_t n = 4099, part = 1030;
+        const auto g = normal_vec(n, 530, 3.0f), u = normal_vec(n, 531);
+        auto dg = upload_f32(b, g), du = upload_f32(b, u);
+        auto out = b.tensor_f32(n, "o");
+        bool ok = require(b.zero_tensor(*out), "zero") && require(b.silu_mul_n(*out, *dg, *du, part), "silu_mul_n");
+        auto got = download_f32(b, *out);
+        auto check = [&](size_t upto) {
+            for (size_t i = 0; i < n && ok; ++i) {
+                const double want = i < upto ? static_cast<double>(g[i]) / (1.0 + std::exp(-static_cast<double>(g[i]))) * u[i] : 0.0;
+                if (!(std::fabs(got[i] - want) <= 1e-6 * std::fabs(want))) { ok = false; d = "element " + std::to_string(i); }
+            }
+        };
+        check(part);
+        ok = ok && require(b.silu_mul(*out, *dg, *du), "silu_mul");
+        got = download_f32(b, *out);
+        check(n);
+        report("silu_mul_n", ok, d);
+    }
+}
+
+// A norm and the projection that reads its output share a launch (one row) or the quantized rows
+// (up to eight); whatever a caller does in between, the results are the bits of the separate steps.
+void case_norm_reuse(qw3::HipQ8Backend &b) {
+    std::string d;
+    const uint32_t cols = 2048, rows = 640;
+    const float eps = 1e-6f;
+    const HostWeight w = make_weight(rows, cols, 601), w2 = make_weight(rows, cols, 602), wd = make_weight(cols, rows, 603);
+    auto dw = b.weight_q8_0(w.gguf.data(), rows, cols, "w");
+    auto dw2 = b.weight_q8_0(w2.gguf.data(), rows, cols, "w2");
+    auto nwv = normal_vec(cols, 604, 0.4f);
+    for (auto &f : nwv) f += 1.0f;
+    auto nw = b.weight_f32(nwv.data(), cols, "norm.weight");
+    auto bits_equal = [](const std::vector<float> &a, const std::vector<float> &c) {
+        return a.size() == c.size() && std::memcmp(a.data(), c.data(), a.size() * 4) == 0;
+    };
+    for (uint32_t batch : {1u, 3u}) {
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 610 + batch, 2.0f);
+        auto dx = upload_f32(b, x);
+        std::vector<float> nref(x.size());
+        q8o_rms_norm(x.data(), nwv.data(), nref.data(), batch, cols, cols, cols, eps);
+        auto norm_a = b.tensor_f32(x.size(), "na"), norm_b = b.tensor_f32(x.size(), "nb");
+        auto oa = b.tensor_f32(static_cast<size_t>(batch) * rows, "oa"), ob = b.tensor_f32(static_cast<size_t>(batch) * rows, "ob");
+        auto sa = b.tensor_f32(static_cast<size_t>(batch) * rows, "sa"), sb = b.tensor_f32(static_cast<size_t>(batch) * rows, "sb");
+        // back to back: the projection may take the norm into its launch / read the norm's blocks
+        bool ok = require(b.rms_norm_batch(*norm_a, *dx, *nw, batch, cols, eps), "norm") &&
+                  require(b.q8_0_matmul(*oa, *dw, *norm_a, batch, cols, rows), "matmul after norm") &&
+                  require(b.rms_norm_batch(*norm_a, *dx, *nw, batch, cols, eps), "norm") &&
+                  require(b.q8_0_matmul_silu_mul(*sa, *dw, *dw2, *norm_a, batch, cols, rows), "silu after norm");
+        // with a synchronisation in between: separate launches
+        ok = ok && require(b.rms_norm_batch(*norm_b, *dx, *nw, batch, cols, eps), "norm") && require(b.synchronize(), "sync") &&
+             require(b.zero_tensor(*ob), "zero") &&
+             require(b.q8_0_matmul(*ob, *dw, *norm_b, batch, cols, rows), "matmul") &&
+             require(b.zero_tensor(*sb), "zero") &&
+             require(b.q8_0_matmul_silu_mul(*sb, *dw, *dw2, *norm_b, batch, cols, rows), "silu");
+        ok = ok && bits_equal(download_f32(b, *norm_a), nref) && bits_equal(download_f32(b, *norm_b), nref);
+        ok = ok && bits_equal(download_f32(b, *oa), download_f32(b, *ob)) && bits_equal(download_f32(b, *sa), download_f32(b, *sb));
+        std::vector<float> ref, mag;
+        oracle_linear(w, nref.data(), batch, cols, rows, ref, mag);
+        ok = ok && close_fp32(download_f32(b, *oa), ref, mag, batch, rows, rows, d);
+        report(("norm_then_projection_batch" + std::to_string(batch)).c_str(), ok, d);
+
+        // the normalised rows change between two projections: the second must see the new rows
+        std::vector<float> other = normal_vec(x.size(), 620 + batch);
+        ok = require(b.rms_norm_batch(*norm_a, *dx, *nw, batch, cols, eps), "norm") &&
+             require(b.q8_0_matmul(*oa, *dw, *norm_a, batch, cols, rows), "matmul") &&
+             require(b.copy_bytes_from_host(*norm_a, 0, other.data(), other.size() * 4), "overwrite") &&
+             require(b.q8_0_matmul(*oa, *dw, *norm_a, batch, cols, rows), "matmul again");
+        oracle_linear(w, other.data(), batch, cols, rows, ref, mag);
+        ok = ok && close_fp32(download_f32(b, *oa), ref, mag, batch, rows, rows, d);
+        // ... also when a projection itself overwrites them (its output is the norm's output tensor)
+        auto sq = b.tensor_f32(static_cast<size_t>(batch) * cols, "sq");
+        auto dwd = b.weight_q8_0(wd.gguf.data(), cols, rows, "wd");
+        ok = ok && require(b.rms_norm_batch(*norm_a, *dx, *nw, batch, cols, eps), "norm") &&
+             require(b.q8_0_matmul(*oa, *dw, *norm_a, batch, cols, rows), "matmul") &&
+             require(b.q8_0_matmul(*norm_a, *dwd, *oa, batch, rows, cols), "matmul into the norm's tensor") &&
+             require(b.q8_0_matmul(*ob, *dw, *norm_a, batch, cols, rows), "matmul of the new rows");
+        const auto mid = download_f32(b, *norm_a);
+        oracle_linear(w, mid.data(), batch, cols, rows, ref, mag);
+        ok = ok && close_fp32(download_f32(b, *ob), ref, mag, batch, rows, rows, d);
+        report(("norm_rows_overwritten_batch" + std::to_string(batch)).c_str(), ok, d);
+    }
+    // one row, a projection that writes the norm's input: the norm must run first
+    {
+        const auto x = normal_vec(cols, 630, 2.0f);
+        auto h = upload_f32(b, x);
+        std::vector<float> nref(cols);
+        q8o_rms_norm(x.data(), nwv.data(), nref.data(), 1, cols, cols, cols, eps);
+        auto norm = b.tensor_f32(cols, "n");
+        const HostWeight wsq = make_weight(cols, cols, 631);
+        auto dsq = b.weight_q8_0(wsq.gguf.data(), cols, cols, "sq");
+        bool ok = require(b.rms_norm(*norm, *h, *nw, eps), "norm") && require(b.q8_0_matvec(*h, *dsq, *norm), "matvec into the norm's input");
+        std::vector<float> ref, mag;
+        oracle_linear(wsq, nref.data(), 1, cols, cols, ref, mag);
+        ok = ok && close_fp32(download_f32(b, *h), ref, mag, 1, cols, cols, d) && bits_equal(download_f32(b, *norm), nref);
+        report("norm_input_overwritten_by_projection", ok, d);
+    }
+    // a held-back norm inside a captured graph: replays equal the eager run
+    {
+        const auto x = normal_vec(cols, 640, 2.0f);
+        auto h = upload_f32(b, x);
+        auto norm = b.tensor_f32(cols, "n");
+        auto out = b.tensor_f32(rows, "o");
+        auto step = [&]() { return b.rms_norm(*norm, *h, *nw, eps).ok && b.q8_0_matvec_silu_mul(*out, *dw, *dw2, *norm).ok; };
+        bool ok = step() && require(b.synchronize(), "sync");
+        const auto eager = download_f32(b, *out);
+        ok = ok && b.begin_capture() && step();
+        ok = require(b.end_capture(), "end_capture") && ok;
+        for (int rep = 0; rep < 3 && ok; ++rep) {
+            ok = require(b.zero_tensor(*out), "zero") && require(b.zero_tensor(*norm), "zero") && require(b.replay_graph(), "replay") &&
+                 require(b.synchronize(), "sync");
+            ok = ok && bits_equal(download_f32(b, *out), eager);
+        }
+        // ... and a norm left pending when the capture ends is part of the graph
+        ok = ok && b.begin_capture() && b.rms_norm(*norm, *h, *nw, eps).ok;
+        ok = require(b.end_capture(), "end_capture") && ok;
+        std::vector<float> nref(cols);
+        q8o_rms_norm(x.data(), nwv.data(), nref.data(), 1, cols, cols, cols, eps);
+        ok = ok && require(b.zero_tensor(*norm), "zero") && require(b.replay_graph(), "replay") && bits_equal(download_f32(b, *norm), nref);
+        report("norm_held_back_under_capture", ok);
     }
 }
 
@@ -813,7 +1004,7 @@ int main(int argc, char **argv) {
     struct Case { const char *name; void (*fn)(qw3::HipQ8Backend &); };
     const Case cases[] = {
         {"closed_form", case_closed_form}, {"matvec", case_matvec_family}, {"matmul", case_matmul},
-        {"matmul_add", case_matmul_add_batched},
+        {"matmul_add", case_matmul_add_batched}, {"silu_mul", case_silu_mul}, {"norm_reuse", case_norm_reuse},
         {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"gguf", case_gguf}, {"lm_head", case_lm_head_verify}, {"rms_norm", case_rms_norm}, {"graph", case_graph_replay},
     };
     for (const auto &c : cases) {
