@@ -362,6 +362,37 @@ def bench_launches_m1(q8mi, hip, synth, step, layers, reps=300):
     return out
 
 
+def bench_row_length_sweep(q8mi, hip, synth, rows=HIDDEN, reps=300):
+    """q8mi_gemv at M=1 on `rows` weight rows of K columns, K = every whole number of KiB up to 17
+    and a few lengths in between, beside a plain streaming read of the same bytes: what a row length
+    without a kernel of its own costs.  Weights cycle through copies laid out in a 1 GiB buffer."""
+    L, ok = q8mi.lib(), q8mi.ok
+    big, sink = hip.DeviceBuffer(1 << 30), hip.DeviceBuffer(64)
+    out = {}
+    for cols in sorted(set(range(1024, 17408 + 1, 1024)) | {2560, 3584, 5632, 9728}):
+        host = synth.q8_0_weight(rows, cols, seed=cols)
+        nbytes = w_bytes(rows, cols)
+        span = (nbytes + 4095) // 4096 * 4096
+        copies = min((1 << 30) // span, 64)
+        for c in range(copies):
+            big.upload(host, c * span)
+        x = hip.to_device(synth.normal(1, cols, seed=cols + 1))
+        y = hip.DeviceBuffer(q81_bytes(1, cols))
+        dst = hip.DeviceBuffer(4 * rows)
+        ok(L.q8mi_quantize_q8_1(x.ptr, y.ptr, 1, cols, cols, None), "quantize")
+        t = time_loop(hip, lambda i: ok(L.q8mi_gemv(big.at((i % copies) * span), y.ptr, dst.ptr, rows, cols, 1, rows, None),
+                                        "gemv"), reps, copies)
+        p = time_loop(hip, lambda i: synth.ok(synth.lib().q8sup_probe_read(big.at((i % copies) * span), nbytes, 2, sink.ptr,
+                                                                           None), "probe_read"), reps, copies)
+        out[f"k{cols}"] = {"us": round(t * 1e3, 2), "plain_read_us": round(p * 1e3, 2), "ratio": round(t / p, 3),
+                           "gbps": round((nbytes + q81_bytes(1, cols) + 4 * rows) / (t * 1e-3) / 1e9, 1)}
+        for b in (x, y, dst):
+            b.free()
+    big.free()
+    sink.free()
+    return out
+
+
 def bench_read_probe(synth, hip, nbytes=1 << 30, reps=20):
     """Measured ceiling of a plain streaming read (every lane 16 bytes per load, grid-stride)."""
     buf, sink = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(64)
@@ -676,7 +707,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="distinct weight copies cycled through (streaming)")
     ap.add_argument("--quick", action="store_true", help="headline number only: skip M sweep, GEMM, LM head, CPU")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["gemm", "lm_head", "ceilings", "sweep", "backend", "prefill_ffn"], help="one secondary figure alone (for profiling runs)")
+    ap.add_argument("--only", choices=["gemm", "lm_head", "ceilings", "sweep", "backend", "prefill_ffn", "row_lengths"], help="one secondary figure alone (for profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's throughput; run with --gpus 1 "
@@ -703,6 +734,9 @@ def main():
     if args.only == "backend":
         lb = sum(w_bytes(r, c) for _, r, c in BackendSteps.SHAPES)
         print(json.dumps({"through_hip_q8_backend": bench_backend_layers(synth, args.copies, max(args.steps // 2, 300), lb)}))
+        return
+    if args.only == "row_lengths":
+        print(json.dumps({"gemv_m1_by_row_length_n5120": bench_row_length_sweep(q8mi, hip, synth)}))
         return
     if args.only == "prefill_ffn":
         print(json.dumps({"prefill_ffn_block": {f"m{m}": bench_prefill_ffn(q8mi, hip, synth, m=m, reps=r)
@@ -780,6 +814,7 @@ def main():
     if not args.quick:
         result["config0_gemv_m1"] = bench_config0(q8mi, hip, synth)
         result["hbm_read_probe_gbps"] = bench_read_probe(synth, hip)
+        result["gemv_m1_by_row_length_n5120"] = bench_row_length_sweep(q8mi, hip, synth)
         result["gemm_int8"] = bench_gemm(q8mi, hip, synth)
         ceil = bench_mfma_ceilings(synth, hip)
         for v in result["gemm_int8"].values():

@@ -98,12 +98,12 @@ int q8mi_gemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uint
  * The results of q8mi_quantize_q8_1 followed by the matching q8mi_gemv* call,
  * in one launch: every workgroup quantizes the fp32 activations
  * (x: [batch][stride_x_row] floats) itself with the quantizer's own arithmetic
- * behind its first weight requests (rows of 4096 / 5120 / 6144 / 8192 columns:
+ * behind its first weight requests (rows of 4096 / 5120 / 6144 / 7168 / 8192 columns:
  * each wave the 1024 columns it works on, in registers; other lengths: into
  * LDS), so no Q8_1 scratch buffer and no quantizer launch are needed.  The
  * quantized values and the per-block products are the same bits as in the
  * two-step form.  So are the outputs at batch 1 for rows of up to 8192 columns
- * and at batch 2 for the four row lengths above; longer rows, and other lengths
+ * and at batch 2 for the five row lengths above; longer rows, and other lengths
  * at batch 2 (where the Q8_1 entry points may run another kernel), add the same
  * products in another order (inside the GEMV's tolerance).  This is what
  * the reference's operators do in two steps (src/kernels_cuda.cu:10764-10888,
@@ -266,7 +266,13 @@ int q8mi_get_rows(const uint8_t *weight, const uint64_t *row_ids, uint32_t batch
 
 /* ---- argmax -------------------------------------------------------------- */
 /* replaces argmax_kernel, src/kernels_cuda.cu:1693-1734 (launched at :20759):
- * out2[0] = index (-1 if no element is above -inf), out2[1] = bits of the max. */
+ * out2[0] = index (-1 if no element is above -inf), out2[1] = bits of the max.
+ * Rows of 32768 elements and more (a vocabulary) are scanned by up to 128 workgroups whose
+ * partial winners meet in a 1 KiB array the library holds in every GPU's memory (two launches;
+ * the reference's single workgroup reads such a row at one CU's bandwidth).  This and
+ * q8mi_argmax_to_pair share that array: calls on such rows that overlap on one GPU (two streams,
+ * two threads) must be serialised by the caller.  The first such call on a device looks the
+ * array's address up: make it outside a graph capture. */
 int q8mi_argmax(const float *x, uint64_t n, int32_t *out2, void *stream);
 /* replaces argmax_pair_kernel, src/kernels_cuda.cu:1804-1857 (launched :20787) */
 int q8mi_argmax_to_pair(const float *x, uint64_t n, q8mi_argmax_pair *out, uint32_t out_index,
@@ -309,7 +315,9 @@ int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y_q8_1, uint32
  * partials go to a 64 KiB array the library holds in every GPU's memory from load to exit
  * (8 verify rows x 1024 workgroups, the most any call needs; a shape that would need more is
  * Q8MI_REJECTED).  The call allocates and frees nothing.  Its first call on a device looks the
- * array's address up (make that call outside a capture).  Every call on one GPU uses that GPU's
+ * array's address up, and the first call of every (rows, cols, batch) combination asks the runtime
+ * for the LDS grant and the occupancy of the kernel instantiation it picks: make one eager call
+ * of each combination that will be captured before capturing it.  Every call on one GPU uses that GPU's
  * one array: calls that overlap on the same GPU (two streams, two threads) race on it and must be
  * serialised by the caller; nothing in it needs clearing between calls. */
 int q8mi_lm_head_argmax_accept_static(const uint8_t *weight, const void *y_q8_1, uint32_t rows, uint32_t cols,

@@ -6,8 +6,17 @@
 // The batched pair keeps the reference's reduction network (a 256-wide and a
 // 1024-wide LDS tree comparing slot t with slot t+stride) so that rows holding
 // NaN resolve to the same element as the reference's kernels.
+#include <mutex>
+
 #include "q8mi_device.hpp"
 #include "q8mi_internal.hpp"
+
+// Partial results of the single-row argmax of a long row (one per first-stage workgroup): a row of
+// a vocabulary's length is more than one CU reads quickly, and the reference's entry points for a
+// single row carry no scratch argument (src/kernels_cuda.cu:20750-20790).  Every GPU holds its own
+// copy; host code uses the address hipGetSymbolAddress returns for the current device.
+constexpr unsigned kArgmaxSplitGroups = 128;
+static __device__ __align__(256) q8mi_argmax_pair argmax_split_partials[kArgmaxSplitGroups];
 
 namespace q8mi {
 namespace {
@@ -79,6 +88,131 @@ __device__ __forceinline__ Best single_row_scan(const float *__restrict__ x, uin
         __syncthreads();
     }
     return Best{sv[0], si[0]};
+}
+
+// ---- long single rows: two stages ---------------------------------------------------------------
+// Stage 1: workgroup g scans elements [g * span, (g + 1) * span) (span a multiple of 4, so that a
+// 16-byte aligned row stays aligned) with the single-row rule and leaves its winner in partial[g];
+// stage 2: one workgroup merges the partials with the same rule.  NaN never wins a `>` and equal
+// values go to the lower index at every merge, so the result is that of the one-workgroup scan.
+constexpr uint32_t kSplitThreads = 256;
+constexpr uint64_t kSplitFrom = 32768;   // shorter rows: one workgroup (a second launch costs more than it saves)
+
+__global__ __launch_bounds__(kSplitThreads) void argmax_split_stage1(const float *__restrict__ x, uint64_t n, uint64_t span,
+                                                                   q8mi_argmax_pair *__restrict__ partial) {
+    const uint64_t lo = blockIdx.x * span, hi = lo + span < n ? lo + span : n;
+    Best b{-INFINITY, -1};
+    if (reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        const uint64_t c0 = lo / 4, c1 = hi / 4;   // whole float4 chunks of the range (lo is a multiple of 4)
+        const float4 *x4 = reinterpret_cast<const float4 *>(x);
+        for (uint64_t c = c0 + threadIdx.x; c < c1; c += kSplitThreads) {
+            const float4 q = x4[c];
+            const int i = static_cast<int>(c * 4);
+            if (q.x > b.v) { b.v = q.x; b.i = i; }
+            if (q.y > b.v) { b.v = q.y; b.i = i + 1; }
+            if (q.z > b.v) { b.v = q.z; b.i = i + 2; }
+            if (q.w > b.v) { b.v = q.w; b.i = i + 3; }
+        }
+        for (uint64_t i = c1 * 4 + threadIdx.x; i < hi; i += kSplitThreads) {   // the row's last n % 4 elements
+            const float v = x[i];
+            if (v > b.v) { b.v = v; b.i = static_cast<int>(i); }
+        }
+    } else {
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += kSplitThreads) {
+            const float v = x[i];
+            if (v > b.v) { b.v = v; b.i = static_cast<int>(i); }
+        }
+    }
+    __shared__ float sv[kSplitThreads];
+    __shared__ int si[kSplitThreads];
+    sv[threadIdx.x] = b.v;
+    si[threadIdx.x] = b.i;
+    __syncthreads();
+    for (uint32_t stride = kSplitThreads / 2; stride > 0; stride >>= 1) {
+        if (threadIdx.x < stride) {
+            const float ov = sv[threadIdx.x + stride];
+            const int oi = si[threadIdx.x + stride];
+            if (beats_single(ov, oi, sv[threadIdx.x], si[threadIdx.x])) { sv[threadIdx.x] = ov; si[threadIdx.x] = oi; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partial[blockIdx.x].value = sv[0];
+        partial[blockIdx.x].index = si[0];
+    }
+}
+
+// out2 != nullptr: {index, bits of the value}; else pair_out[out_index] = {value, index}
+__global__ __launch_bounds__(kArgmaxSplitGroups) void argmax_split_stage2(const q8mi_argmax_pair *__restrict__ partial,
+                                                                        uint32_t groups, int32_t *__restrict__ out2,
+                                                                        q8mi_argmax_pair *__restrict__ pair_out,
+                                                                        uint32_t out_index) {
+    __shared__ float sv[kArgmaxSplitGroups];
+    __shared__ int si[kArgmaxSplitGroups];
+    float v = -INFINITY;
+    int i = -1;
+    if (threadIdx.x < groups) {
+        v = partial[threadIdx.x].value;
+        i = partial[threadIdx.x].index;
+    }
+    sv[threadIdx.x] = v;
+    si[threadIdx.x] = i;
+    __syncthreads();
+    for (uint32_t stride = kArgmaxSplitGroups / 2; stride > 0; stride >>= 1) {
+        if (threadIdx.x < stride) {
+            const float ov = sv[threadIdx.x + stride];
+            const int oi = si[threadIdx.x + stride];
+            if (beats_single(ov, oi, sv[threadIdx.x], si[threadIdx.x])) { sv[threadIdx.x] = ov; si[threadIdx.x] = oi; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        if (out2 != nullptr) {
+            out2[0] = si[0];
+            out2[1] = __builtin_bit_cast(int32_t, sv[0]);
+        } else {
+            pair_out[out_index].value = sv[0];
+            pair_out[out_index].index = si[0];
+        }
+    }
+}
+
+// This device's copy of the partials array (looked up once per device, with that device current).
+int split_partials_of_current_device(q8mi_argmax_pair **out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *ptr_of[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return fail(Q8MI_LAUNCH_ERROR, "argmax: no current device, or a device id beyond %d", kMaxDevices - 1);
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr_of[dev] == nullptr) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_split_partials));
+        if (e != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return fail(Q8MI_LAUNCH_ERROR, "argmax: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        }
+        ptr_of[dev] = p;
+    }
+    *out = static_cast<q8mi_argmax_pair *>(ptr_of[dev]);
+    return Q8MI_OK;
+}
+
+int launch_split(const float *x, uint64_t n, int32_t *out2, q8mi_argmax_pair *pair_out, uint32_t out_index,
+                 hipStream_t stream) {
+    q8mi_argmax_pair *partial = nullptr;
+    if (int rc = split_partials_of_current_device(&partial)) return rc;
+    // at least 2048 elements per workgroup, in whole float4 chunks
+    uint64_t span = (n + kArgmaxSplitGroups - 1) / kArgmaxSplitGroups;
+    span = span < 2048 ? 2048 : (span + 3) / 4 * 4;
+    const uint32_t groups = static_cast<uint32_t>((n + span - 1) / span);
+    argmax_split_stage1<<<groups, kSplitThreads, 0, stream>>>(x, n, span, partial);
+    if (int rc = check_launch("argmax stage 1")) return rc;
+    argmax_split_stage2<<<1, kArgmaxSplitGroups, 0, stream>>>(partial, groups, out2, pair_out, out_index);
+    return check_launch("argmax stage 2");
 }
 
 __global__ __launch_bounds__(kRowThreads) void argmax_kernel(const float *__restrict__ x, uint64_t n,
@@ -162,12 +296,14 @@ __global__ __launch_bounds__(kStage2Block) void argmax_rows_stage2(const q8mi_ar
 using namespace q8mi;
 
 extern "C" int q8mi_argmax(const float *x, uint64_t n, int32_t *out2, void *stream) {
+    if (n >= kSplitFrom && n <= 0x7fffffffull) return launch_split(x, n, out2, nullptr, 0, as_stream(stream));
     argmax_kernel<<<1, kRowThreads, 0, as_stream(stream)>>>(x, n, out2);
     return check_launch("argmax");
 }
 
 extern "C" int q8mi_argmax_to_pair(const float *x, uint64_t n, q8mi_argmax_pair *out, uint32_t out_index,
                                 void *stream) {
+    if (n >= kSplitFrom && n <= 0x7fffffffull) return launch_split(x, n, nullptr, out, out_index, as_stream(stream));
     argmax_pair_kernel<<<1, kRowThreads, 0, as_stream(stream)>>>(x, n, out, out_index);
     return check_launch("argmax_pair");
 }

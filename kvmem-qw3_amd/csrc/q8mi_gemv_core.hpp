@@ -41,10 +41,7 @@ template <int M>
 struct RowsPerUnit {
     static constexpr int value = M >= 4 ? 4 : 2;
 };
-#ifndef Q8MI_GEMV_DEPTH
-#define Q8MI_GEMV_DEPTH 2
-#endif
-constexpr int kDepth = Q8MI_GEMV_DEPTH;        // items in flight per wave
+constexpr int kDepth = 2;                       // items in flight per wave
 constexpr uint32_t kLdsLimit = 160u * 1024u;    // LDS per CU on gfx950
 constexpr uint32_t kParkFloats = 1024;           // per-wave LDS area (floats) for the sums of the units it touched
 
@@ -443,19 +440,20 @@ constexpr uint32_t kMfmaFromBatch = 2;    // smallest batch served by the matrix
 constexpr uint32_t kPairsMaxBatch = 4;    // largest batch the row-pair family serves
 // Which GEMV family serves a launch of batch 2 and more (measured on MI355X, row-pair kernel with
 // the rows shared by the waves of a workgroup against matrix-core kernel, us):
-//   rows of 4, 5, 6 or 8 KiB   batch 2: always row pairs (8192 x 5120 fan-out 9.3 / 11.9, SwiGLU 30.2 / 34.1);
+//   rows of 4 .. 8 KiB         batch 2: always row pairs (8192 x 5120 fan-out 9.3 / 11.9, SwiGLU 30.2 / 34.1);
 //                              batch 3: row pairs (fan-out 10.0 / 11.9, 5120 x 6144 9.2 / 10.3, SwiGLU 32.0 / 33.9);
 //                              batch 4: row pairs but for the SwiGLU form (fan-out 10.8 / 11.7, 5120 x 6144
 //                              10.2 / 10.2, SwiGLU 33.7 / 33.7 at best); from batch 5 the dot products bind
 //                              (batch 6: 13.1 / 12.3 on the fan-out)
-//   rows of 17 KiB             batch 2: row pairs (5120 x 17408: 18.8 / 20.0); batch 3 and 4: 22.4 / 20.3, 30.0 / 20.6
+//   rows of 9 .. 17 KiB        batch 2: row pairs (5120 x 17408: 18.8 / 20.0); batch 3 and 4: 22.4 / 20.3, 30.0 / 20.6
 //   any other length           batch 2 with 8192 row pairs or more: row pairs (ring kernel); else matrix cores
 // nb: blocks per row; silu: the SwiGLU form.
 inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch, uint32_t nb, bool silu) {
     if (batch < 2) return false;
     if (batch > kPairsMaxBatch) return true;
-    const bool short_rows = nb == 128 || nb == 160 || nb == 192 || nb == 256;
-    if (batch == 2) return !short_rows && nb != 544 && row_pairs < 8192;
+    const bool short_rows = nb % 32 == 0 && nb >= 128 && nb <= 256;   // 4 .. 8 KiB
+    const bool whole_kib = nb % 32 == 0 && nb >= 128 && nb <= 544;     // 4 .. 17 KiB: a shared-row kernel of its own
+    if (batch == 2) return !whole_kib && row_pairs < 8192;
     if (batch == 3) return !short_rows;
     return !short_rows || silu;
 }

@@ -19,12 +19,12 @@
 // over the lanes of equal parity lane 0 holds the first row's result and lane 1 the second's.
 //
 // Two kernels, by where the activations live:
-//   gemv_pairs_ksplit_kernel   rows of 4, 5, 6, 8 and 17 KiB: the waves of a workgroup cut every row
+//   gemv_pairs_ksplit_kernel   rows of 4 to 17 KiB (whole KiB): the waves of a workgroup cut every row
 //       into interleaved 1 KiB steps, so each wave needs the activations of its own steps only,
 //       loads them once into registers (5 per step and activation row) and keeps them for all
 //       pairs of the workgroup; partial sums meet in LDS after the last pair.  With fp32
 //       activations (the entry points that quantize inside the GEMV, optionally after an RMS norm;
-//       one row of 4..8 KiB) every wave quantizes the 1024 floats of its own step in registers,
+//       rows of 4..8 KiB) every wave quantizes the 1024 floats of its own step in registers,
 //       with the stand-alone quantizer's arithmetic; only the norm's sum of squares crosses the
 //       waves, through LDS, in the stand-alone norm's order
 //   gemv_pairs_ring_kernel     any other row length: one wave per pair, the activation bytes of a
@@ -309,9 +309,16 @@ __global__ __launch_bounds__(XF32 ? 512 : kWave) void gemv_pairs_ring_kernel(con
 // SwiGLU with the norm inside 36.3 -> 31.5 us, fan-out 11.4 -> 11.1, 5120 x 6144 9.3 -> 8.4.
 constexpr uint32_t kKsplitMaxPairs = 12;   // pairs a workgroup may take (its partial sums wait in LDS)
 
+// Register slots a wave of the shared-row kernel holds: its whole steps plus one for a shared last step.
+constexpr int ksplit_slots(int nsteps, int waves) { return nsteps / waves + (nsteps % waves ? 1 : 0); }
+// Waves per SIMD the registers are budgeted for: three at batch 2, which also serves the long rows;
+// four for the SwiGLU form on rows of four slots and more (five would spill); five otherwise.
+constexpr int ksplit_waves_per_simd(int m, int nsteps, int waves, bool silu) {
+    return m == 2 ? 3 : (silu && ksplit_slots(nsteps, waves) >= 4) ? 4 : 5;
+}
+
 template <int M, int NSTEPS, int WAVES, bool SILU = false, bool XF32 = false, bool NORM = false>
-// (waves per SIMD the registers are budgeted for: three at batch 2, which also serves the 17 KiB rows; five otherwise)
-__global__ __launch_bounds__(WAVES * kWave, M == 2 ? 3 : 5) void gemv_pairs_ksplit_kernel(const GemvParams p, const PairSpace ps) {
+__global__ __launch_bounds__(WAVES * kWave, ksplit_waves_per_simd(M, NSTEPS, WAVES, SILU)) void gemv_pairs_ksplit_kernel(const GemvParams p, const PairSpace ps) {
     constexpr uint32_t nb = NSTEPS * 32;
     constexpr uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
     constexpr int S = NSTEPS / WAVES;                              // whole steps per wave
@@ -509,7 +516,7 @@ int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     // four 29.4; fan-out (4096 pairs) one 8.7, two 9.0, four 9.0.  At batch 2: SwiGLU two 30.8, four 30.2;
     // fan-out two 9.5, four 9.3; 5120 x 6144 (2560 pairs) two 8.0, four 8.2.  At batch 3: SwiGLU four 32.7,
     // eight 32.0; 5120 x 6144 four 9.2, eight 10.8.
-    if (NSTEPS >= 17) ps.ppw = 2;
+    if (NSTEPS / WAVES >= 3) ps.ppw = 2;   // rows of three and more steps per wave (15 and 17 KiB)
     else if (M == 1) ps.ppw = ps.pairs >= 8192 ? 2 : 1;
     else if (M == 2) ps.ppw = ps.pairs >= 4096 ? 4 : 2;
     else ps.ppw = ps.pairs >= 8192 ? 8 : 4;
@@ -610,6 +617,56 @@ int launch_ring_f32(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     return launch(gemv_pairs_ring_kernel<M, false, true>);
 }
 
+// Rows that are not a whole number of KiB: one wave per pair at batch 1 and 2 (the ring kernel when
+// the launch has row pairs enough to fill the chip that way is the caller's rule), else not ours.
+template <int M>
+int ring_or_reject(const GemvParams &p, const PairSpace &ps, hipStream_t stream) {
+    if constexpr (M <= 2) return launch_ring<M>(p, ps, stream);
+    else return Q8MI_REJECTED;
+}
+
+// Rows of N KiB, N = 4 .. 17 (the reference's kernel is generic in cols % 32, src/mmvq_q8.cu:193-280;
+// here every whole number of KiB from 4 on has an instantiation of the shared-row kernel; shorter
+// rows are launches of a few microseconds whatever reads them), always a split without a left-over
+// step except at 17: one wave per 1 KiB step up to 8 KiB and at 9, 11 and 13; two steps per wave at
+// 10, 12, 14 and 16; 15 -> 5 x 3; 17 -> 4 x 4 and a shared last step.  Measured on MI355X at batch 1,
+// 5120 rows, time / plain streaming read of the same bytes: 1.08 .. 1.17 on every length (with four
+// waves and a shared last step 9, 11 and 13 KiB were at 1.30, 1.22, 1.22; 15 KiB on 15 waves 1.28, on
+// 8 waves 1.23; the ring kernel on lengths in between, 5632 and 9728 columns: 1.29, 1.22).
+// Q8MI_REJECTED: not a length (or batch) of this kernel.
+template <int M>
+int ksplit_by_length(const GemvParams &p, const PairSpace &ps, hipStream_t stream) {
+    if (p.nb % 32 != 0) return ring_or_reject<M>(p, ps, stream);
+    if constexpr (M >= 3) {   // batch 3 and 4: the 4..8 KiB rows only (longer rows: the matrix-core kernel)
+        switch (p.nb / 32) {
+            case 4: return launch_ksplit<M, 4, 4>(p, ps, stream);
+            case 5: return launch_ksplit<M, 5, 5>(p, ps, stream);
+            case 6: return launch_ksplit<M, 6, 6>(p, ps, stream);
+            case 7: return launch_ksplit<M, 7, 7>(p, ps, stream);
+            case 8: return launch_ksplit<M, 8, 8>(p, ps, stream);
+            default: return Q8MI_REJECTED;
+        }
+    } else {
+        switch (p.nb / 32) {
+            case 4: return launch_ksplit<M, 4, 4>(p, ps, stream);
+            case 5: return launch_ksplit<M, 5, 5>(p, ps, stream);
+            case 6: return launch_ksplit<M, 6, 6>(p, ps, stream);
+            case 7: return launch_ksplit<M, 7, 7>(p, ps, stream);
+            case 8: return launch_ksplit<M, 8, 8>(p, ps, stream);
+            case 9: return launch_ksplit<M, 9, 9>(p, ps, stream);
+            case 10: return launch_ksplit<M, 10, 5>(p, ps, stream);
+            case 11: return launch_ksplit<M, 11, 11>(p, ps, stream);
+            case 12: return launch_ksplit<M, 12, 6>(p, ps, stream);
+            case 13: return launch_ksplit<M, 13, 13>(p, ps, stream);
+            case 14: return launch_ksplit<M, 14, 7>(p, ps, stream);
+            case 15: return launch_ksplit<M, 15, 5>(p, ps, stream);
+            case 16: return launch_ksplit<M, 16, 8>(p, ps, stream);
+            case 17: return launch_ksplit<M, 17, 4>(p, ps, stream);   // two waves spill, eight: 17.1 us against 16.9
+            default: return ring_or_reject<M>(p, ps, stream);
+        }
+    }
+}
+
 }  // namespace
 
 int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
@@ -637,6 +694,7 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
                 case 4096: return launch_ksplit_f32<M, 4>(p, ps, stream);
                 case 5120: return launch_ksplit_f32<M, 5>(p, ps, stream);
                 case 6144: return launch_ksplit_f32<M, 6>(p, ps, stream);
+                case 7168: return launch_ksplit_f32<M, 7>(p, ps, stream);
                 case 8192: return launch_ksplit_f32<M, 8>(p, ps, stream);
                 default: return launch_ring_f32<M>(p, ps, stream);
             }
@@ -648,37 +706,14 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         }
     }
     if (reinterpret_cast<uintptr_t>(p.y) % 4 != 0) return Q8MI_REJECTED;
-    // rows of 4, 5, 6, 8 and 17 KiB: shared by the waves of a workgroup, activations in registers;
+    // rows of whole KiB up to 17: shared by the waves of a workgroup, activations in registers
+    // (batch 1 and 2 on every such length, batch 3 and 4 on the 4..8 KiB rows measured for them);
     // any other length: one wave per pair, activations read with every step
-    if (batch == 1) {
-        switch (cols) {
-            case 4096: return launch_ksplit<1, 4, 4>(p, ps, stream);
-            case 5120: return launch_ksplit<1, 5, 5>(p, ps, stream);
-            case 6144: return launch_ksplit<1, 6, 6>(p, ps, stream);
-            case 8192: return launch_ksplit<1, 8, 8>(p, ps, stream);
-            case 17408: return launch_ksplit<1, 17, 4>(p, ps, stream);   // two waves spill, eight: 17.1 us against 16.9
-            default: return launch_ring<1>(p, ps, stream);
-        }
-    }
-    auto by_cols = [&](auto mtag) -> int {
-        constexpr int M = decltype(mtag)::value;
-        switch (cols) {
-            case 4096: return launch_ksplit<M, 4, 4>(p, ps, stream);
-            case 5120: return launch_ksplit<M, 5, 5>(p, ps, stream);
-            case 6144: return launch_ksplit<M, 6, 6>(p, ps, stream);
-            case 8192: return launch_ksplit<M, 8, 8>(p, ps, stream);
-            default: break;
-        }
-        if constexpr (M == 2) {
-            if (cols == 17408) return launch_ksplit<2, 17, 4>(p, ps, stream);   // 18.8 us at 5120 x 17408 against 20.0 on the matrix cores
-            return launch_ring<2>(p, ps, stream);
-        }
-        return Q8MI_REJECTED;   // batch 3 and 4 on other lengths: the matrix-core kernel
-    };
     switch (batch) {
-        case 2: return by_cols(std::integral_constant<int, 2>{});
-        case 3: return by_cols(std::integral_constant<int, 3>{});
-        case 4: return by_cols(std::integral_constant<int, 4>{});
+        case 1: return ksplit_by_length<1>(p, ps, stream);
+        case 2: return ksplit_by_length<2>(p, ps, stream);
+        case 3: return ksplit_by_length<3>(p, ps, stream);
+        case 4: return ksplit_by_length<4>(p, ps, stream);
         default: return Q8MI_REJECTED;
     }
 }

@@ -34,8 +34,12 @@ struct Drafts {
     int32_t v[kMaxDrafts];
 };
 
+// Whether candidate (ov, oi) replaces (v, i).  Only a value above -inf is a candidate at all (a NaN
+// or -inf logit never wins, and a row with no other logits ends as (-inf, -1): the single-row rule
+// of the reference's argmax_kernel), so the winner is the largest candidate, the lowest index among
+// equals, in whatever order lanes, waves and workgroups meet and merge them.
 __device__ __forceinline__ bool beats(float ov, int oi, float v, int i) {
-    if (oi < 0) return false;
+    if (oi < 0 || !(ov > -INFINITY)) return false;
     if (i < 0) return true;
     if (ov > v) return true;
     return ov == v && oi < i;

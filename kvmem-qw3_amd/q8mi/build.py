@@ -29,21 +29,13 @@ FLAGS = [
 ]
 
 
-def build(verbose=False, save_temps_dir=None, defines=(), out_path=None, obj_dir=None):
-    """Compile every source and link the shared library.  Always recompiles.
-    `defines`, `out_path` and `obj_dir` exist for tuning builds of variants."""
-    objs = []
-    out_path = out_path or LIB_PATH
-    obj_dir = obj_dir or CSRC
-    os.makedirs(obj_dir, exist_ok=True)
+def build(verbose=False):
+    """Compile every source and link the shared library.  Always recompiles."""
 
     def compile_one(src):
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        cmd = [HIPCC, *FLAGS, *[f"-D{d}" for d in defines], "-c", os.path.join(CSRC, src), "-o", obj]
-        if save_temps_dir:
-            os.makedirs(save_temps_dir, exist_ok=True)
-            cmd += [f"-save-temps={'obj'}"]
-        r = subprocess.run(cmd, capture_output=True, text=True, cwd=save_temps_dir or CSRC)
+        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        r = subprocess.run(cmd, capture_output=True, text=True, cwd=CSRC)
         out = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
                         if "packed-fp32-ops" not in l and "is not a recognized feature" not in l
                         and "loop not unrolled" not in l)
@@ -55,11 +47,11 @@ def build(verbose=False, save_temps_dir=None, defines=(), out_path=None, obj_dir
 
     with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as ex:
         objs = list(ex.map(compile_one, SOURCES))
-    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out_path, *objs, "-lpthread"]
+    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs, "-lpthread"]
     r = subprocess.run(link, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
-    return out_path
+    return LIB_PATH
 
 
 if __name__ == "__main__":

@@ -343,9 +343,11 @@ int q8o_gemv_abs(const uint8_t *w, const uint8_t *y, float *dst, uint32_t rows, 
                  uint32_t batch, uint32_t stride_dst_row) {
     if (!gemv_shape_ok(cols, batch)) return -1;
     const uint32_t nb = cols / Q8O_QK;
-    for (uint32_t r = 0; r < rows; ++r)
+    int64_t r;   /* rows are independent: tall matrices (a vocabulary) are split over the cores */
+#pragma omp parallel for schedule(static) if (rows >= 8192)
+    for (r = 0; r < (int64_t)rows; ++r)
         for (uint32_t j = 0; j < batch; ++j)
-            dst[(uint64_t)j * stride_dst_row + r] = gemv_one_abs(w, y, nb, r, j);
+            dst[(uint64_t)j * stride_dst_row + (uint64_t)r] = gemv_one_abs(w, y, nb, (uint32_t)r, j);
     return 0;
 }
 

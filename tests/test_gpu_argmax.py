@@ -36,7 +36,7 @@ def adversarial_rows(n, seed):
     return np.stack(rows)
 
 
-@pytest.mark.parametrize("n", [1, 31, 256, 1024, 1025, 248320])
+@pytest.mark.parametrize("n", [1, 31, 256, 1024, 1025, 32767, 32768, 32771, 248320, 262147])
 def test_argmax_single_row(gpu, oracle, n):
     rows = adversarial_rows(n, seed=n)
     L = q8mi.lib()
@@ -206,29 +206,26 @@ def full_head(gpu):
 
 @pytest.mark.parametrize("batch", [1, 2, 4, 6, 8])
 def test_lm_head_full_vocabulary(gpu, oracle, full_head, batch):
-    """At the model's size the oracle does not run the whole head in seconds, so: (1) the plain GEMV's
-    logits are held against the oracle on a seeded sample of rows plus every winning row, (2) the
-    oracle's argmax of those logits is the expected token of each verify row, (3) the fused head must
-    return those tokens and the accept length of every forced-match prefix."""
+    """The model's LM head.  The oracle runs the whole 248 320 x 5120 head (row-parallel, well under
+    a second per activation row): (1) its argmax is the expected token of each verify row, (2) the
+    plain GEMV's logits and the fused head's own optional logits are held against it on every row,
+    (3) the fused head must return those tokens and the accept length of every forced-match prefix."""
     L = gpu.lib()
     w, dw = full_head
     x = synth.normal(batch, FULL_COLS, seed=700 + batch)
     dy, y = quantize_q8_1(x)
+    rc, ref = oracle.gemv(w, y, FULL_VOCAB, FULL_COLS, batch, threads=16)
+    rc, absum = oracle.gemv_abs(w, y, FULL_VOCAB, FULL_COLS, batch)
+    ref_pairs = oracle.argmax_rows_scan(ref, batch, FULL_VOCAB)
+    tokens = ref_pairs["index"]
+    # top-2 gaps of this seed are far above the fp32 tolerance, so the tokens are unambiguous
+    top2 = np.partition(ref, -2, axis=1)[:, -2:]
+    assert np.all(top2[:, 1] - top2[:, 0] > 1e-4 * np.abs(top2[:, 1]))
     logits_dev = hip.DeviceBuffer(4 * batch * FULL_VOCAB)
     ok(L.q8mi_gemv(dw.ptr, dy.ptr, logits_dev.ptr, FULL_VOCAB, FULL_COLS, batch, FULL_VOCAB, NULL), "gemv")
     hip.synchronize()
-    logits = logits_dev.download(np.float32).reshape(batch, FULL_VOCAB)
-    ref_pairs = oracle.argmax_rows_scan(logits, batch, FULL_VOCAB)
-    tokens = ref_pairs["index"]
+    assert_close_fp32(logits_dev.download(np.float32), ref, absum, "LM-head logits, plain GEMV, every row")
     rng = np.random.default_rng(batch)
-    sample = np.unique(np.concatenate([rng.integers(0, FULL_VOCAB, 3000), tokens, [0, FULL_VOCAB - 1]]))
-    sub = np.ascontiguousarray(w[sample])
-    rc, ref = oracle.gemv(sub, y, sample.size, FULL_COLS, batch, threads=8)
-    rc, absum = oracle.gemv_abs(sub, y, sample.size, FULL_COLS, batch)
-    assert_close_fp32(logits[:, sample], ref, absum, "LM-head logits on sampled rows")
-    # top-2 gaps of this seed are far above the fp32 tolerance, so the tokens are unambiguous
-    top2 = np.partition(logits, -2, axis=1)[:, -2:]
-    assert np.all(top2[:, 1] - top2[:, 0] > 1e-4 * np.abs(top2[:, 1]))
     for prefix in sorted({0, batch // 2, batch - 1}):
         drafts = rng.integers(0, FULL_VOCAB, batch - 1).astype(np.int32)
         drafts[:prefix] = tokens[:prefix]
@@ -236,8 +233,57 @@ def test_lm_head_full_vocabulary(gpu, oracle, full_head, batch):
             drafts[prefix] = (drafts[prefix] + 1) % FULL_VOCAB
         exp_len, exp_next = oracle.accept(tokens, drafts, eos=2)
         assert exp_len == prefix
-        pairs, n_acc, nxt, _ = run_lm_head(dw, dy, FULL_VOCAB, FULL_COLS, batch, drafts, 2, on_device=(prefix % 2 == 1))
+        pairs, n_acc, nxt, lg = run_lm_head(dw, dy, FULL_VOCAB, FULL_COLS, batch, drafts, 2, want_logits=(prefix == 0),
+                                            on_device=(prefix % 2 == 1))
         assert np.array_equal(pairs["index"], tokens), "row argmax tokens differ"
         assert n_acc == exp_len and nxt == exp_next
-        want = logits[np.arange(batch), tokens]
-        assert np.all(np.abs(pairs["value"] - want) <= 1e-5 * np.abs(want) + 1e-6)
+        want = ref[np.arange(batch), tokens]
+        assert np.all(np.abs(pairs["value"] - want) <= 1e-5 * np.abs(want) + 1e-6 * absum[np.arange(batch), tokens])
+        if lg is not None:
+            assert_close_fp32(lg, ref, absum, "LM-head logits, fused head, every row")
+            assert np.array_equal(pairs["value"].view(np.uint32), lg[np.arange(batch), tokens].view(np.uint32))
+
+
+@pytest.mark.parametrize("batch", [2, 4, 7])
+def test_lm_head_rows_without_a_number(gpu, oracle, batch):
+    """Logits that are NaN never win and a verify row with nothing above -inf has no token (-1, read
+    as eos by the accept rule), whichever lane, wave or workgroup meets them first: weight rows
+    with a NaN scale at both ends and in the middle of the vocabulary, and one activation row whose
+    every block scale is NaN.  Batch 2 runs the dot-product kernel, 4 and 7 the matrix-core one."""
+    vocab, cols, eos = 20000, 1024, 3
+    dead = batch - 2                       # the activation row whose logits are all NaN
+    w = synth.q8_0_weight(vocab, cols, seed=31).copy()
+    x = synth.normal(batch, cols, seed=32 + batch)
+    dy, y = quantize_q8_1(x)
+    y = y.copy()
+    nb = cols // 32
+    rc, clean = oracle.gemv(w, y, vocab, cols, batch)
+    tops = [int(np.argmax(clean[j])) for j in range(batch)]
+    nan_rows = sorted({0, 1, 63, 64, 4095, 4096, 9999, vocab - 2, vocab - 1, tops[0], tops[-1]})
+    nan16 = np.frombuffer(np.uint16(0x7e00).tobytes(), np.uint8)
+    wv = w.reshape(vocab, nb * 34)
+    for r in nan_rows:
+        wv[r, 0:2] = nan16                 # fp16 NaN scale of the row's first block
+    y.reshape(batch, nb, 36)[dead, :, 0:2] = nan16
+    dw, dyp = dev(w), dev(y)
+    rc, logits = oracle.gemv(w, y, vocab, cols, batch)
+    assert np.isnan(logits[:, nan_rows]).all() and np.isnan(logits[dead]).all()
+    want_tok, want_val = [], []
+    for j in range(batch):
+        row = np.where(np.isnan(logits[j]), -np.inf, logits[j])
+        t = int(np.argmax(row)) if np.isfinite(row).any() else -1
+        want_tok.append(t)
+        want_val.append(row[t] if t >= 0 else -np.inf)
+    assert want_tok[dead] == -1 and want_tok[-1] != tops[-1]
+    live = [j for j in range(batch) if j != dead]
+    for prefix in sorted({0, dead, batch - 1}):
+        drafts = np.array([(t if t >= 0 else eos) for t in want_tok[:batch - 1]], np.int32)
+        if prefix < batch - 1:
+            drafts[prefix] = (drafts[prefix] + 1) % vocab
+        for on_device in (False, True):
+            pairs, n_acc, nxt, _ = run_lm_head(dw, dyp, vocab, cols, batch, drafts, eos, on_device=on_device)
+            assert list(pairs["index"]) == want_tok
+            assert pairs["value"][dead] == -np.inf
+            assert np.allclose(pairs["value"][live], np.array(want_val)[live], rtol=1e-5, atol=1e-6)
+            assert n_acc == prefix
+            assert nxt == (want_tok[prefix] if want_tok[prefix] >= 0 else eos)

@@ -1,7 +1,7 @@
 """GPU parity at the model's own shapes: the decode GEMV set of one layer exactly as bench.py times
 it (QKV fan-out 5120 -> 6144 + 1024 + 1024, O 6144 -> 5120 with residual, gate/up 5120 -> 17408 SwiGLU,
-down 17408 -> 5120 with residual), at M = 1 (quantizer inside the launches), 2, 3, 4, 6 and 8, against the
-CPU oracle."""
+down 17408 -> 5120 with residual), at M = 1 (quantizer inside the fan-out and O launches), 2, 3, 4, 6 and
+8, on three weight seeds, against the CPU oracle."""
 import numpy as np
 import pytest
 
@@ -17,11 +17,15 @@ SHAPES = {"q": (bench.QDIM, bench.HIDDEN), "k": (bench.KVDIM, bench.HIDDEN), "v"
           "down": (bench.HIDDEN, bench.FFN)}
 
 
-@pytest.fixture(scope="module")
-def layer(gpu):
-    dev_layer = bench.Layer(synth, hip, seed=3)
-    host = {name: synth.q8_0_weight(r, c, seed=3 * 16 + i, sigma=0.02) for i, (name, (r, c)) in enumerate(SHAPES.items())}
-    return dev_layer, host
+# three weight seeds: the benchmark definition regenerates the layer's weights per seed
+@pytest.fixture(scope="module", params=[3, 5, 11], ids=lambda s: f"seed{s}")
+def layer(gpu, request):
+    seed = request.param
+    dev_layer = bench.Layer(synth, hip, seed=seed)
+    host = {name: synth.q8_0_weight(r, c, seed=seed * 16 + i, sigma=0.02) for i, (name, (r, c)) in enumerate(SHAPES.items())}
+    yield dev_layer, host
+    for b in dev_layer.w.values():
+        b.free()
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 6, 8])
@@ -30,6 +34,7 @@ def test_decode_layer_at_model_shapes(gpu, oracle, layer, m):
     step = bench.DecodeStep(gpu, hip, m, seed=40 + m)
     hip.synchronize()
     x = step.x.download(np.float32).reshape(m, bench.HIDDEN)
+    x_ffn = step.x_ffn.download(np.float32).reshape(m, bench.HIDDEN)
     attn = step.attn.download(np.float32).reshape(m, bench.ATTN_OUT)
     h0 = step.h.download(np.float32).reshape(m, bench.HIDDEN)
     step.run(dev_layer)
@@ -45,9 +50,10 @@ def test_decode_layer_at_model_shapes(gpu, oracle, layer, m):
     for name, buf in (("q", step.q), ("k", step.k), ("v", step.v)):
         ref, mag = linear(name, yx)
         assert_close_fp32(buf.download(np.float32), ref, mag, f"{name} projection, M={m}")
-    g, gmag = linear("gate", yx)
-    u, umag = linear("up", yx)
-    rc, silu_ref = oracle.gemv_silu_mul(host["gate"], host["up"], yx, bench.FFN, bench.HIDDEN, m)
+    rc, yx_ffn = oracle.quantize_q8_1(x_ffn)
+    g, gmag = linear("gate", yx_ffn)
+    u, umag = linear("up", yx_ffn)
+    rc, silu_ref = oracle.gemv_silu_mul(host["gate"], host["up"], yx_ffn, bench.FFN, bench.HIDDEN, m)
     ffn = step.ffn.download(np.float32).reshape(m, bench.FFN)
     g64, u64 = g.astype(np.float64), u.astype(np.float64)
     sig = 1.0 / (1.0 + np.exp(-g64))

@@ -69,3 +69,58 @@ def test_static_scratch_entry_point_rejections(gpu):
     assert "batch" in q8mi.last_error()
     assert L.q8mi_lm_head_argmax_accept_static(*args(100, 500, 2)) == q8mi.REJECTED
     assert L.q8mi_lm_head_argmax_accept_static(*args(0, 512, 2)) == q8mi.REJECTED
+
+
+def mem_free():
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    hip.check(hip.rt().hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+    return free.value
+
+
+def test_static_scratch_entry_point_under_capture(gpu):
+    """After one eager call of the same shape and batch (the first launch of a kernel instantiation
+    asks the runtime for its LDS grant and occupancy), the call is captured into a HIP graph and
+    replayed with eager work of another shape in between: every replay gives the eager call's
+    bits, and the device's free memory does not change over the replays and the eager calls
+    between them (nothing is allocated)."""
+    L = q8mi.lib()
+    vocab, cols, batch = 40000, 1024, 5
+    dw = dev(synth.q8_0_weight(vocab, cols, seed=951))
+    dy, _ = quantize_q8_1(synth.normal(batch, cols, seed=952))
+    other_w = dev(synth.q8_0_weight(5000, cols, seed=953))
+    other_y, _ = quantize_q8_1(synth.normal(2, cols, seed=954))
+    drafts = np.array([1, 2, 3, 4], np.int32)
+    dptr = drafts.ctypes.data_as(C.c_void_p)
+    row_out, acc = hip.DeviceBuffer(8 * batch), hip.DeviceBuffer(8)
+    o_rows, o_acc = hip.DeviceBuffer(16), hip.DeviceBuffer(8)
+    stream = hip.Stream()
+
+    def call(s):
+        ok(L.q8mi_lm_head_argmax_accept_static(dw.ptr, dy.ptr, vocab, cols, batch, dptr, 0, 2, row_out.ptr, acc.ptr,
+                                               None, vocab, s), "lm_head static")
+
+    def other():
+        ok(L.q8mi_lm_head_argmax_accept_static(other_w.ptr, other_y.ptr, 5000, cols, 2, dptr, 0, 2, o_rows.ptr, o_acc.ptr,
+                                               None, 5000, stream.handle), "lm_head static, other shape")
+
+    call(stream.handle)
+    other()
+    stream.synchronize()
+    want_rows, want_acc = row_out.download(np.uint32).copy(), acc.download(np.int32).copy()
+    g = hip.Graph(stream)
+    with g:
+        call(stream.handle)
+    before = None
+    for rep in range(5):
+        if rep == 1:
+            before = mem_free()      # after the runtime has set the graph up with its first launch
+        row_out.fill(0xff)
+        acc.fill(0xff)
+        hip.synchronize()
+        g.launch()
+        stream.synchronize()
+        assert np.array_equal(row_out.download(np.uint32), want_rows)
+        assert np.array_equal(acc.download(np.int32), want_acc)
+        other()                      # overwrites the shared partials between replays
+        stream.synchronize()
+    assert mem_free() == before
