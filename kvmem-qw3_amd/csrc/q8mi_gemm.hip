@@ -953,11 +953,12 @@ bool uses_main_tiles(uint32_t rows, uint32_t batch) {
 int launch_gemm_dma(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, hipStream_t stream) {
     if (uses_main_tiles(rows, batch)) return launch_dma_rows<false>(c, rows, nb, batch, c.out.epi == kEpiStore, stream);
     // too few main tiles to fill the chip: 32-row tiles behind a ring of stages, as wide as the batch needs
-    // Batches of 33..64 rows on matrices tall enough for more than 1.5 32-row tiles per CU take 64-row
-    // tiles: half as many workgroups re-read the activation records of a step (measured at
-    // 17408 x 5120, batch 64: 59 -> 51 us).  The 32- and 128-row-wide tiles lose with 64 rows (54
-    // against 43 us, 88 against 77 us): their rings then leave room for one workgroup per CU only.
-    if (batch > 32 && batch <= 64 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * static_cast<uint32_t>(device_cu_count()))
+    // Batches of 33..128 rows on matrices tall enough for more than 1.5 32-row tiles per CU take
+    // 64 x 64 tiles: fewer workgroups re-read the activation records of a step (measured at
+    // 17408 x 5120: batch 64 59 -> 51 us; batch 128, two column tiles of 64 against one 32-row tile
+    // 128 wide, 75.9 -> 66.3 us).  The 32- and 128-row-wide tiles lose with 64 rows (54 against
+    // 43 us, 88 against 77 us): their rings then leave room for one workgroup per CU only.
+    if (batch > 32 && batch <= 128 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * static_cast<uint32_t>(device_cu_count()))
         return launch_ring<2, kRingWaves2, kRing2, 2>(c, rows, nb, batch, stream);
     if (batch <= 32) return launch_ring<1, 4, kRing1>(c, rows, nb, batch, stream);
     if (batch <= 64) return launch_ring<2, kRingWaves2, kRing2>(c, rows, nb, batch, stream);

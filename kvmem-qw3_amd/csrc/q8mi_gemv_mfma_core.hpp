@@ -74,6 +74,9 @@ struct MfmaItem {
 template <int MG, int THREADS, bool HS>
 struct MfmaStage {
     static constexpr uint32_t MP = 4 * MG;
+    // Blocks a thread has in flight per trip.  (Six per trip, which makes eight rows of 5120 columns
+    // one trip instead of two and eight rows of 17408 two instead of five, changed no launch by
+    // more than its run-to-run spread: the trips overlap the first weight requests.)
     static constexpr int kBatch = 2;
     struct Dwords4 {
         int x, y, z, w;

@@ -332,7 +332,7 @@ def test_gemm_medium_batches(gpu, oracle, rows, cols, batch):
     """Batches too small to fill the chip with 128 x 128 tiles run 32-row tiles behind a ring of
     LDS stages, 32, 64 or 128 activation rows wide, the narrow ones with K split over the waves:
     rows and batch ragged against every tile width, K shorter and much longer than the ring.  The
-    last two matrices are tall enough for the 64-row tiles that batches of 33..64 then take (one
+    last two matrices are tall enough for the 64-row tiles that batches of 33..128 then take (one
     of them ragged against 64 rows)."""
     w = synth.q8_0_weight(rows, cols, seed=rows * 3 + cols)
     x = synth.normal(batch, cols, seed=batch * 17 + cols)
