@@ -824,7 +824,7 @@ def main():
         g = result["gemm_int8"]["m2048_k5120_n17408"]
         result["roofline_gemm"] = {"bound": "mfma", "achieved": g["tops"], "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                                    "frac": g["frac_of_int8_peak"], "traffic": None,
-                                   "kernel": "gemm_d4_dma_kernel<false, 4> (128 x 128 tiles, M=2048, K=5120, N=17408)",
+                                   "kernel": "gemm_d4_dma_kernel<false, 4, false> (128 x 128 tiles, M=2048, K=5120, N=17408)",
                                    "ops_per_launch": 2 * 2048 * FFN * HIDDEN, "launch_ms": g["gemm_ms"],
                                    "frac_of_measured_rescale_ceiling": g["frac_of_rescale_ceiling"]}
         result["gemm_medium_batches"] = bench_gemm_medium(q8mi, hip, synth)

@@ -267,7 +267,7 @@ int q8mi_get_rows(const uint8_t *weight, const uint64_t *row_ids, uint32_t batch
 /* ---- argmax -------------------------------------------------------------- */
 /* replaces argmax_kernel, src/kernels_cuda.cu:1693-1734 (launched at :20759):
  * out2[0] = index (-1 if no element is above -inf), out2[1] = bits of the max.
- * Rows of 32768 elements and more (a vocabulary) are scanned by up to 128 workgroups whose
+ * Rows of 81920 elements and more (a vocabulary) are scanned by up to 128 workgroups whose
  * partial winners meet in a 1 KiB array the library holds in every GPU's memory (two launches;
  * the reference's single workgroup reads such a row at one CU's bandwidth).  This and
  * q8mi_argmax_to_pair share that array: calls on such rows that overlap on one GPU (two streams,

@@ -580,11 +580,11 @@ DeviceStatus HipQ8Backend::rms_norm_batch(DeviceTensor &out, const DeviceTensor 
     const float *nwp = reinterpret_cast<const float *>(w.ptr);
     float *nrm = T(out).f32();
     auto aligned16 = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    if (batch == 1 && n % 256 == 0 && n <= 6144 && nrm != xin && aligned16(xin) && aligned16(nwp) && aligned16(nrm)) {
+    if (norm_shortcuts_ && batch == 1 && n % 256 == 0 && n <= 6144 && nrm != xin && aligned16(xin) && aligned16(nwp) && aligned16(nrm)) {
         pending_ = PendingNorm{true, xin, nwp, nrm, n, eps};
         return {};
     }
-    if (batch <= 8 && n % 32 == 0) {
+    if (norm_shortcuts_ && batch <= 8 && n % 32 == 0) {
         forget_quantized();
         if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(batch, n), "q8_1 scratch alloc"); !st.ok) return st;
         if (q8mi_rms_norm_quantize_q8_1(xin, nwp, nrm, q8_1_.ptr, batch, n, n, n, eps, stream_) != Q8MI_OK)
@@ -594,6 +594,16 @@ DeviceStatus HipQ8Backend::rms_norm_batch(DeviceTensor &out, const DeviceTensor 
     }
     if (q8mi_rms_norm(xin, nwp, nrm, batch, n, n, n, eps, stream_) != Q8MI_OK) return failed("rms_norm");
     return launch_status("hip rms_norm_batch");
+}
+
+void HipQ8Backend::set_norm_shortcuts(bool on) {
+    if (!on) (void)invalidate_norm_state();
+    norm_shortcuts_ = on;
+}
+
+DeviceStatus HipQ8Backend::invalidate_norm_state() {
+    forget_quantized();
+    return flush_norm();
 }
 
 // include/qw3/device_backend.hpp:421-444

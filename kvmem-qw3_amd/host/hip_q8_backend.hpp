@@ -75,6 +75,15 @@ public:
     DeviceStatus begin() { return {}; }
     DeviceStatus end();           // drains the exec stream (src/kernels_cuda.cu:9807-9823)
     DeviceStatus synchronize();
+    // The two shortcuts behind rms_norm_batch (a one-row norm held back for the projection that
+    // reads it; the Q8_1 blocks a 2..8-row norm leaves for the projections that follow) rely on this
+    // backend seeing every write to the tensors involved.  A host that lets other code write those
+    // tensors between the norm and the projection (kernels of its own on exec_stream(), views that
+    // alias them) either calls invalidate_norm_state() before such a write or turns the shortcuts
+    // off; results are the same bits either way, only the launch count changes.
+    void set_norm_shortcuts(bool on);
+    bool norm_shortcuts() const { return norm_shortcuts_; }
+    DeviceStatus invalidate_norm_state();   // runs a held-back norm, forgets the cached blocks
     hipStream_t exec_stream() const { return stream_; }
 
     // HIP-graph capture of whatever is launched between begin_capture and end_capture
@@ -282,6 +291,7 @@ private:
 
     hipStream_t stream_ = nullptr;
     PendingNorm pending_;
+    bool norm_shortcuts_ = true;
     QuantizedRows quantized_;
     Scratch q8_1_, d4_, argmax_partial_, argmax_result_, lm_head_, lm_rows_, out_f32_, row_ids_;
     int32_t *argmax_dev_ = nullptr;    // {token, logit bits}

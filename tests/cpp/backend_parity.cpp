@@ -637,6 +637,26 @@ void case_norm_reuse(qw3::HipQ8Backend &b) {
         ok = ok && require(b.zero_tensor(*norm), "zero") && require(b.replay_graph(), "replay") && bits_equal(download_f32(b, *norm), nref);
         report("norm_held_back_under_capture", ok);
     }
+    // the shortcuts switched off (a host whose other kernels write these tensors): same bits
+    for (uint32_t batch : {1u, 4u}) {
+        const auto x = normal_vec(static_cast<size_t>(batch) * cols, 650 + batch, 2.0f);
+        auto dx = upload_f32(b, x);
+        auto norm = b.tensor_f32(x.size(), "n");
+        auto on = b.tensor_f32(static_cast<size_t>(batch) * rows, "on"), off = b.tensor_f32(static_cast<size_t>(batch) * rows, "off");
+        bool ok = require(b.rms_norm_batch(*norm, *dx, *nw, batch, cols, eps), "norm") &&
+                  require(b.q8_0_matmul_silu_mul(*on, *dw, *dw2, *norm, batch, cols, rows), "silu, shortcuts on");
+        b.set_norm_shortcuts(false);
+        ok = ok && !b.norm_shortcuts() && require(b.rms_norm_batch(*norm, *dx, *nw, batch, cols, eps), "norm") &&
+             require(b.q8_0_matmul_silu_mul(*off, *dw, *dw2, *norm, batch, cols, rows), "silu, shortcuts off");
+        b.set_norm_shortcuts(true);
+        ok = ok && bits_equal(download_f32(b, *on), download_f32(b, *off));
+        // invalidate_norm_state() runs a held-back norm: its output is there before any projection
+        std::vector<float> nref(x.size());
+        q8o_rms_norm(x.data(), nwv.data(), nref.data(), batch, cols, cols, cols, eps);
+        ok = ok && require(b.zero_tensor(*norm), "zero") && require(b.rms_norm_batch(*norm, *dx, *nw, batch, cols, eps), "norm") &&
+             require(b.invalidate_norm_state(), "invalidate") && bits_equal(download_f32(b, *norm), nref);
+        report(("norm_shortcuts_off_batch" + std::to_string(batch)).c_str(), ok);
+    }
 }
 
 void case_argmax(qw3::HipQ8Backend &b) {

@@ -36,7 +36,7 @@ def adversarial_rows(n, seed):
     return np.stack(rows)
 
 
-@pytest.mark.parametrize("n", [1, 31, 256, 1024, 1025, 32767, 32768, 32771, 248320, 262147])
+@pytest.mark.parametrize("n", [1, 31, 256, 1024, 1025, 32771, 81919, 81920, 81923, 248320, 262147])
 def test_argmax_single_row(gpu, oracle, n):
     rows = adversarial_rows(n, seed=n)
     L = q8mi.lib()
@@ -55,7 +55,7 @@ def test_argmax_single_row(gpu, oracle, n):
         assert p["index"] == idx and p["value"].view(np.int32) == np.float32(v).view(np.int32)
 
 
-@pytest.mark.parametrize("n", [5, 1027, 70001])
+@pytest.mark.parametrize("n", [5, 1027, 70001, 100003])
 def test_argmax_single_row_off_a_16_byte_boundary(gpu, oracle, n):
     """Rows on a 16-byte boundary are scanned four elements per load, others one by one: same result."""
     rows = adversarial_rows(n, seed=n + 7)
