@@ -39,9 +39,16 @@ namespace {
 
 thread_local char g_msg[256];
 
+using OwnerRef = std::shared_ptr<HipQ8Backend::Owner>;
+void tell_owner(const OwnerRef &owner, const void *ptr) {
+    if (owner && owner->backend && ptr) owner->backend->released(ptr);
+}
+
 struct HipTensor final : DeviceTensor {
     void *ptr = nullptr;
+    OwnerRef owner;
     ~HipTensor() override {
+        tell_owner(owner, ptr);
         if (ptr) (void)hipFree(ptr);
     }
     float *f32() const { return static_cast<float *>(ptr); }
@@ -52,7 +59,9 @@ struct HipTensor final : DeviceTensor {
 struct HipWeight final : DeviceWeight {
     uint8_t *ptr = nullptr;
     uint64_t bytes = 0;
+    OwnerRef owner;
     ~HipWeight() override {
+        tell_owner(owner, ptr);
         if (ptr) (void)hipFree(ptr);
     }
 };
@@ -74,8 +83,9 @@ DeviceStatus hip_status(hipError_t e, const char *where) {
     return {false, g_msg};
 }
 
-std::unique_ptr<DeviceTensor> make_tensor(uint64_t count, uint32_t elem_size, DeviceTensorDType dtype) {
+std::unique_ptr<DeviceTensor> make_tensor(uint64_t count, uint32_t elem_size, DeviceTensorDType dtype, const OwnerRef &owner) {
     auto t = std::make_unique<HipTensor>();
+    t->owner = owner;
     t->count = count;
     t->elem_size = elem_size;
     t->dtype = dtype;
@@ -88,13 +98,15 @@ std::unique_ptr<DeviceTensor> make_tensor(uint64_t count, uint32_t elem_size, De
 
 }  // namespace
 
-HipQ8Backend::HipQ8Backend() {
+HipQ8Backend::HipQ8Backend() : owner_(std::make_shared<Owner>()) {
+    owner_->backend = this;
     (void)hipSetDevice(0);
     // one non-blocking exec stream at the default priority (src/kernels_cuda.cu:9675-9679)
     (void)hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking);
 }
 
 HipQ8Backend::~HipQ8Backend() {
+    owner_->backend = nullptr;   // tensors and weights that outlive the backend have nobody to tell
     if (stream_) (void)hipStreamSynchronize(stream_);
     for (Scratch *s : {&q8_1_, &d4_, &argmax_partial_, &argmax_result_, &lm_head_, &lm_rows_, &out_f32_, &row_ids_}) {
         if (s->ptr) (void)hipFree(s->ptr);
@@ -146,16 +158,17 @@ DeviceStatus HipQ8Backend::replay_graph() {
 // (A new tensor may reuse the address of a freed one: whatever the scratch holds for that address is stale.)
 std::unique_ptr<DeviceTensor> HipQ8Backend::tensor_f32(uint64_t count, const char *) {
     forget_quantized();
-    return make_tensor(count, 4, DeviceTensorDType::F32);
+    return make_tensor(count, 4, DeviceTensorDType::F32, owner_);
 }
 
 std::unique_ptr<DeviceTensor> HipQ8Backend::tensor_bf16(uint64_t count, const char *) {
     forget_quantized();
-    return make_tensor(count, 2, DeviceTensorDType::BF16);
+    return make_tensor(count, 2, DeviceTensorDType::BF16, owner_);
 }
 
 std::unique_ptr<DeviceWeight> HipQ8Backend::weight_f32(const float *data, uint64_t count, const char *) {
     auto w = std::make_unique<HipWeight>();
+    w->owner = owner_;
     w->rows = 1;
     w->cols = count;
     w->format = DeviceWeightFormat::F32;
@@ -173,6 +186,7 @@ std::unique_ptr<DeviceWeight> HipQ8Backend::weight_q8_0(const void *data, uint64
                                                         const char *) {
     if (cols % 32 != 0) return nullptr;
     auto w = std::make_unique<HipWeight>();
+    w->owner = owner_;
     w->rows = rows;
     w->cols = cols;
     w->format = DeviceWeightFormat::Q8_0;
@@ -272,6 +286,13 @@ DeviceStatus HipQ8Backend::flush_norm() {
         return failed("rms_norm_quantize_q8_1");
     quantized_ = QuantizedRows{n.out, 1, n.cols, n.cols};
     return launch_status("hip rms_norm");
+}
+
+void HipQ8Backend::released(const void *ptr) {
+    if (ptr == quantized_.src) forget_quantized();
+    if (!pending_.active) return;
+    if (ptr == pending_.out) pending_.active = false;
+    else if (ptr == pending_.x || ptr == pending_.weight) (void)flush_norm();
 }
 
 // Whether a batch-1 projection of x (cols floats) whose first output is out0 can run the held-back

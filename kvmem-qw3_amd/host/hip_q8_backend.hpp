@@ -84,6 +84,14 @@ public:
     void set_norm_shortcuts(bool on);
     bool norm_shortcuts() const { return norm_shortcuts_; }
     DeviceStatus invalidate_norm_state();   // runs a held-back norm, forgets the cached blocks
+    // Called by the destructors of this backend's tensors and weights, before they free `ptr`: a
+    // held-back norm that reads it runs now, one that only writes it is dropped (nobody can read
+    // the result), cached blocks of its rows are forgotten.
+    void released(const void *ptr);
+    // What those objects keep of the backend: cleared when the backend goes first.
+    struct Owner {
+        HipQ8Backend *backend = nullptr;
+    };
     hipStream_t exec_stream() const { return stream_; }
 
     // HIP-graph capture of whatever is launched between begin_capture and end_capture
@@ -292,6 +300,7 @@ private:
     hipStream_t stream_ = nullptr;
     PendingNorm pending_;
     bool norm_shortcuts_ = true;
+    std::shared_ptr<Owner> owner_;
     QuantizedRows quantized_;
     Scratch q8_1_, d4_, argmax_partial_, argmax_result_, lm_head_, lm_rows_, out_f32_, row_ids_;
     int32_t *argmax_dev_ = nullptr;    // {token, logit bits}

@@ -637,6 +637,27 @@ void case_norm_reuse(qw3::HipQ8Backend &b) {
         ok = ok && require(b.zero_tensor(*norm), "zero") && require(b.replay_graph(), "replay") && bits_equal(download_f32(b, *norm), nref);
         report("norm_held_back_under_capture", ok);
     }
+    // tensors destroyed while a norm is held back: an output nobody can read is dropped, an input
+    // is read before it is freed
+    {
+        const auto x = normal_vec(cols, 645, 2.0f);
+        std::vector<float> nref(cols);
+        q8o_rms_norm(x.data(), nwv.data(), nref.data(), 1, cols, cols, cols, eps);
+        auto h = upload_f32(b, x);
+        auto gone = b.tensor_f32(cols, "gone");
+        bool ok = require(b.rms_norm(*gone, *h, *nw, eps), "norm into a tensor about to go");
+        gone.reset();
+        auto norm = b.tensor_f32(cols, "n");
+        ok = ok && require(b.rms_norm(*norm, *h, *nw, eps), "norm");
+        h.reset();                                  // the norm's input goes: the norm runs first
+        ok = ok && bits_equal(download_f32(b, *norm), nref);
+        auto out = b.tensor_f32(rows, "o");
+        ok = ok && require(b.q8_0_matvec(*out, *dw, *norm), "matvec after the tensors went");
+        std::vector<float> ref, mag;
+        oracle_linear(w, nref.data(), 1, cols, rows, ref, mag);
+        ok = ok && close_fp32(download_f32(b, *out), ref, mag, 1, rows, rows, d);
+        report("norm_held_back_tensors_destroyed", ok, d);
+    }
     // the shortcuts switched off (a host whose other kernels write these tensors): same bits
     for (uint32_t batch : {1u, 4u}) {
         const auto x = normal_vec(static_cast<size_t>(batch) * cols, 650 + batch, 2.0f);
