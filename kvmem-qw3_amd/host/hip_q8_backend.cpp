@@ -112,7 +112,7 @@ HipQ8Backend::~HipQ8Backend() {
         if (s->ptr) (void)hipFree(s->ptr);
     }
     if (argmax_dev_) (void)hipFree(argmax_dev_);
-    if (accept_dev_) (void)hipFree(accept_dev_);
+    if (lm_host_) (void)hipHostFree(lm_host_);
     if (argmax_host_) (void)hipHostFree(argmax_host_);
     if (graph_exec_) (void)hipGraphExecDestroy(graph_exec_);
     if (graph_) (void)hipGraphDestroy(graph_);
@@ -956,25 +956,27 @@ DeviceStatus HipQ8Backend::lm_head_verify(const DeviceWeight &w_out, const Devic
     const uint32_t cols = static_cast<uint32_t>(w.cols), vocab = static_cast<uint32_t>(w.rows);
     if (auto st = ensure(lm_head_, q8mi_lm_head_scratch_bytes(vocab, cols, batch), "lm head scratch alloc"); !st.ok)
         return st;
-    if (auto st = ensure(lm_rows_, 8 * sizeof(q8mi_argmax_pair), "lm head rows alloc"); !st.ok) return st;
-    if (!accept_dev_) {
-        if (auto st = hip_status(hipMalloc(reinterpret_cast<void **>(&accept_dev_), 8), "accept alloc"); !st.ok)
+    // eight row pairs and {accepted, next} side by side on the device, and a pinned mirror: one copy back
+    constexpr size_t kResultBytes = 8 * sizeof(q8mi_argmax_pair) + 2 * sizeof(int32_t);
+    if (auto st = ensure(lm_rows_, kResultBytes, "lm head rows alloc"); !st.ok) return st;
+    if (!lm_host_) {
+        if (capturing_) return {false, "lm_head_verify: first call must run outside graph capture"};
+        if (auto st = hip_status(hipHostMalloc(reinterpret_cast<void **>(&lm_host_), kResultBytes, hipHostMallocDefault),
+                                 "lm head pinned mirror"); !st.ok)
             return st;
     }
     if (auto st = quantize_q8_1(T(norm).f32(), batch, cols, in_stride ? in_stride : cols); !st.ok) return st;
     auto *rows_dev = static_cast<q8mi_argmax_pair *>(lm_rows_.ptr);
-    if (q8mi_lm_head_argmax_accept(w.ptr, q8_1_.ptr, vocab, cols, batch, drafts, 0, eos, rows_dev, accept_dev_,
+    auto *accept_dev = reinterpret_cast<int32_t *>(rows_dev + 8);
+    if (q8mi_lm_head_argmax_accept(w.ptr, q8_1_.ptr, vocab, cols, batch, drafts, 0, eos, rows_dev, accept_dev,
                                    nullptr, vocab, lm_head_.ptr, stream_) != Q8MI_OK)
         return failed("lm_head_argmax_accept");
-    q8mi_argmax_pair host_rows[8];
-    int32_t host_acc[2] = {0, eos};
-    if (auto st = hip_status(hipMemcpyAsync(host_rows, rows_dev, batch * sizeof(q8mi_argmax_pair),
-                                            hipMemcpyDeviceToHost, stream_), "lm head rows copy"); !st.ok)
-        return st;
-    if (auto st = hip_status(hipMemcpyAsync(host_acc, accept_dev_, 8, hipMemcpyDeviceToHost, stream_),
-                             "lm head accept copy"); !st.ok)
+    if (auto st = hip_status(hipMemcpyAsync(lm_host_, rows_dev, kResultBytes, hipMemcpyDeviceToHost, stream_),
+                             "lm head result copy"); !st.ok)
         return st;
     if (auto st = synchronize(); !st.ok) return st;
+    const auto *host_rows = reinterpret_cast<const q8mi_argmax_pair *>(lm_host_);
+    const auto *host_acc = reinterpret_cast<const int32_t *>(host_rows + 8);
     rows_out.assign(batch, DeviceArgmax{});
     for (uint32_t i = 0; i < batch; ++i) rows_out[i] = {host_rows[i].index, host_rows[i].value};
     accepted = static_cast<uint32_t>(host_acc[0]);

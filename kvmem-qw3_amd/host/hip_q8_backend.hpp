@@ -305,7 +305,7 @@ private:
     Scratch q8_1_, d4_, argmax_partial_, argmax_result_, lm_head_, lm_rows_, out_f32_, row_ids_;
     int32_t *argmax_dev_ = nullptr;    // {token, logit bits}
     int32_t *argmax_host_ = nullptr;   // pinned mirror
-    int32_t *accept_dev_ = nullptr;    // {accepted, next}
+    uint8_t *lm_host_ = nullptr;       // pinned mirror of lm_head_verify's row pairs and {accepted, next}
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
     bool capturing_ = false;
