@@ -113,7 +113,10 @@ __global__ __launch_bounds__(THREADS) void gemv_kernel(const GemvParams p) {
 // ---- matrix-core variant for batch 3..32 (see q8mi_gemv_mfma_core.hpp) --------------------------
 // Unit u covers rows 4u .. 4u+3 of the concatenated row space; for SwiGLU gate rows 2u, 2u+1
 // (fragment rows 0, 1) and the matching up rows (fragment rows 2, 3).
-template <int MG, int THREADS, bool SILU, bool HS, bool D4, int DEPTH, bool STREAMING>
+// ITEMWISE: the workgroup's items are dealt round-robin to its waves (see mfma_stream) and every
+// item's sums are parked, [item][fragment row][activation row]; otherwise a wave takes a contiguous
+// range of items and parks once per unit it touched.
+template <int MG, int THREADS, bool SILU, bool HS, bool D4, int DEPTH, bool STREAMING, bool ITEMWISE>
 __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, uint32_t batch,
                                                             uint32_t park_floats) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -129,8 +132,13 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
     const uint32_t ucount = useq.count;
     const uint32_t n_items = ucount * nitems;
     uint32_t i0, i1;
-    wave_items(n_items, wave, kWaves, i0, i1);
-    float *park_base = reinterpret_cast<float *>(smem + p.x_bytes);   // [wave][park_floats]
+    if constexpr (ITEMWISE) {
+        i0 = wave < n_items ? wave : n_items;
+        i1 = n_items;
+    } else {
+        wave_items(n_items, wave, kWaves, i0, i1);
+    }
+    float *park_base = reinterpret_cast<float *>(smem + p.x_bytes);   // [wave][park_floats], or [item][kMfmaUnitRows][MP]
     float *my_park = park_base + wave * park_floats;
     const uint32_t last_row = p.total_rows - 1;
 
@@ -157,27 +165,47 @@ __global__ __launch_bounds__(THREADS) void gemv_mfma_kernel(const GemvParams p, 
             }
         }
     };
-    mfma_stream<MG, THREADS, HS, D4, DEPTH, STREAMING>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
-    __syncthreads();
-
-    // unit ranges of the waves, worked out once (wave w touched unit ordinals kf[w] .. kl[w])
+    // the wave's t-th item is item wave + t kWaves of the workgroup; lane (rho, q odd, n) holds the
+    // total for fragment row n and activation row (q >> 1) + 2 rho (MG 2) or rho (MG 1)
+    auto park_item = [&](uint32_t t, float total) {
+        const uint32_t rho = lane >> 4, q = (lane >> 2) & 3u, n = lane & 3u;
+        const uint32_t m = MG == 2 ? (q >> 1) + 2 * rho : rho;
+        if (MG == 2 ? (q & 1u) != 0 : q == 1)
+            park_base[(wave + t * kWaves) * (kMfmaUnitRows * MP) + n * MP + m] = total;
+    };
     __shared__ uint32_t s_kf[kWaves], s_kl[kWaves];
-    if (threadIdx.x < kWaves) {
-        uint32_t a0, a1;
-        wave_items(n_items, threadIdx.x, kWaves, a0, a1);
-        s_kf[threadIdx.x] = a1 > a0 ? a0 / nitems : 1u;
-        s_kl[threadIdx.x] = a1 > a0 ? (a1 - 1) / nitems : 0u;   // empty range: kf > kl
+    if constexpr (ITEMWISE) {
+        (void)park;
+        (void)park_floats;
+        mfma_stream<MG, THREADS, HS, D4, DEPTH, STREAMING, true>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park_item);
+        __syncthreads();
+    } else {
+        mfma_stream<MG, THREADS, HS, D4, DEPTH, STREAMING>(smem, p.y, p.nb, batch, p.x_stride, useq, i0, i1, row_ptr, park);
+        __syncthreads();
+        // unit ranges of the waves, worked out once (wave w touched unit ordinals kf[w] .. kl[w])
+        if (threadIdx.x < kWaves) {
+            uint32_t a0, a1;
+            wave_items(n_items, threadIdx.x, kWaves, a0, a1);
+            s_kf[threadIdx.x] = a1 > a0 ? a0 / nitems : 1u;
+            s_kl[threadIdx.x] = a1 > a0 ? (a1 - 1) / nitems : 0u;   // empty range: kf > kl
+        }
+        __syncthreads();
     }
-    __syncthreads();
-    // total for unit ordinal k, fragment row rr, activation row m: partials in wave order, chunks in order
+    // total for unit ordinal k, fragment row rr, activation row m: the unit's items in order, or the
+    // waves' partials in wave order, chunks in order
     auto total_of = [&](uint32_t k, uint32_t rr, uint32_t m) {
         float t = 0.0f;
+        if constexpr (ITEMWISE) {
+            const float *e = park_base + static_cast<size_t>(k) * nitems * (kMfmaUnitRows * MP) + rr * MP + m;
+            for (uint32_t part = 0; part < nitems; ++part) t += e[part * (kMfmaUnitRows * MP)];
+        } else {
 #pragma unroll
-        for (uint32_t w = 0; w < kWaves; ++w) {
-            const uint32_t kf = s_kf[w], kl = s_kl[w];
-            if (k < kf || k > kl) continue;
-            const float *e = park_base + w * park_floats + (k - kf) * kPerUnit + rr * MP + m;
-            t += ((e[0] + e[kMfmaUnitRows * MP]) + e[2 * kMfmaUnitRows * MP]) + e[3 * kMfmaUnitRows * MP];
+            for (uint32_t w = 0; w < kWaves; ++w) {
+                const uint32_t kf = s_kf[w], kl = s_kl[w];
+                if (k < kf || k > kl) continue;
+                const float *e = park_base + w * park_floats + (k - kf) * kPerUnit + rr * MP + m;
+                t += ((e[0] + e[kMfmaUnitRows * MP]) + e[2 * kMfmaUnitRows * MP]) + e[3 * kMfmaUnitRows * MP];
+            }
         }
         return t;
     };
@@ -303,17 +331,30 @@ int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     // 5120 x 17408 22.0 -> 20.6 us, but 8192 x 5120 11.7 -> 12.5 us and 5120 x 6144 10.1 -> 10.8 us)
     constexpr uint64_t kStreamFrom = 64ull * 1000 * 1000;
     const bool streaming = (SILU ? 2ull : 1ull) * p.total_rows * p.nb * 34 >= kStreamFrom;
-    auto kern = streaming ? gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, true>
-                          : gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, false>;
     const uint32_t grid = p.units < cus ? p.units : cus;
     const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
     const uint32_t per_group = (p.units + grid - 1) / grid;
+    constexpr uint32_t kDynLimit = kLdsLimit - 256;   // the kernel also has a few static LDS words
+    static KernelGeometry geometry[2][2];
+    // Items dealt round-robin to the waves wherever every item's sums fit LDS beside the activations
+    // (up to eight activation rows, one item in flight per wave); else contiguous ranges per wave.
+    if constexpr (MG <= 2 && DEPTH == 1) {
+        const uint64_t item_park = static_cast<uint64_t>(per_group) * nitems * kMfmaUnitRows * 4 * MG * 4;
+        if (p.x_bytes + item_park <= kDynLimit) {
+            auto kern = streaming ? gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, true, true>
+                                  : gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, false, true>;
+            if (!geometry[1][streaming].grant(reinterpret_cast<const void *>(kern), kDynLimit))
+                return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", kDynLimit);
+            kern<<<grid, THREADS, p.x_bytes + static_cast<uint32_t>(item_park), stream>>>(p, batch, 0);
+            return check_launch("gemv_mfma");
+        }
+    }
+    auto kern = streaming ? gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, true, false>
+                          : gemv_mfma_kernel<MG, THREADS, SILU, HS, D4, DEPTH, false, false>;
     const uint32_t park_floats = max_units_touched(per_group, nitems, THREADS / kWave) * mfma_park_floats_per_unit(MG);
     const uint32_t lds = p.x_bytes + (THREADS / kWave) * park_floats * 4;
-    constexpr uint32_t kDynLimit = kLdsLimit - 256;   // the kernel also has a few static LDS words
     if (lds > kDynLimit) return fail(Q8MI_REJECTED, "gemv (matrix-core variant): %u bytes of LDS needed", lds);
-    static KernelGeometry geometry[2];
-    if (!geometry[streaming].grant(reinterpret_cast<const void *>(kern), kDynLimit))
+    if (!geometry[0][streaming].grant(reinterpret_cast<const void *>(kern), kDynLimit))
         return fail(Q8MI_LAUNCH_ERROR, "gemv: cannot reserve %u bytes of LDS", lds);
     kern<<<grid, THREADS, lds, stream>>>(p, batch, park_floats);
     return check_launch("gemv_mfma");

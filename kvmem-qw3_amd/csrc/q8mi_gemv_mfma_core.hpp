@@ -213,6 +213,47 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *y,
     __syncthreads();
 }
 
+// The sums of one item over the sixteen lane quads of the wave, for the item-wise split below: lane
+// 16 rho + 4 q + n holds acc[g][v] for weight row n; on return lane (rho, q odd, n) holds the wave's
+// total for weight row n and activation row (q >> 1) + 2 rho (MG == 2; both odd q hold activation
+// row rho for MG == 1).  Every step halves the registers instead of leaving copies: the halves of
+// two registers change places (v_permlane32_swap, then v_permlane16_swap for the rows of 16 lanes)
+// and one addition folds both; the quads of a row of 16 follow by two DPP additions.  A fixed tree:
+// same bits on every run.
+template <int MG>
+__device__ __forceinline__ float mfma_item_total(const float (&acc)[MG][4]) {
+    static_assert(MG == 1 || MG == 2, "item-wise sums are built for up to eight activation rows");
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    auto fold32 = [](float a, float b) {   // lanes 0..31: a summed over lane bit 5; lanes 32..63: b
+        const v2u r = __builtin_amdgcn_permlane32_swap(static_cast<unsigned>(as_i32(a)), static_cast<unsigned>(as_i32(b)), false, false);
+        return as_f32(static_cast<int>(r.x)) + as_f32(static_cast<int>(r.y));
+    };
+    auto fold16 = [](float a, float b) {   // rows 0, 2: a summed over lane bit 4; rows 1, 3: b
+        const v2u r = __builtin_amdgcn_permlane16_swap(static_cast<unsigned>(as_i32(a)), static_cast<unsigned>(as_i32(b)), false, false);
+        return as_f32(static_cast<int>(r.x)) + as_f32(static_cast<int>(r.y));
+    };
+    auto quads = [](float w) {        // w summed over the quads q and q ^ 2 of its row
+        // row_ror:8: lane i of every row of 16 reads lane (i + 8) % 16
+        return w + as_f32(__builtin_amdgcn_update_dpp(0, as_i32(w), 0x128, 0xf, 0xf, false));
+    };
+    float v;
+    if constexpr (MG == 2) {
+        float z[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) z[j] = fold32(acc[0][j], acc[1][j]);   // lower half: activation row j, upper: 4 + j
+        const float u0 = quads(fold16(z[0], z[2]));   // row rho: activation row 2 rho
+        const float u1 = quads(fold16(z[1], z[3]));   // row rho: activation row 2 rho + 1
+        // quads 0, 1 keep u0, quads 2, 3 take u1
+        v = as_f32(__builtin_amdgcn_update_dpp(as_i32(u0), as_i32(u1), 0xE4, 0xf, 0xC, false));
+    } else {
+        const float z0 = fold32(acc[0][0], acc[0][2]);   // lower half: activation row 0, upper: 2
+        const float z1 = fold32(acc[0][1], acc[0][3]);   // lower half: 1, upper: 3
+        v = quads(fold16(z0, z1));                       // row rho: activation row rho
+    }
+    // quad q + quad q - 1: complete in the odd quads
+    return v + as_f32(__builtin_amdgcn_update_dpp(0, as_i32(v), kDppRowShr4, 0xf, 0xf, true));
+}
+
 // Streams the items [i0, i1) of the workgroup's unit sequence (item i = part i % nitems of unit
 // i / nitems, nitems = ceil(nb / 32)).
 //   row_ptr(u)             the weight row (scale plane) this lane LOADS for unit u: fragment row lane % 4,
@@ -225,7 +266,14 @@ __device__ __forceinline__ void mfma_stage_x_d4(uint8_t *smem, const uint8_t *y,
 // DEPTH: items a wave keeps in flight.
 // STREAMING: the quant loads carry the non-temporal hint (every weight byte is read once per launch);
 //            worth 5..7 % on streams of 100 MB and more, costs 5..8 % on those of 30..45 MB.
-template <int MG, int THREADS, bool HS, bool D4, int DEPTH = kMfmaDepth, bool STREAMING = true, class RowPtr, class Park>
+// ITEMWISE: the wave takes the items i0, i0 + W, i0 + 2 W, ... below i1 (W = waves of the workgroup)
+//            instead of a contiguous range, so that the workgroup's loads in flight are W neighbouring
+//            items: whole rows, not one KiB of eight different row quads (measured with a bare read of
+//            the same pattern: 2 x 17408 x 5120 30.7 -> 28.8 us, 8192 x 5120 10.5 -> 9.1 us, 5120 x 17408
+//            17.2 -> 16.4 us).  Consecutive items of a wave then belong to different units, so
+//            park(t, total) is called after every item t = 0, 1, ... with the lane's entry of
+//            mfma_item_total().
+template <int MG, int THREADS, bool HS, bool D4, int DEPTH = kMfmaDepth, bool STREAMING = true, bool ITEMWISE = false, class RowPtr, class Park>
 __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uint32_t nb, uint32_t batch,
                                             uint32_t d4_batch_total, const UnitSeq &useq, uint32_t i0, uint32_t i1, RowPtr row_ptr,
                                             Park park) {
@@ -239,7 +287,17 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
         else mfma_stage_x<MG, THREADS, HS>(smem, y, nb, batch);
         return;
     }
-    const uint32_t n_items = i1 - i0;
+    constexpr uint32_t kStride = ITEMWISE ? THREADS / kWave : 1;   // items from one of the wave's to the next
+    const uint32_t n_items = (i1 - i0 + kStride - 1) / kStride;
+    auto advance = [&](uint32_t &k, uint32_t &step) {   // (unit ordinal, part) of the wave's next item; true: another unit
+        step += kStride;
+        const uint32_t k0 = k;
+        while (step >= nitems) {
+            step -= nitems;
+            ++k;
+        }
+        return k != k0;
+    };
 
     // activation loads first, the first weight items behind them (they stay in flight while the
     // activations are converted)
@@ -276,11 +334,7 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
         }
         if (ileft > 1) {          // otherwise keep re-reading the last real item
             --ileft;
-            if (++istep == nitems) {
-                istep = 0;
-                ++ik;
-                irow = row_ptr(useq.unit(ik));
-            }
+            if (advance(ik, istep)) irow = row_ptr(useq.unit(ik));
         }
     };
 #pragma unroll
@@ -375,25 +429,35 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
                 acc[g][3] = fmaf(fmaf(as_f32(r[g].w), dw, cw), dx[g].w, acc[g][3]);
             }
         }
-        ++cstep;
-        if (cstep == nitems || done == n_items) {
-            // the sixteen lanes of equal row meet in four: lanes 0 .. 15 then hold, for row lane % 4,
-            // the sum over a quarter of the blocks
-#pragma unroll
-            for (int g = 0; g < MG; ++g)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    acc[g][v] += lane_xor<16>(acc[g][v]);
-                    acc[g][v] += lane_xor<32>(acc[g][v]);
-                }
-            park(kk, acc);
-            ++kk;
+        if constexpr (ITEMWISE) {
+            park(done - 1, mfma_item_total<MG>(acc));
 #pragma unroll
             for (int g = 0; g < MG; ++g)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) acc[g][v] = 0.0f;
+            uint32_t unused = 0;
+            advance(unused, cstep);
+        } else {
+            ++cstep;
+            if (cstep == nitems || done == n_items) {
+                // the sixteen lanes of equal row meet in four: lanes 0 .. 15 then hold, for row lane % 4,
+                // the sum over a quarter of the blocks
+#pragma unroll
+                for (int g = 0; g < MG; ++g)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        acc[g][v] += lane_xor<16>(acc[g][v]);
+                        acc[g][v] += lane_xor<32>(acc[g][v]);
+                    }
+                park(kk, acc);
+                ++kk;
+#pragma unroll
+                for (int g = 0; g < MG; ++g)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[g][v] = 0.0f;
+            }
+            if (cstep == nitems) cstep = 0;
         }
-        if (cstep == nitems) cstep = 0;
     };
     // Whole rounds of DEPTH items, each slot refilled as soon as it is consumed (past the
     // last item the refills re-read it, so the loop stays branch-free and the load counters
