@@ -441,10 +441,10 @@ constexpr uint32_t kPairsMaxBatch = 4;    // largest batch the row-pair family s
 // Which GEMV family serves a launch of batch 2 and more (measured on MI355X, row-pair kernel with
 // the rows shared by the waves of a workgroup against matrix-core kernel, us):
 //   rows of 4 .. 8 KiB         batch 2: always row pairs (8192 x 5120 fan-out 9.3 / 11.9, SwiGLU 30.2 / 34.1);
-//                              batch 3: row pairs (fan-out 10.0 / 11.9, 5120 x 6144 9.2 / 10.3, SwiGLU 32.0 / 33.9);
-//                              batch 4: row pairs but for the SwiGLU form (fan-out 10.8 / 11.7, 5120 x 6144
-//                              10.2 / 10.2, SwiGLU 33.7 / 33.7 at best); from batch 5 the dot products bind
-//                              (batch 6: 13.1 / 12.3 on the fan-out)
+//                              batch 3 and 4: row pairs but for the SwiGLU form (fan-out 10.3 / 11.7 and
+//                              11.4 / 11.7, 5120 x 6144 9.8 / 11 and 10.2 / 11, SwiGLU 32.1 / 31.0 and
+//                              33.7 / 31.0 since the matrix-core kernel deals its items round-robin to the
+//                              waves); from batch 5 the dot products bind (batch 6: 13.1 / 12.3 on the fan-out)
 //   rows of 9 .. 17 KiB        batch 2: row pairs (5120 x 17408: 18.8 / 20.0); batch 3 and 4: 22.4 / 20.3, 30.0 / 20.6
 //   any other length           batch 2 with 8192 row pairs or more: row pairs (ring kernel); else matrix cores
 // nb: blocks per row; silu: the SwiGLU form.
@@ -454,7 +454,6 @@ inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch, uint32_t nb, b
     const bool short_rows = nb % 32 == 0 && nb >= 128 && nb <= 256;   // 4 .. 8 KiB
     const bool whole_kib = nb % 32 == 0 && nb >= 128 && nb <= 544;     // 4 .. 17 KiB: a shared-row kernel of its own
     if (batch == 2) return !whole_kib && row_pairs < 8192;
-    if (batch == 3) return !short_rows;
     return !short_rows || silu;
 }
 

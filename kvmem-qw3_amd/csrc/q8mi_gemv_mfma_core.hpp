@@ -379,8 +379,8 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
     };
 
     uint32_t cstep = i0 % nitems, kk = 0;
-    // one item: `done` counts the items consumed so far, this one included
-    auto consume = [&](const MfmaItem &it, uint32_t done) {
+    // one item's products into acc
+    auto compute = [&](const MfmaItem &it) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const uint32_t kb = cstep * kMfmaItemBlocks + 16 * t + blk;
@@ -429,6 +429,9 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
                 acc[g][3] = fmaf(fmaf(as_f32(r[g].w), dw, cw), dx[g].w, acc[g][3]);
             }
         }
+    };
+    // after an item: `done` counts the items consumed so far, this one included
+    auto finish = [&](uint32_t done) {
         if constexpr (ITEMWISE) {
             park(done - 1, mfma_item_total<MG>(acc));
 #pragma unroll
@@ -459,20 +462,24 @@ __device__ __forceinline__ void mfma_stream(uint8_t *smem, const uint8_t *y, uin
             if (cstep == nitems) cstep = 0;
         }
     };
-    // Whole rounds of DEPTH items, each slot refilled as soon as it is consumed (past the
-    // last item the refills re-read it, so the loop stays branch-free and the load counters
-    // exact); then the items of a last, partial round, without refills.
+    // Whole rounds of DEPTH items, each slot refilled as soon as its products are formed and before
+    // its sums are parked (past the last item the refills re-read it, so the loop stays branch-free
+    // and the load counters exact); then the items of a last, partial round, without refills.
     uint32_t t = 0;
     for (; t + DEPTH <= n_items; t += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
-            consume(items[d], t + d + 1);
+            compute(items[d]);
             issue(items[d]);
+            finish(t + d + 1);
         }
     }
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; ++d)
-        if (t + d < n_items) consume(items[d], t + d + 1);
+        if (t + d < n_items) {
+            compute(items[d]);
+            finish(t + d + 1);
+        }
 }
 
 }  // namespace q8mi

@@ -139,6 +139,11 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
 // the first and the last of its range) are parked, two slots per wave, and added up in wave order
 // after the stream.  LDS use does not grow with the number of rows, so one workgroup per CU
 // covers a vocabulary of any size in a single pass.
+// Units per round of the item-wise kernel below: with 512 threads and four (eight) activation rows
+// 128 (64) units give every thread four triples to add up per round.
+__host__ __device__ constexpr uint32_t lm_head_round_units(int mg) { return mg == 2 ? 64u : 128u; }
+constexpr int kLmHeadItemsDepth = 1;   // items a wave keeps in flight in that kernel
+
 template <int MG, int THREADS>
 __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
         const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, uint32_t rows, uint32_t nb, uint32_t batch,
@@ -281,6 +286,111 @@ __global__ __launch_bounds__(THREADS) void lm_head_mfma_kernel(
     }
 }
 
+// The matrix-core variant with the workgroup's items dealt round-robin to its waves (ITEMWISE in
+// mfma_stream: the loads in flight are eight neighbouring items, i.e. whole rows, which streams a
+// few per cent faster than eight waves each working through a range of its own).  Every item's
+// sums are parked, so the units are taken in rounds of lm_head_round_units(): after a wave's last
+// item of a round (its next item is already requested) the workgroup meets at a barrier and every
+// thread adds up the items of kOut (unit, row, activation row) triples of that round, always for
+// the same activation row, and folds them into its running best.  Two park buffers, used in turn,
+// let the waves go on with the next round while others still add.  LDS use does not depend on the
+// number of rows.
+template <int MG, int THREADS, int DEPTH, bool LOGITS>
+__global__ __launch_bounds__(THREADS) void lm_head_items_kernel(
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, uint32_t rows, uint32_t nb, uint32_t batch,
+        q8mi_argmax_pair *__restrict__ partial, float *__restrict__ logits, uint32_t stride_logits,
+        int interleave, uint32_t x_bytes) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr uint32_t MP = 4 * MG;
+    constexpr uint32_t kWaves = THREADS / kWave;
+    constexpr uint32_t kPerItem = kMfmaUnitRows * MP;                  // floats parked per item: [row][activation row]
+    constexpr uint32_t kRoundUnits = lm_head_round_units(MG);
+    constexpr uint32_t kOut = kRoundUnits * kPerItem / THREADS;        // triples a thread adds up per round
+    static_assert(kRoundUnits % kWaves == 0 && kRoundUnits * kPerItem % THREADS == 0 && THREADS % MP == 0, "round geometry");
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t r = lane & 3u;
+    const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
+    const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
+    const uint32_t units = (rows + kMfmaUnitRows - 1) / kMfmaUnitRows;
+    const UnitSeq useq = group_units(units, blockIdx.x, gridDim.x, interleave);
+    const uint32_t ucount = useq.count;
+    const uint32_t n_items = ucount * nitems;
+    const uint32_t round_items = kRoundUnits * nitems;          // a multiple of kWaves
+    const uint32_t full_rounds = n_items / round_items;
+    const uint32_t per_wave = round_items / kWaves;             // items of a wave per full round
+    float *park_base = reinterpret_cast<float *>(smem + x_bytes);   // [2][round_items][kPerItem]
+
+    // this thread's triples of a round: (unit k_mine + j kUnitStep, row rr_mine, activation row m_mine)
+    const uint32_t m_mine = threadIdx.x % MP, rr_mine = (threadIdx.x / MP) % kMfmaUnitRows;
+    const uint32_t k_mine = threadIdx.x / kPerItem;              // 0 .. THREADS / kPerItem - 1
+    constexpr uint32_t kUnitStep = THREADS / kPerItem;
+    float bv = -INFINITY;
+    int bi = -1;
+    // adds up round `round` (its first `count` units) from its park buffer
+    auto add_round = [&](uint32_t round, uint32_t count) {
+        const float *buf = park_base + static_cast<size_t>(round & 1u) * round_items * kPerItem;
+#pragma unroll
+        for (uint32_t j = 0; j < kOut; ++j) {
+            const uint32_t kl = k_mine + j * kUnitStep;
+            if (kl >= count) break;
+            const float *e = buf + static_cast<size_t>(kl) * nitems * kPerItem + rr_mine * MP + m_mine;
+            float t = 0.0f;
+            for (uint32_t part = 0; part < nitems; ++part) t += e[part * kPerItem];
+            const uint32_t row = kMfmaUnitRows * useq.unit(round * kRoundUnits + kl) + rr_mine;
+            if (row < rows && m_mine < batch) {
+                if (beats(t, static_cast<int>(row), bv, bi)) { bv = t; bi = static_cast<int>(row); }
+                if constexpr (LOGITS) logits[static_cast<uint64_t>(m_mine) * stride_logits + row] = t;
+            }
+        }
+    };
+
+    auto row_ptr = [&](uint32_t u) -> const uint8_t * {
+        uint32_t row = kMfmaUnitRows * u + r;
+        row = row < rows - 1 ? row : rows - 1;
+        return w + row * row_bytes;
+    };
+    // the wave's t-th item is item wave + t kWaves of the workgroup; lane (rho, q odd, n) holds the
+    // total for row n of the item's unit and activation row (q >> 1) + 2 rho (MG 2) or rho (MG 1)
+    auto park = [&](uint32_t t, float total) {
+        const uint32_t item = wave + t * kWaves;
+        const uint32_t round = t / per_wave;                   // the same for every wave: per_wave items each
+        const uint32_t in_round = item - round * round_items;
+        const uint32_t rho = lane >> 4, q = (lane >> 2) & 3u, n = lane & 3u;
+        const uint32_t m = MG == 2 ? (q >> 1) + 2 * rho : rho;
+        if (MG == 2 ? (q & 1u) != 0 : q == 1)
+            park_base[(static_cast<size_t>(round & 1u) * round_items + in_round) * kPerItem + n * MP + m] = total;
+        if ((t + 1) % per_wave == 0 && round < full_rounds) {  // the wave's last item of a whole round
+            __syncthreads();
+            add_round(round, kRoundUnits);
+        }
+    };
+    const uint32_t i0 = wave < n_items ? wave : n_items;
+    mfma_stream<MG, THREADS, false, false, DEPTH, true, true>(smem, y, nb, batch, 0, useq, i0, n_items, row_ptr, park);
+    __syncthreads();
+    add_round(full_rounds, ucount - full_rounds * kRoundUnits);   // the units left over
+
+    // every thread holds a best for activation row thread % MP: a tree over the threads of equal row
+    __shared__ float sv[THREADS];
+    __shared__ int si[THREADS];
+    sv[threadIdx.x] = bv;
+    si[threadIdx.x] = bi;
+    __syncthreads();
+    const uint32_t j = threadIdx.x / MP;
+    for (uint32_t stride = THREADS / MP / 2; stride > 0; stride >>= 1) {
+        if (j < stride) {
+            const uint32_t o = threadIdx.x + stride * MP;
+            if (beats(sv[o], si[o], sv[threadIdx.x], si[threadIdx.x])) { sv[threadIdx.x] = sv[o]; si[threadIdx.x] = si[o]; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x < batch) {
+        q8mi_argmax_pair *p = partial + static_cast<uint64_t>(threadIdx.x) * gridDim.x + blockIdx.x;
+        p->value = sv[threadIdx.x];
+        p->index = si[threadIdx.x];
+    }
+}
+
 // One wave per verify row merges that row's partials (each lane a strided share, then a butterfly
 // over the lanes; the merge rule does not depend on the order); thread 0 then walks the drafts.
 constexpr int kFinalizeThreads = Q8MI_MAX_GEMV_BATCH * kWave;
@@ -355,9 +465,28 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
                         q8mi_argmax_pair *partial, float *logits, uint32_t stride_logits, uint32_t *grid_out,
                         hipStream_t stream) {
     constexpr int THREADS = 512;
-    auto kern = lm_head_mfma_kernel<MG, THREADS>;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     const uint32_t units = (rows + kMfmaUnitRows - 1) / kMfmaUnitRows;
+    if constexpr (MG <= 2) {   // items dealt round-robin to the waves, units in rounds
+        const uint32_t x_bytes = mfma_x_lds_bytes(nb, batch, MG);
+        const uint32_t nitems = (nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
+        const uint64_t park = 2ull * lm_head_round_units(MG) * nitems * kMfmaUnitRows * 4 * MG * 4;
+        constexpr uint32_t kDynLimit = kLdsLimit - THREADS * 8 - 256;   // static LDS: the argmax tree
+        if (x_bytes + park <= kDynLimit) {
+            auto kern = logits != nullptr ? lm_head_items_kernel<MG, THREADS, kLmHeadItemsDepth, true>
+                                          : lm_head_items_kernel<MG, THREADS, kLmHeadItemsDepth, false>;
+            static KernelGeometry geometry[2];
+            if (!geometry[logits != nullptr].grant(reinterpret_cast<const void *>(kern), kDynLimit))
+                return fail(Q8MI_LAUNCH_ERROR, "lm_head: cannot reserve %u bytes of LDS", kDynLimit);
+            uint32_t grid = cus < units ? cus : units;
+            if (grid > kMaxPartials) grid = kMaxPartials;
+            *grid_out = grid;
+            kern<<<grid, THREADS, x_bytes + static_cast<uint32_t>(park), stream>>>(w, y, rows, nb, batch, partial, logits,
+                                                                                  stride_logits, kGemvInterleave, x_bytes);
+            return check_launch("lm_head");
+        }
+    }
+    auto kern = lm_head_mfma_kernel<MG, THREADS>;
     // One workgroup per CU, the geometry of the GEMV's matrix-core launch; the kernel parks only the
     // units its waves share (two slots per wave), so the LDS need does not depend on the row count.
     const uint32_t x_bytes = mfma_x_lds_bytes(nb, batch, MG);
