@@ -504,15 +504,14 @@ int launch_lm_head_mfma(const uint8_t *w, const uint8_t *y, uint32_t rows, uint3
     return check_launch("lm_head");
 }
 
-// Which variant streams the weight: the matrix-core one from 3 verify rows on, at 2 rows for weights
-// of fewer than 16384 rows (the same family and
-// geometry as q8mi_gemv at that batch, so the optional logits are the GEMV's bits) whenever the
+// Which variant streams the weight: the matrix-core one from 2 verify rows on, whenever the
 // activations fit LDS beside the parked sums.  Measured on the 248 320-row vocabulary, dot-product
-// against matrix-core variant: 220 / 209 us at 3 rows, 216 / 212 at 4, 227 / 221 at 5, 234 / 225 at 6,
-// 296 / 230 at 8.
+// against matrix-core variant (items dealt round-robin, units in rounds): 197 / 198 us at 1 row,
+// 206 / 194 at 2, 216 / 195 at 4, 234 / 201 at 6, 296 / 201 at 8.
 bool lm_head_uses_mfma(uint32_t rows, uint32_t nb, uint32_t batch) {
+    (void)rows;
     const uint32_t mg = (batch + 3) / 4;
-    if (batch < 3 && !gemv_prefers_mfma((static_cast<uint64_t>(rows) + 1) / 2, batch, nb, false)) return false;   // 2 rows: q8mi_gemv's own rule
+    if (batch < 2) return false;
     return mfma_x_lds_bytes(nb, batch, mg) + 16u * 1024u <= kLdsLimit - 256;
 }
 

@@ -153,13 +153,13 @@ def test_lm_head_fused_matches_unfused_and_oracle(gpu, oracle, batch):
             assert np.allclose(pairs["value"], ref_pairs["value"], rtol=1e-5, atol=1e-6)
             if lg is not None:
                 # the winners are the kernel's own logits; every logit is within the GEMV's tolerance
-                # of the oracle's, and up to two rows (where head and GEMV add in the same order)
-                # equal the plain GEMV's bit for bit
+                # of the oracle's, and one row (where head and GEMV add in the same order) equals the
+                # plain GEMV's bit for bit
                 assert np.array_equal(pairs["value"].view(np.uint32),
                                       lg[np.arange(batch), pairs["index"]].view(np.uint32))
                 rc, mag = oracle.gemv_abs(w, y, vocab, cols, batch)
                 assert_close_fp32(lg, ref_logits, mag, f"fused head logits, batch {batch}")
-                if batch <= 2:
+                if batch == 1:
                     out = hip.DeviceBuffer(4 * batch * vocab)
                     ok(q8mi.lib().q8mi_gemv(dw.ptr, dy.ptr, out.ptr, vocab, cols, batch, vocab, NULL), "gemv")
                     hip.synchronize()
