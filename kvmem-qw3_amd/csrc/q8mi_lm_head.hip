@@ -140,8 +140,10 @@ __global__ __launch_bounds__(THREADS) void lm_head_kernel(
 // after the stream.  LDS use does not grow with the number of rows, so one workgroup per CU
 // covers a vocabulary of any size in a single pass.
 // Units per round of the item-wise kernel below: with 512 threads and four (eight) activation rows
-// 128 (64) units give every thread four triples to add up per round.
-__host__ __device__ constexpr uint32_t lm_head_round_units(int mg) { return mg == 2 ? 64u : 128u; }
+// 64 (32) units give every thread two triples to add up per round.  Measured on the 248 320 x 5120
+// vocabulary at 2 / 4 / 8 rows: rounds of 32 (16) units 193 / 194 / 205 us, 64 (32) units
+// 192 / 192 / 202, 128 (64) units 195 / 195 / 201 .. 207; two items in flight per wave 206 / 206 / 208.
+__host__ __device__ constexpr uint32_t lm_head_round_units(int mg) { return mg == 2 ? 32u : 64u; }
 constexpr int kLmHeadItemsDepth = 1;   // items a wave keeps in flight in that kernel
 
 template <int MG, int THREADS>
