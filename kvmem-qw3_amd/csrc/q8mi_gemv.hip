@@ -338,6 +338,9 @@ int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     static KernelGeometry geometry[2][2];
     // Items dealt round-robin to the waves wherever every item's sums fit LDS beside the activations
     // (up to eight activation rows, one item in flight per wave); else contiguous ranges per wave.
+    // (With nine to sixteen rows, the D4 route of the GEMM's small batches, an item's arithmetic is
+    // long enough to want a second item on its way, and the item-wise form then loses: 17408 x 5120
+    // at batch 16 27.9 us by ranges, 30.8 item-wise with two items in flight, 31.6 with one.)
     if constexpr (MG <= 2 && DEPTH == 1) {
         const uint64_t item_park = static_cast<uint64_t>(per_group) * nitems * kMfmaUnitRows * 4 * MG * 4;
         if (p.x_bytes + item_park <= kDynLimit) {
