@@ -249,6 +249,35 @@ def test_lm_head_full_vocabulary(gpu, oracle, full_head, batch):
             assert np.array_equal(pairs["value"].view(np.uint32), lg[np.arange(batch), tokens].view(np.uint32))
 
 
+@pytest.mark.parametrize("batch", [3, 5, 8])
+def test_lm_head_several_rounds_ragged(gpu, oracle, batch):
+    """A head whose workgroups take their units in several whole rounds and a partial one (97 or 98
+    units of two items per workgroup), with a row count that is no multiple of four: tokens, accept
+    result and every logit against the oracle, with and without the optional logits."""
+    vocab, cols = 100003, 2048
+    w = synth.q8_0_weight(vocab, cols, seed=1300)
+    x = synth.normal(batch, cols, seed=1310 + batch)
+    dw = dev(w)
+    dy, y = quantize_q8_1(x)
+    rc, ref = oracle.gemv(w, y, vocab, cols, batch, threads=16)
+    rc, absum = oracle.gemv_abs(w, y, vocab, cols, batch)
+    tokens = oracle.argmax_rows_scan(ref, batch, vocab)["index"]
+    top2 = np.partition(ref, -2, axis=1)[:, -2:]
+    assert np.all(top2[:, 1] - top2[:, 0] > 1e-4 * np.abs(top2[:, 1]))
+    for prefix, want_logits in ((0, True), (batch - 1, False)):
+        drafts = np.full(batch - 1, 7, np.int32)
+        drafts[:prefix] = tokens[:prefix]
+        if prefix < batch - 1 and drafts[prefix] == tokens[prefix]:
+            drafts[prefix] = 8
+        exp_len, exp_next = oracle.accept(tokens, drafts, eos=2)
+        pairs, n_acc, nxt, lg = run_lm_head(dw, dy, vocab, cols, batch, drafts, 2, want_logits=want_logits, on_device=False)
+        assert np.array_equal(pairs["index"], tokens), "row argmax tokens differ"
+        assert (n_acc, nxt) == (exp_len, exp_next)
+        if lg is not None:
+            assert_close_fp32(lg, ref, absum, f"fused head logits, ragged head, batch {batch}")
+            assert np.array_equal(pairs["value"].view(np.uint32), lg[np.arange(batch), tokens].view(np.uint32))
+
+
 @pytest.mark.parametrize("batch", [2, 4, 7])
 def test_lm_head_rows_without_a_number(gpu, oracle, batch):
     """Logits that are NaN never win and a verify row with nothing above -inf has no token (-1, read

@@ -54,6 +54,24 @@ def test_gemv_matches_oracle(gpu, oracle, rows, cols, batch):
         block_dot_check(oracle, dw, w, dy, y, rows, cols, batch, seed=rows + batch, n=1024)
 
 
+@pytest.mark.parametrize("rows,cols,batch", [(9001, 17408, 8), (9001, 17408, 3), (40003, 5120, 7), (2049, 8192, 5)])
+def test_gemv_matrix_core_splits(gpu, oracle, rows, cols, batch):
+    """Both ways the matrix-core kernel splits a workgroup's items over its waves: round-robin with
+    every item's sums parked (40003 x 5120 and 2049 x 8192: several units per workgroup, a ragged
+    last unit), and contiguous ranges where those sums do not fit LDS beside the activations
+    (9001 x 17408: nine units of seventeen items per workgroup next to eight rows of 17408 columns)."""
+    w = synth.q8_0_weight(rows, cols, seed=rows + cols)
+    x = synth.normal(batch, cols, seed=batch + cols)
+    dw = dev(w)
+    dy, y = quantize_q8_1(x)
+    out = hip.DeviceBuffer(4 * batch * rows).fill(0xff)
+    ok(q8mi.lib().q8mi_gemv(dw.ptr, dy.ptr, out.ptr, rows, cols, batch, rows, NULL), "gemv")
+    hip.synchronize()
+    rc, ref = oracle.gemv(w, y, rows, cols, batch, threads=16)
+    rc, absum = oracle.gemv_abs(w, y, rows, cols, batch)
+    assert_close_fp32(out.download(np.float32).reshape(batch, rows), ref, absum, f"gemv {rows}x{cols} M={batch}")
+
+
 @pytest.mark.parametrize("offset", [4, 8, 12])
 @pytest.mark.parametrize("batch", [1, 2, 4, 8])
 def test_gemv_activations_on_a_4_byte_boundary(gpu, oracle, offset, batch):
