@@ -315,9 +315,9 @@ int q8mi_lm_head_argmax_accept(const uint8_t *weight, const void *y_q8_1, uint32
  * partials go to a 64 KiB array the library holds in every GPU's memory from load to exit
  * (8 verify rows x 1024 workgroups, the most any call needs; a shape that would need more is
  * Q8MI_REJECTED).  The call allocates and frees nothing.  Its first call on a device looks the
- * array's address up, and the first call of every (rows, cols, batch) combination asks the runtime
- * for the LDS grant and the occupancy of the kernel instantiation it picks: make one eager call
- * of each combination that will be captured before capturing it.  Every call on one GPU uses that GPU's
+ * array's address up, and the first call of every (rows, cols, batch, logits or none) combination
+ * asks the runtime for the LDS grant and the occupancy of the kernel instantiation it picks: make
+ * one eager call of each combination that will be captured before capturing it.  Every call on one GPU uses that GPU's
  * one array: calls that overlap on the same GPU (two streams, two threads) race on it and must be
  * serialised by the caller; nothing in it needs clearing between calls. */
 int q8mi_lm_head_argmax_accept_static(const uint8_t *weight, const void *y_q8_1, uint32_t rows, uint32_t cols,
