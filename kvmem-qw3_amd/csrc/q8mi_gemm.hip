@@ -603,32 +603,25 @@ __device__ __forceinline__ void wait_ring(uint32_t steps) {
 // SILU (RB even): the first RB / 2 blocks of 32 LDS rows hold rows of the gate weight `w`, the others
 // the same rows of the up weight `w2`; the tile yields 16 * RB rows of silu(gate) * up and `rows`
 // counts the rows of one weight.
-template <int CB, int W, int NS, bool KSPLIT, int RB = 1, bool SILU = false>
-__global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
-        const uint8_t *__restrict__ w, const uint8_t *__restrict__ w2, const uint8_t *__restrict__ y, const TileOut out,
-        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t row_tiles, uint32_t col_tiles) {
-    constexpr bool ksplit = KSPLIT;
-    static_assert(!KSPLIT || (RB == 1 && !SILU), "only the narrowest tile is cut along K");
+// One tile (row tile rt, column tile ct) over the super-blocks sb0 .. sb0 + nsb - 1 of K.  ATOMIC: the
+// sums are added into dst (a tile whose K range is shared by two workgroups, dst zeroed before the
+// launch); else they are stored through the launch's epilogue.  Every wave of the workgroup calls it.
+template <int CB, int W, int NS, bool ATOMIC, int RB, bool SILU>
+__device__ __forceinline__ void ring_tile_segment(
+        uint8_t *smem, const uint8_t *__restrict__ w, const uint8_t *__restrict__ w2, const uint8_t *__restrict__ y,
+        const TileOut &out, uint32_t rows, uint32_t nb, uint32_t batch, uint32_t rt, uint32_t ct, uint32_t sb0, uint32_t nsb) {
+    static_assert(!ATOMIC || !SILU, "a SwiGLU tile needs its whole sums");
     static_assert(!SILU || RB % 2 == 0, "a SwiGLU tile holds as many gate rows as up rows");
     using T = RingTile<CB, W, RB>;
     constexpr uint32_t S = T::kShares;
     constexpr uint32_t kOut = SILU ? T::kRows / 2 : T::kRows;   // output rows of a tile
     const uint32_t stride_dst = out.stride_dst;
-    extern __shared__ __align__(16) uint8_t smem[];
     const uint32_t lane = threadIdx.x % kWave;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t l32 = lane & 31u, lhalf = lane >> 5;
     const uint32_t grp = wave % CB, share = wave / CB;   // activation group, K share
-    // ksplit: every tile is computed by two workgroups, one per half of K, which add their sums
-    // into a zeroed dst (see launch_ring)
-    const uint32_t id = ksplit ? blockIdx.x >> 1 : blockIdx.x, k_half = ksplit ? blockIdx.x & 1u : 0u;
-    const uint32_t xcd = id % 8u, seq = id / 8u;
-    const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
-    if (rt >= row_tiles) return;   // uniform for the workgroup
     const uint32_t row0 = rt * kOut, col0 = ct * T::kCols;
     const uint32_t nsb_all = nb / 4;
-    const uint32_t sb0 = (ksplit && k_half) ? nsb_all / 2 : 0u;                   // first super-block of this workgroup
-    const uint32_t nsb = ((ksplit && !k_half) ? nsb_all / 2 : nsb_all) - sb0;     // and how many it covers
     const uint64_t row_bytes = static_cast<uint64_t>(nb) * 34;
 
     // The pieces of a step this wave loads: kind and LDS position are wave-uniform, the per-lane
@@ -745,7 +738,7 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
         const uint32_t j = col0 + grp * 32 + 8 * (v / 4) + 4 * lhalf + (v % 4);
         if (r_out < rows && j < batch) {
             const uint64_t idx = static_cast<uint64_t>(j) * stride_dst + r_out;
-            if constexpr (KSPLIT) unsafeAtomicAdd(static_cast<float *>(out.dst) + idx, value);   // two addends onto zero: order-independent
+            if constexpr (ATOMIC) unsafeAtomicAdd(static_cast<float *>(out.dst) + idx, value);   // two addends onto zero: order-independent
             else if constexpr (SILU) static_cast<float *>(out.dst)[idx] = value;
             else emit(out, idx, value);
         }
@@ -784,6 +777,55 @@ __global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
                 if constexpr (SILU) store(rb, v, silu_mul(total_of(rb, v), total_of(rb + RB / 2, v)));
                 else store(rb, v, total_of(rb, v));
             }
+    }
+}
+
+template <int CB, int W, int NS, bool KSPLIT, int RB = 1, bool SILU = false>
+__global__ __launch_bounds__(kWave * W) void gemm_d4_ring_kernel(
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ w2, const uint8_t *__restrict__ y, const TileOut out,
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t row_tiles, uint32_t col_tiles) {
+    static_assert(!KSPLIT || (RB == 1 && !SILU), "only the narrowest tile is cut along K");
+    extern __shared__ __align__(16) uint8_t smem[];
+    // KSPLIT: every tile is computed by two workgroups, one per half of K, which add their sums
+    // into a zeroed dst (see launch_ring)
+    const uint32_t id = KSPLIT ? blockIdx.x >> 1 : blockIdx.x, k_half = KSPLIT ? blockIdx.x & 1u : 0u;
+    const uint32_t xcd = id % 8u, seq = id / 8u;
+    const uint32_t rt = (seq / col_tiles) * 8u + xcd, ct = seq % col_tiles;
+    if (rt >= row_tiles) return;   // uniform for the workgroup
+    const uint32_t nsb_all = nb / 4;
+    const uint32_t sb0 = (KSPLIT && k_half) ? nsb_all / 2 : 0u;                   // first super-block of this workgroup
+    const uint32_t nsb = ((KSPLIT && !k_half) ? nsb_all / 2 : nsb_all) - sb0;     // and how many it covers
+    ring_tile_segment<CB, W, NS, KSPLIT, RB, SILU>(smem, w, w2, y, out, rows, nb, batch, rt, ct, sb0, nsb);
+}
+
+// The same tiles with the K steps of all tiles dealt out evenly: workgroup i takes the steps
+// [total i / G, total (i + 1) / G) of the tile-major step sequence, i.e. the end of one tile, whole
+// tiles, and the start of another.  For launches with a few more tiles than the chip holds
+// workgroups (17408 rows in 64 x 64 tiles at batch 128: 544 tiles for 512 slots), where a last round
+// of a few tiles otherwise lasts as long again as half a round.  A range is at least one tile long,
+// so a tile's K range is shared by at most two workgroups: its sums are added into a dst zeroed by
+// gemm_zero_dst_kernel (two addends onto zero: results repeat bit for bit); tiles that one workgroup
+// covers alone are stored.  Workgroups of one XCD (index % 8) take neighbouring ranges.
+template <int CB, int W, int NS, int RB>
+__global__ __launch_bounds__(kWave * W) void gemm_d4_ring_balanced_kernel(
+        const uint8_t *__restrict__ w, const uint8_t *__restrict__ y, const TileOut out,
+        uint32_t rows, uint32_t nb, uint32_t batch, uint32_t tiles, uint32_t col_tiles) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const uint32_t nsb_all = nb / 4;
+    const uint64_t total = static_cast<uint64_t>(tiles) * nsb_all;
+    const uint32_t groups = gridDim.x;                                   // a multiple of 8
+    const uint32_t index = (blockIdx.x % 8u) * (groups / 8u) + blockIdx.x / 8u;
+    uint64_t step = total * index / groups;
+    const uint64_t end = total * (index + 1) / groups;
+    while (step < end) {
+        const uint32_t tile = static_cast<uint32_t>(step / nsb_all), sb0 = static_cast<uint32_t>(step % nsb_all);
+        const uint64_t left = end - step;
+        const uint32_t nsb = left < nsb_all - sb0 ? static_cast<uint32_t>(left) : nsb_all - sb0;
+        const uint32_t rt = tile / col_tiles, ct = tile % col_tiles;
+        if (nsb == nsb_all) ring_tile_segment<CB, W, NS, false, RB, false>(smem, w, nullptr, y, out, rows, nb, batch, rt, ct, 0, nsb);
+        else ring_tile_segment<CB, W, NS, true, RB, false>(smem, w, nullptr, y, out, rows, nb, batch, rt, ct, sb0, nsb);
+        step += nsb;
+        __syncthreads();   // the stages (and the partial sums kept in them) are free for the next tile
     }
 }
 
@@ -919,6 +961,29 @@ bool ring_splits_k(uint32_t rows, uint32_t nb, uint32_t batch) {
            nb / 4 >= 8;
 }
 
+// Workgroups a balanced launch of these tiles uses: two per CU for the four-wave tile, one for the
+// eight- and sixteen-wave tiles (measured on MI355X at 17408 x 5120: batch 32 in 32 x 32 tiles, 544
+// tiles: one round of 512 and a rest 40.2 us, 512 ranges 32.7; batch 64 in 64 x 64 tiles, 272 tiles:
+// as 272 workgroups 50.1 us, 256 ranges 37.5, and two ranges per CU no better than the 50; batch 128,
+// 544 tiles: 63.3 us as they come, 63.9 in 256 ranges, 69.5 in 512).
+template <int CB, int W, int NS, int RB>
+uint32_t ring_balanced_slots() {
+    constexpr uint32_t lds = NS * RingTile<CB, W, RB>::kStage;
+    constexpr uint32_t per_cu = (W <= 4 && 2 * lds <= 160u * 1024u) ? 2 : 1;   // 160 KB of LDS per CU
+    return per_cu * static_cast<uint32_t>(device_cu_count()) / 8u * 8u;
+}
+
+// Whether a plain-store launch of these tiles deals the K steps of all tiles out evenly (see
+// gemm_d4_ring_balanced_kernel): a few more tiles than the chip holds workgroups, so that the last
+// round would be at most half full.
+template <int CB, int W, int NS, int RB>
+bool ring_balances(uint32_t rows, uint32_t batch) {
+    using T = RingTile<CB, W, RB>;
+    const uint64_t tiles = static_cast<uint64_t>((rows + T::kRows - 1) / T::kRows) * ((batch + T::kCols - 1) / T::kCols);
+    const uint32_t slots = ring_balanced_slots<CB, W, NS, RB>();
+    return slots >= 8 && tiles > slots && tiles % slots != 0 && tiles % slots <= slots / 2 && tiles < 0x7fffffffull;
+}
+
 template <int CB, int W, int NS, int RB = 1, bool SILU = false>
 int launch_ring(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, hipStream_t stream) {
     using T = RingTile<CB, W, RB>;
@@ -927,6 +992,28 @@ int launch_ring(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, h
     const uint32_t col_tiles = (batch + T::kCols - 1) / T::kCols;
     const uint64_t grid64 = static_cast<uint64_t>((row_tiles + 7u) / 8u * 8u) * col_tiles;
     if (grid64 > 0x3fffffffull) return fail(Q8MI_REJECTED, "gemm: too many tiles");
+    if constexpr (!SILU) {
+        // A few more tiles than the chip holds workgroups: the K steps of all tiles dealt out evenly
+        // (see gemm_d4_ring_balanced_kernel) instead of a short last round.
+        if (c.out.epi == kEpiStore && ring_balances<CB, W, NS, RB>(rows, batch)) {
+            constexpr int lds = NS * T::kStage;
+            static std::atomic<bool> granted{false};   // two threads may both get here first: the grant is idempotent
+            if (!granted) {
+                if (lds > 64 * 1024 &&
+                    hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_d4_ring_balanced_kernel<CB, W, NS, RB>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+                    (void)hipGetLastError();
+                    return fail(Q8MI_LAUNCH_ERROR, "gemm: cannot reserve %d bytes of LDS", lds);
+                }
+                granted = true;
+            }
+            gemm_zero_dst_kernel<<<dim3((rows + 1023u) / 1024u, batch), 256, 0, stream>>>(
+                static_cast<float *>(c.out.dst), rows, c.out.stride_dst);
+            gemm_d4_ring_balanced_kernel<CB, W, NS, RB><<<ring_balanced_slots<CB, W, NS, RB>(), kWave * W, lds, stream>>>(
+                c.w, c.y, c.out, rows, nb, batch, row_tiles * col_tiles, col_tiles);
+            return check_launch("gemm");
+        }
+    }
     if constexpr (CB == 1 && RB == 1 && !SILU) {
         if (c.out.epi == kEpiStore && ring_splits_k(rows, nb, batch)) {
             gemm_zero_dst_kernel<<<dim3((rows + 1023u) / 1024u, batch), 256, 0, stream>>>(
@@ -948,6 +1035,21 @@ bool uses_main_tiles(uint32_t rows, uint32_t batch) {
     const uint64_t slots = 2ull * static_cast<uint32_t>(device_cu_count());
     const uint64_t tiles = static_cast<uint64_t>((rows + kTileRows - 1) / kTileRows) * ((batch + kTileCols - 1) / kTileCols);
     return tiles * 5 >= slots * 2;
+}
+
+// Whether q8mi_gemm sums some tiles of this shape from two ranges of K (ring tiles with their K steps
+// dealt out evenly): the fused-store entry points then decline, as for the other K splits.  Follows
+// the tile choice of launch_gemm_dma below.
+bool plain_gemm_balances(uint32_t rows, uint32_t nb, uint32_t batch) {
+    if (uses_main_tiles(rows, batch)) return false;
+    const uint32_t cus = static_cast<uint32_t>(device_cu_count());
+    if (batch > 32 && batch <= 128 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * cus)
+        return ring_balances<2, kRingWaves2, kRing2, 2>(rows, batch);
+    if (batch <= 32) return !ring_splits_k(rows, nb, batch) && ring_balances<1, 4, kRing1, 1>(rows, batch);
+    if (batch <= 64) return ring_balances<2, kRingWaves2, kRing2, 1>(rows, batch);
+    const uint64_t ring_tiles = static_cast<uint64_t>((rows + 31u) / 32u) * ((batch + 127u) / 128u);
+    if (ring_tiles <= cus) return ring_balances<4, 16, kRing4, 1>(rows, batch);
+    return ring_balances<4, kRingWaves4, kRing4, 1>(rows, batch);
 }
 
 int launch_gemm_dma(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batch, hipStream_t stream) {
@@ -1040,10 +1142,12 @@ extern "C" int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *
     return launch_gemm_d4(weight, y_d4, dst, rows, cols, batch, stride_dst_row, as_stream(stream));
 }
 
-// Shapes whose plain GEMM cuts its last round of main tiles in two along K keep that route (the
-// caller runs q8mi_gemm and the second step): there it is the faster one.
+// Shapes whose plain GEMM cuts its last round of main tiles in two along K, or deals the K steps of
+// its ring tiles out evenly, keep that route (the caller runs q8mi_gemm and the second step): there
+// it is the faster one.
 static bool plain_gemm_splits(uint32_t rows, uint32_t cols, uint32_t batch) {
-    return uses_main_tiles(rows, batch) && split_round_tiles(rows, cols / kQK, batch) != 0;
+    return (uses_main_tiles(rows, batch) && split_round_tiles(rows, cols / kQK, batch) != 0) ||
+           plain_gemm_balances(rows, cols / kQK, batch);
 }
 
 extern "C" int q8mi_gemm_add(const uint8_t *weight, const void *y_d4, const float *residual, float *dst, uint32_t rows,
@@ -1058,7 +1162,7 @@ extern "C" int q8mi_gemm_add(const uint8_t *weight, const void *y_d4, const floa
     if (batch <= 32 && ring_splits_k(rows, cols / kQK, batch))
         return fail(Q8MI_REJECTED, "gemm_add: this shape is summed from two halves of K (use q8mi_gemm, then q8mi_add)");
     if (plain_gemm_splits(rows, cols, batch))
-        return fail(Q8MI_REJECTED, "gemm_add: the last round of this shape is summed from two halves of K (use q8mi_gemm, then q8mi_add)");
+        return fail(Q8MI_REJECTED, "gemm_add: some tiles of this shape are summed from two ranges of K (use q8mi_gemm, then q8mi_add)");
     return launch_gemm_dma(TileCall{weight, nullptr, static_cast<const uint8_t *>(y_d4),
                                     TileOut{dst, residual, stride_dst_row, kEpiAdd}},
                            rows, cols / kQK, batch, as_stream(stream));
@@ -1072,7 +1176,7 @@ extern "C" int q8mi_gemm_bf16(const uint8_t *weight, const void *y_d4, uint16_t 
     if (batch <= 32 && ring_splits_k(rows, cols / kQK, batch))
         return fail(Q8MI_REJECTED, "gemm_bf16: this shape is summed from two halves of K (use q8mi_gemm, then q8mi_f32_to_bf16)");
     if (plain_gemm_splits(rows, cols, batch))
-        return fail(Q8MI_REJECTED, "gemm_bf16: the last round of this shape is summed from two halves of K (use q8mi_gemm, then q8mi_f32_to_bf16)");
+        return fail(Q8MI_REJECTED, "gemm_bf16: some tiles of this shape are summed from two ranges of K (use q8mi_gemm, then q8mi_f32_to_bf16)");
     return launch_gemm_dma(TileCall{weight, nullptr, static_cast<const uint8_t *>(y_d4),
                                     TileOut{dst, nullptr, stride_dst_row, kEpiStoreBf16}},
                            rows, cols / kQK, batch, as_stream(stream));

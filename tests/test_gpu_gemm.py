@@ -136,6 +136,38 @@ def test_gemm_narrow_tiles_split_along_k_are_deterministic(gpu, oracle):
     assert_close_fp32(first[jj.reshape(-1), rr.reshape(-1)], ref_s, absum, "narrow tiles, K split")
 
 
+@pytest.mark.parametrize("rows,cols,batch", [(17408, 1024, 20), (17408, 1024, 32), (17500, 512, 64), (17408, 768, 100)])
+def test_gemm_ring_tiles_with_their_k_steps_dealt_out_evenly(gpu, oracle, rows, cols, batch):
+    """A few more ring tiles than the chip holds workgroups (544 tiles of 32 x 32 for 512 slots, 272
+    or 274 or 544 tiles of 64 x 64 for 256): every workgroup takes an equal range of the K steps of
+    all tiles, tiles shared by two workgroups are added into a zeroed output.  Every output against
+    the oracle, a wider stride left alone, repeated calls and graph replays bit for bit."""
+    w = synth.q8_0_weight(rows, cols, seed=rows + cols + batch)
+    dw = dev(w)
+    dy, y = quantize_d4(synth.normal(batch, cols, seed=batch + 3))
+    rc, ref = oracle.gemm_d4(w, y, rows, cols, batch, threads=8)
+    rr, jj = np.meshgrid(np.arange(rows, dtype=np.uint32), np.arange(batch, dtype=np.uint32))
+    rc, _, absum = oracle.gemm_d4_sampled(w, y, rows, cols, batch, rr.reshape(-1), jj.reshape(-1))
+    stride = rows + 12
+    first = run_gemm(dw, dy, rows, cols, batch, stride=stride)
+    assert_close_fp32(first[:, :rows], ref, absum, f"gemm ring tiles, K steps dealt out, batch {batch}")
+    assert np.all(first[:, rows:].view(np.uint32) == 0xffffffff), "stores must stay inside the rows"
+    for _ in range(2):
+        assert np.array_equal(run_gemm(dw, dy, rows, cols, batch, stride=stride).view(np.uint32), first.view(np.uint32))
+    out = hip.DeviceBuffer(4 * batch * stride).fill(0xff)
+    stream = hip.Stream()
+    g = hip.Graph(stream)
+    with g:
+        ok(q8mi.lib().q8mi_gemm(dw.ptr, dy.ptr, out.ptr, rows, cols, batch, stride, stream.handle), "gemm")
+    for replay in range(2):
+        g.launch()
+        stream.synchronize()
+        got = out.download(np.float32).reshape(batch, stride)
+        assert np.array_equal(got[:, :rows].view(np.uint32), first[:, :rows].view(np.uint32)), f"replay {replay}"
+        out.fill(0x7f)
+        hip.synchronize()
+
+
 def test_gemm_split_last_round_replays_in_a_graph(gpu):
     """The two-kernel call (zeroing kernel + GEMM with a K-split last round) captured into a HIP
     graph: every replay, onto an output poisoned in between, gives the eager call's bits."""

@@ -131,7 +131,7 @@ def test_gemm_silu_mul_prefill_chunk(gpu, oracle):
 
 # rows, cols, batch, in place
 ADD_SHAPES = [(384, 1024, 40, True), (384, 1024, 64, False), (1000, 512, 300, True), (6656, 512, 512, True),
-              (6656, 512, 500, False), (384, 1024, 12, True), (17408, 5120, 64, True)]
+              (6656, 512, 500, False), (384, 1024, 12, True), (5120, 5120, 64, True)]
 
 
 @pytest.mark.parametrize("rows,cols,batch,in_place", ADD_SHAPES)
@@ -169,6 +169,7 @@ def test_gemm_add_declines_what_it_cannot_fuse(gpu):
     L = q8mi.lib()
     cases = [(384, 1024, 32, True),      # one 32-row tile per CU at most: cut along K
              (5120, 1024, 2048, True),   # 640 main tiles: the last round of 128 is cut along K
+             (17408, 512, 64, True),     # 272 tiles of 64 x 64 for 256 CUs: their K steps are dealt out evenly
              (384, 1024, 12, False)]     # a weight stream adds in place only
     for rows, cols, batch, in_place in cases:
         dw = dev(synth.q8_0_weight(rows, cols, seed=1))
