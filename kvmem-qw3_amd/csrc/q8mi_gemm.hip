@@ -1044,7 +1044,8 @@ bool plain_gemm_balances(uint32_t rows, uint32_t nb, uint32_t batch) {
     if (uses_main_tiles(rows, batch)) return false;
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     if (batch > 32 && batch <= 128 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * cus)
-        return ring_balances<2, kRingWaves2, kRing2, 2>(rows, batch);
+        return (batch > 64 && ring_balances<4, kRingWaves4, kRing4, 2>(rows, batch)) ||
+               ring_balances<2, kRingWaves2, kRing2, 2>(rows, batch);
     if (batch <= 32) return !ring_splits_k(rows, nb, batch) && ring_balances<1, 4, kRing1, 1>(rows, batch);
     if (batch <= 64) return ring_balances<2, kRingWaves2, kRing2, 1>(rows, batch);
     const uint64_t ring_tiles = static_cast<uint64_t>((rows + 31u) / 32u) * ((batch + 127u) / 128u);
@@ -1059,9 +1060,15 @@ int launch_gemm_dma(const TileCall &c, uint32_t rows, uint32_t nb, uint32_t batc
     // 64 x 64 tiles: fewer workgroups re-read the activation records of a step (measured at
     // 17408 x 5120: batch 64 59 -> 51 us; batch 128, two column tiles of 64 against one 32-row tile
     // 128 wide, 75.9 -> 66.3 us).  The 32- and 128-row-wide tiles lose with 64 rows (54 against
-    // 43 us, 88 against 77 us): their rings then leave room for one workgroup per CU only.
-    if (batch > 32 && batch <= 128 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * static_cast<uint32_t>(device_cu_count()))
+    // 43 us, 88 against 77 us): their rings then leave room for one workgroup per CU only.  That is
+    // no drawback once the K steps of all tiles are dealt out evenly to one workgroup per CU: with
+    // 65..128 activation rows a 64-row tile 128 wide then reads every weight byte once (17408 x 5120,
+    // batch 128: 272 tiles in 256 ranges 56.1 us, against 63.3 .. 63.9 in 64 x 64 tiles either way).
+    if (batch > 32 && batch <= 128 && static_cast<uint64_t>((rows + 31u) / 32u) * 2 >= 3ull * static_cast<uint32_t>(device_cu_count())) {
+        if (batch > 64 && c.out.epi == kEpiStore && ring_balances<4, kRingWaves4, kRing4, 2>(rows, batch))
+            return launch_ring<4, kRingWaves4, kRing4, 2>(c, rows, nb, batch, stream);
         return launch_ring<2, kRingWaves2, kRing2, 2>(c, rows, nb, batch, stream);
+    }
     if (batch <= 32) return launch_ring<1, 4, kRing1>(c, rows, nb, batch, stream);
     if (batch <= 64) return launch_ring<2, kRingWaves2, kRing2>(c, rows, nb, batch, stream);
     // at most one tile per CU: sixteen waves (four K shares per group) instead of eight
