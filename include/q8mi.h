@@ -183,12 +183,13 @@ int q8mi_quantize_q8_1_d4(const float *x, void *y_d4, uint32_t batch, uint32_t c
  * rows >= 128 && cols % 128 == 0 -> y is D4 (144-B super-blocks); otherwise y is
  * Q8_1 (36-B blocks).  Rejects cols % 32 != 0, rows == 0, batch == 0.
  * dst must be ordinary (coarse-grained) device memory: when the 128 x 128 tiles
- * leave a last round that fills at most half of the chip, or when a batch of
- * up to 32 rows gives at most one 32-row tile per CU, those outputs are
- * zeroed by a small kernel and then summed from two halves of K with hardware
- * fp32 atomic adds (two addends onto zero, so results repeat bit for bit); the
- * call then enqueues two kernels instead of one.  The same holds for
- * q8mi_gemm_medium. */
+ * leave a last round that fills at most half of the chip, when a batch of
+ * up to 32 rows gives at most one 32-row tile per CU, or when a medium batch
+ * has a few more 32- or 64-row tiles than the chip holds workgroups (the K
+ * steps of all tiles are then dealt out evenly), those outputs are zeroed by a
+ * small kernel and then summed from two ranges of K with hardware fp32 atomic
+ * adds (two addends onto zero, so results repeat bit for bit); the call then
+ * enqueues two kernels instead of one.  The same holds for q8mi_gemm_medium. */
 int q8mi_gemm(const uint8_t *weight, const void *y, float *dst, uint32_t rows, uint32_t cols,
               uint32_t batch, uint32_t stride_dst_row, void *stream);
 /* replaces launch_mmq_q8_0_medium, src/mmq_q8.cu:2512-2548: y is always D4.
@@ -207,15 +208,15 @@ int q8mi_gemm_medium(const uint8_t *weight, const void *y_d4, float *dst, uint32
  * add_kernel (q8_0_matmul_add, include/qw3/device_backend.hpp:529-540, src/kernels_cuda.cu:11919-11957,
  * 1644-1652); same bits as q8mi_gemm + q8mi_add wherever q8mi_gemm does not sum from two halves of K.
  * Rejected: batch <= 16 out of place (in place the matrix-core GEMV adds as q8mi_gemv_add does), and
- * shapes q8mi_gemm serves by adding two halves of K into a zeroed dst (a partly filled last round of
- * 128 x 128 tiles, or at most one 32-row tile per CU at batch <= 32): a sum that arrives in halves
- * cannot meet the residual in an order that repeats, and on those shapes q8mi_gemm + q8mi_add is the
- * faster route anyway. */
+ * shapes q8mi_gemm serves by adding two ranges of K into a zeroed dst (a partly filled last round of
+ * 128 x 128 tiles, at most one 32-row tile per CU at batch <= 32, a few more ring tiles than the
+ * chip holds workgroups): a sum that arrives in two parts cannot meet the residual in an order that
+ * repeats, and on those shapes q8mi_gemm + q8mi_add is the faster route anyway. */
 int q8mi_gemm_add(const uint8_t *weight, const void *y_d4, const float *residual, float *dst, uint32_t rows,
                   uint32_t cols, uint32_t batch, uint32_t stride_dst_row, void *stream);
 /* q8mi_gemm with bf16 outputs (round to nearest even in the store): replaces launch_mmq_q8_0 into an
  * fp32 workspace followed by convert_q8_output_bf16 (src/kernels_cuda.cu:14509-14530).  Rejected:
- * batch <= 16 (a weight stream: quantize to Q8_1 and use q8mi_gemv_bf16) and the two-halves shapes above. */
+ * batch <= 16 (a weight stream: quantize to Q8_1 and use q8mi_gemv_bf16) and the two-part shapes above. */
 int q8mi_gemm_bf16(const uint8_t *weight, const void *y_d4, uint16_t *dst, uint32_t rows, uint32_t cols,
                    uint32_t batch, uint32_t stride_dst_row, void *stream);
 /* dst[j][r] = silu((Wg x)[j][r]) * (Wu x)[j][r], silu(g) = g / (1 + exp(-g)): the batched SwiGLU the
