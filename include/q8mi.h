@@ -98,12 +98,12 @@ int q8mi_gemv_fanout4(const uint8_t *weight0, const uint8_t *weight1, const uint
  * The results of q8mi_quantize_q8_1 followed by the matching q8mi_gemv* call,
  * in one launch: every workgroup quantizes the fp32 activations
  * (x: [batch][stride_x_row] floats) itself with the quantizer's own arithmetic
- * behind its first weight requests (rows of 4096 / 5120 / 6144 / 7168 / 8192 columns:
+ * behind its first weight requests (rows of 1024, 2048, ... 8192 columns:
  * each wave the 1024 columns it works on, in registers; other lengths: into
  * LDS), so no Q8_1 scratch buffer and no quantizer launch are needed.  The
  * quantized values and the per-block products are the same bits as in the
  * two-step form.  So are the outputs at batch 1 for rows of up to 8192 columns
- * and at batch 2 for the five row lengths above; longer rows, and other lengths
+ * and at batch 2 for those whole numbers of 1024 columns; longer rows, and other lengths
  * at batch 2 (where the Q8_1 entry points may run another kernel), add the same
  * products in another order (inside the GEMV's tolerance).  This is what
  * the reference's operators do in two steps (src/kernels_cuda.cu:10764-10888,

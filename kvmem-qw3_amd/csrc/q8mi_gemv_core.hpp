@@ -440,6 +440,10 @@ constexpr uint32_t kMfmaFromBatch = 2;    // smallest batch served by the matrix
 constexpr uint32_t kPairsMaxBatch = 4;    // largest batch the row-pair family serves
 // Which GEMV family serves a launch of batch 2 and more (measured on MI355X, row-pair kernel with
 // the rows shared by the waves of a workgroup against matrix-core kernel, us):
+//   rows of 1 .. 3 KiB         batch 2: row pairs (5120 rows of 2 KiB: 4.6 / 7.0; 17408 rows of 1 KiB: 5.8 / 11.7 on the ring
+//                              kernel); batch 3 and 4 from 2 KiB: row pairs (17408 x 2048: 9.3 / 12.9 and 10.7 / 13.0;
+//                              5120 x 3072: 6.1 / 7.6 and 6.9 / 7.7); 1 KiB at batch 3 and 4: matrix cores (5120 rows
+//                              5.2 / 4.7 and 5.6 / 4.8)
 //   rows of 4 .. 8 KiB         batch 2: always row pairs (8192 x 5120 fan-out 9.3 / 11.9, SwiGLU 30.2 / 34.1);
 //                              batch 3 and 4: row pairs but for the SwiGLU form (fan-out 10.3 / 11.7 and
 //                              11.4 / 11.7, 5120 x 6144 9.8 / 11 and 10.2 / 11, SwiGLU 32.1 / 31.0 and
@@ -451,8 +455,8 @@ constexpr uint32_t kPairsMaxBatch = 4;    // largest batch the row-pair family s
 inline bool gemv_prefers_mfma(uint64_t row_pairs, uint32_t batch, uint32_t nb, bool silu) {
     if (batch < 2) return false;
     if (batch > kPairsMaxBatch) return true;
-    const bool short_rows = nb % 32 == 0 && nb >= 128 && nb <= 256;   // 4 .. 8 KiB
-    const bool whole_kib = nb % 32 == 0 && nb >= 128 && nb <= 544;     // 4 .. 17 KiB: a shared-row kernel of its own
+    const bool short_rows = nb % 32 == 0 && nb >= 64 && nb <= 256;   // 2 .. 8 KiB
+    const bool whole_kib = nb % 32 == 0 && nb <= 544;                  // 1 .. 17 KiB: a shared-row kernel of its own
     if (batch == 2) return !whole_kib && row_pairs < 8192;
     return !short_rows || silu;
 }

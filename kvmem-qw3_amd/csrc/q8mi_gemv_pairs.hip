@@ -19,12 +19,12 @@
 // over the lanes of equal parity lane 0 holds the first row's result and lane 1 the second's.
 //
 // Two kernels, by where the activations live:
-//   gemv_pairs_ksplit_kernel   rows of 4 to 17 KiB (whole KiB): the waves of a workgroup cut every row
+//   gemv_pairs_ksplit_kernel   rows of 1 to 17 KiB (whole KiB): the waves of a workgroup cut every row
 //       into interleaved 1 KiB steps, so each wave needs the activations of its own steps only,
 //       loads them once into registers (5 per step and activation row) and keeps them for all
 //       pairs of the workgroup; partial sums meet in LDS after the last pair.  With fp32
 //       activations (the entry points that quantize inside the GEMV, optionally after an RMS norm;
-//       rows of 4..8 KiB) every wave quantizes the 1024 floats of its own step in registers,
+//       rows of 1..8 KiB) every wave quantizes the 1024 floats of its own step in registers,
 //       with the stand-alone quantizer's arithmetic; only the norm's sum of squares crosses the
 //       waves, through LDS, in the stand-alone norm's order
 //   gemv_pairs_ring_kernel     any other row length: one wave per pair, the activation bytes of a
@@ -326,7 +326,7 @@ __global__ __launch_bounds__(WAVES * kWave, ksplit_waves_per_simd(M, NSTEPS, WAV
     static_assert((NSTEPS - S * WAVES) * 64 % WAVES == 0 && kTail % 2 == 0, "the left-over steps split evenly");
     constexpr int SL = S + (kTail ? 1 : 0);                        // register slots per wave
     static_assert(!XF32 || (SL == 1 && kTail == 0), "fp32 activations: one step per wave");
-    static_assert(!NORM || (XF32 && M == 1 && WAVES >= 4), "the norm applies to one fp32 row, and its tree needs four waves");
+    static_assert(!NORM || (XF32 && M == 1), "the norm applies to one fp32 row");
     __shared__ float part[kKsplitMaxPairs][WAVES][M][2];
     __shared__ float squares[NORM ? WAVES : 1][NORM ? kNormThreads : 1];
     __shared__ float red[4];
@@ -394,12 +394,27 @@ __global__ __launch_bounds__(WAVES * kWave, ksplit_waves_per_simd(M, NSTEPS, WAV
 #pragma unroll
             for (int i = 0; i < 4; ++i) squares[w][lane * 4 + i] = chunk_squares(xv[0][i]);
             __syncthreads();
-            float partial = 0.0f;
-            if (threadIdx.x < kNormThreads) {
+            float sum_sq;
+            if constexpr (WAVES >= 4) {
+                float partial = 0.0f;
+                if (threadIdx.x < kNormThreads) {
 #pragma unroll
-                for (int u = 0; u < WAVES; ++u) partial += squares[u][threadIdx.x];
+                    for (int u = 0; u < WAVES; ++u) partial += squares[u][threadIdx.x];
+                }
+                sum_sq = first256_tree_sum(partial, red);
+            } else {
+                // fewer than 256 threads: wave w stands in for the waves w, w + WAVES, ... of that tree
+                for (uint32_t g = w; g < 4; g += WAVES) {
+                    float partial = 0.0f;
+#pragma unroll
+                    for (int u = 0; u < WAVES; ++u) partial += squares[u][g * kWave + lane];
+                    const float s = wave_sum(partial);
+                    if (lane == 0) red[g] = s;
+                }
+                __syncthreads();
+                sum_sq = (red[0] + red[1]) + (red[2] + red[3]);
             }
-            const float scale = rms_scale(first256_tree_sum(partial, red), nb * 32, p.eps);
+            const float scale = rms_scale(sum_sq, nb * 32, p.eps);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 xv[0][i] = rms_apply(xv[0][i], scale, nw[i]);
@@ -625,10 +640,11 @@ int ring_or_reject(const GemvParams &p, const PairSpace &ps, hipStream_t stream)
     else return Q8MI_REJECTED;
 }
 
-// Rows of N KiB, N = 4 .. 17 (the reference's kernel is generic in cols % 32, src/mmvq_q8.cu:193-280;
-// here every whole number of KiB from 4 on has an instantiation of the shared-row kernel; shorter
-// rows are launches of a few microseconds whatever reads them), always a split without a left-over
-// step except at 17: one wave per 1 KiB step up to 8 KiB and at 9, 11 and 13; two steps per wave at
+// Rows of N KiB, N = 1 .. 17 (the reference's kernel is generic in cols % 32, src/mmvq_q8.cu:193-280;
+// here every whole number of KiB has an instantiation of the shared-row kernel), always a split
+// without a left-over step except at 17: one wave per 1 KiB step up to 8 KiB and at 9, 11 and 13
+// (5120 rows of 1 / 2 / 3 KiB at batch 1: 3.8 / 4.3 / 5.1 us against 4.4 / 4.9 / 6.0 with one wave per
+// pair and the activations read per step; 17408 rows of 1 KiB: 5.3 against 9.5); two steps per wave at
 // 10, 12, 14 and 16; 15 -> 5 x 3; 17 -> 4 x 4 and a shared last step.  Measured on MI355X at batch 1,
 // 5120 rows, time / plain streaming read of the same bytes: 1.08 .. 1.17 on every length (with four
 // waves and a shared last step 9, 11 and 13 KiB were at 1.30, 1.22, 1.22; 15 KiB on 15 waves 1.28, on
@@ -637,8 +653,10 @@ int ring_or_reject(const GemvParams &p, const PairSpace &ps, hipStream_t stream)
 template <int M>
 int ksplit_by_length(const GemvParams &p, const PairSpace &ps, hipStream_t stream) {
     if (p.nb % 32 != 0) return ring_or_reject<M>(p, ps, stream);
-    if constexpr (M >= 3) {   // batch 3 and 4: the 4..8 KiB rows only (longer rows: the matrix-core kernel)
+    if constexpr (M >= 3) {   // batch 3 and 4: the 2..8 KiB rows only (shorter and longer rows: the matrix-core kernel)
         switch (p.nb / 32) {
+            case 2: return launch_ksplit<M, 2, 2>(p, ps, stream);
+            case 3: return launch_ksplit<M, 3, 3>(p, ps, stream);
             case 4: return launch_ksplit<M, 4, 4>(p, ps, stream);
             case 5: return launch_ksplit<M, 5, 5>(p, ps, stream);
             case 6: return launch_ksplit<M, 6, 6>(p, ps, stream);
@@ -648,6 +666,9 @@ int ksplit_by_length(const GemvParams &p, const PairSpace &ps, hipStream_t strea
         }
     } else {
         switch (p.nb / 32) {
+            case 1: return launch_ksplit<M, 1, 1>(p, ps, stream);
+            case 2: return launch_ksplit<M, 2, 2>(p, ps, stream);
+            case 3: return launch_ksplit<M, 3, 3>(p, ps, stream);
             case 4: return launch_ksplit<M, 4, 4>(p, ps, stream);
             case 5: return launch_ksplit<M, 5, 5>(p, ps, stream);
             case 6: return launch_ksplit<M, 6, 6>(p, ps, stream);
@@ -691,6 +712,9 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
         auto f32_by_cols = [&](auto mtag) -> int {
             constexpr int M = decltype(mtag)::value;
             switch (cols) {
+                case 1024: return launch_ksplit_f32<M, 1>(p, ps, stream);
+                case 2048: return launch_ksplit_f32<M, 2>(p, ps, stream);
+                case 3072: return launch_ksplit_f32<M, 3>(p, ps, stream);
                 case 4096: return launch_ksplit_f32<M, 4>(p, ps, stream);
                 case 5120: return launch_ksplit_f32<M, 5>(p, ps, stream);
                 case 6144: return launch_ksplit_f32<M, 6>(p, ps, stream);
@@ -707,7 +731,7 @@ int launch_pairs(const GemvParams &p, uint32_t batch, hipStream_t stream) {
     }
     if (reinterpret_cast<uintptr_t>(p.y) % 4 != 0) return Q8MI_REJECTED;
     // rows of whole KiB up to 17: shared by the waves of a workgroup, activations in registers
-    // (batch 1 and 2 on every such length, batch 3 and 4 on the 4..8 KiB rows measured for them);
+    // (batch 1 and 2 on every such length, batch 3 and 4 on the 2..8 KiB rows measured for them);
     // any other length: one wave per pair, activations read with every step
     switch (batch) {
         case 1: return ksplit_by_length<1>(p, ps, stream);

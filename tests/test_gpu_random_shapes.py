@@ -66,17 +66,18 @@ def shared_row_cases(seed, n):
     out = [(1, 5120, 1), (2, 5120, 2), (3, 4096, 3), (1, 17408, 2), (5, 8192, 4)]   # fewer rows than a workgroup takes
     for _ in range(n):
         out.append((int(rng.integers(1, 700)), int(rng.choice([4096, 5120, 6144, 8192, 17408])), int(rng.integers(1, 5))))
-    # every whole number of KiB from 4 to 17 at batch 1 and 2 (each has an instantiation of its own)
-    for kib in range(4, 18):
+    # every whole number of KiB up to 17 at batch 1 and 2 (each has an instantiation of its own)
+    for kib in range(1, 18):
         out.append((int(rng.integers(1, 300)), 1024 * kib, 1))
         out.append((int(rng.integers(1, 300)), 1024 * kib, 2))
-    out += [(700, 7168, 3), (333, 12288, 4), (50, 3072, 2), (50, 2560, 1)]   # lengths and batches other kernels serve
+    out += [(700, 2048, 3), (431, 3072, 4), (9000, 2048, 4), (17001, 1024, 2), (300, 1024, 3)]   # 1 .. 3 KiB at batch 2 .. 4
+    out += [(700, 7168, 3), (333, 12288, 4), (50, 3328, 2), (50, 2560, 1)]   # lengths and batches other kernels serve
     return out
 
 
 @pytest.mark.parametrize("rows,cols,batch", shared_row_cases(3, 15))
 def test_gemv_forms_on_rows_with_kernels_of_their_own(gpu, oracle, rows, cols, batch):
-    """Rows of 4 to 17 KiB at batch 1..4 (the waves of a workgroup share the row pairs):
+    """Rows of 1 to 17 KiB at batch 1..4 (the waves of a workgroup share the row pairs):
     plain store into a padded output, residual add, SwiGLU, and the quantizer-inside forms, with
     row counts that leave single-row pairs and workgroups with fewer pairs than they may take."""
     L = gpu.lib()
@@ -122,7 +123,7 @@ def test_gemv_forms_on_rows_with_kernels_of_their_own(gpu, oracle, rows, cols, b
         ok(L.q8mi_qgemv_silu_mul(dw0.ptr, dw1.ptr, dx.ptr, cols, ones.ptr, rows, cols, batch, rows, NULL), "qgemv_silu_mul")
         hip.synchronize()
         got1 = one.download(np.float32).reshape(batch, stride)
-        if cols <= 8192 and (batch == 1 or (cols >= 4096 and cols % 1024 == 0)):   # both forms run the same kernel
+        if cols <= 8192 and (batch == 1 or cols % 1024 == 0):   # both forms run the same kernel
             assert np.array_equal(got1.view(np.uint32), got.view(np.uint32)), "qgemv against gemv"
             assert np.array_equal(ones.download(np.uint32), os_.download(np.uint32)), "qgemv_silu_mul against gemv_silu_mul"
         else:

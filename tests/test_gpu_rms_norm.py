@@ -100,7 +100,7 @@ def test_rms_norm_rejections(gpu):
     ok(L.q8mi_rms_norm(b.ptr, b.ptr, b.ptr, 0, 64, 64, 64, EPS, NULL), "empty batch")
 
 
-@pytest.mark.parametrize("rows,cols", [(333, 6144), (5120, 5120), (201, 4096), (100, 256), (77, 1024), (40, 2304)])
+@pytest.mark.parametrize("rows,cols", [(333, 6144), (5120, 5120), (201, 4096), (100, 256), (77, 1024), (150, 2048), (91, 3072), (40, 2304)])
 def test_nqgemv_equals_norm_then_qgemv(gpu, oracle, rows, cols):
     L = gpu.lib()
     w = synth.q8_0_weight(rows, cols, seed=rows + cols)
