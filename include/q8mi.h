@@ -147,6 +147,16 @@ int q8mi_rms_norm(const float *x, const float *weight, float *out, uint32_t batc
 int q8mi_rms_norm_quantize_q8_1(const float *x, const float *weight, float *normalized, void *y_q8_1,
                                 uint32_t batch, uint32_t cols, uint32_t stride_x_row,
                                 uint32_t stride_normalized_row, float eps, void *stream);
+/* The residual add in front of a norm, in the norm's launch: sum = a + b (rounded as q8mi_add
+ * rounds it; sum may be a or b), then normalized / y_q8_1 = what q8mi_rms_norm /
+ * q8mi_rms_norm_quantize_q8_1 give on sum, bit for bit.  Replaces the pair add_n + rms_norm_batch
+ * of the batched layer loop (src/qwen_executor.cpp:6642-6645 with 6666-6668, and the add_n at
+ * :6693 with the next layer's norm; kernels src/kernels_cuda.cu:14818-14862, 14781-14816).  Rows
+ * of a, b and sum are stride_row floats apart.  normalized may be NULL when y_q8_1 is given and
+ * the other way round; it must not overlap a, b or sum.  y_q8_1 needs cols % 32 == 0. */
+int q8mi_add_rms_norm(const float *a, const float *b, float *sum, const float *weight, float *normalized,
+                      void *y_q8_1, uint32_t batch, uint32_t cols, uint32_t stride_row,
+                      uint32_t stride_normalized_row, float eps, void *stream);
 /* One activation row normalised, quantized and multiplied in ONE launch: what
  * rms_norm_q8_0_matmul_fanout (include/qw3/device_backend.hpp:421-444) and the
  * rms_norm + q8_0_matvec / q8_0_matvec_silu_mul pairs of the decode loop

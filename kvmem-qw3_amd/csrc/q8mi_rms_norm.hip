@@ -12,18 +12,29 @@
 // restated; this kernel fixes an order of its own (q8mi_quantize_core.hpp) and uses IEEE
 // division and square root, which a CPU can follow bit for bit.
 //
-// One 256-thread workgroup per row.  The first six chunks of a thread stay in registers
-// between the two passes (rows of up to 6144 columns are read once); longer rows are read
-// again, from cache.
+// One workgroup per row.  Many rows (a prefill chunk): 256 threads, the first six chunks of a
+// thread stay in registers between the two passes (rows of up to 6144 columns are read once;
+// longer rows are read again, from cache).  Few rows (decode, verify): 1024 threads with two
+// chunks each, so that the serial part of a launch that occupies a handful of CUs -- the
+// quantizer's arithmetic and lane exchanges per chunk -- is a quarter as long; the squares then
+// meet in LDS, where the first 256 threads add them in the order the 256-thread form adds its
+// own (chunks t, t + 256, ...), so both forms give the same bits.
+#include <type_traits>
+
 #include "q8mi_internal.hpp"
 #include "q8mi_quantize_core.hpp"
 
 namespace q8mi {
 namespace {
 
-constexpr uint32_t kHeld = 6;
+constexpr uint32_t kHeld = 6;          // chunks a thread of the 256-thread form keeps
+constexpr uint32_t kWideThreads = 1024;
+constexpr uint32_t kWideHeld = 2;      // ... and of the 1024-thread form (rows of up to 8192 columns)
+constexpr uint32_t kWideMaxBatch = 64; // rows up to which a launch takes the 1024-thread form
 
 struct NormParams {
+    const float *addend;   // ADD: the row normalised is x + addend ...
+    float *sum_out;        // ... which is also written here (rows stride_x apart; may be x or addend)
     const float *x;
     const float *weight;
     float *out;      // may be null when y is set
@@ -60,29 +71,76 @@ __device__ __forceinline__ void store_chunk(float *row, uint32_t c, uint32_t n, 
     if (i + 3 < n) row[i + 3] = v.w;
 }
 
-template <bool VEC, bool QUANT>
-__global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const NormParams p) {
+// ADD: the residual add in front of the norm runs in the same pass (the executors' add_n followed by
+// rms_norm_batch, src/qwen_executor.cpp:6642-6674): a chunk is x + addend, rounded as the stand-alone
+// add rounds it, and goes to sum_out as well.  A thread meets the same chunks in both passes, so the
+// second pass of a long row reads back from sum_out what the thread itself stored in the first.
+template <bool VEC, bool QUANT, bool ADD = false, uint32_t THREADS = kNormThreads>
+__global__ __launch_bounds__(THREADS) void rms_norm_kernel(const NormParams p) {
+    constexpr uint32_t HELD = THREADS == kNormThreads ? kHeld : kWideHeld;
     __shared__ float red[4];
+    __shared__ float squares[THREADS == kNormThreads ? 1 : THREADS];
     const uint32_t j = blockIdx.x, t = threadIdx.x;
     const float *x = p.x + static_cast<uint64_t>(j) * p.stride_x;
     const uint32_t n = p.cols;
     const uint32_t chunks = (n + 3) / 4;
     const Float4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const float *addend = ADD ? p.addend + static_cast<uint64_t>(j) * p.stride_x : nullptr;
+    float *sum_out = ADD ? p.sum_out + static_cast<uint64_t>(j) * p.stride_x : nullptr;
+    auto summed = [&](uint32_t c) {   // chunk c of the row to normalise (first pass)
+        Float4 v = load_chunk<VEC>(x, c, n);
+        if constexpr (ADD) {
+            const Float4 a = load_chunk<VEC>(addend, c, n);
+            v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+            store_chunk<VEC>(sum_out, c, n, v);
+        }
+        return v;
+    };
 
     // the norm weights of the held chunks are requested together with x: one memory round trip, not two
-    Float4 held[kHeld], wheld[kHeld];
+    Float4 held[HELD], wheld[HELD];
     float partial = 0.0f;
 #pragma unroll
-    for (uint32_t u = 0; u < kHeld; ++u) {
-        const uint32_t c = u * kNormThreads + t;
-        held[u] = c < chunks ? load_chunk<VEC>(x, c, n) : zero;
+    for (uint32_t u = 0; u < HELD; ++u) {
+        const uint32_t c = u * THREADS + t;
+        held[u] = c < chunks ? summed(c) : zero;
         wheld[u] = c < chunks ? load_chunk<VEC>(p.weight, c, n) : zero;
     }
+    float sum_squares;
+    if constexpr (THREADS == kNormThreads) {
 #pragma unroll
-    for (uint32_t u = 0; u < kHeld; ++u) partial += chunk_squares(held[u]);   // + 0 for chunks past the end
-    for (uint32_t c = kHeld * kNormThreads + t; c < chunks; c += kNormThreads)
-        partial += chunk_squares(load_chunk<VEC>(x, c, n));
-    const float scale = rms_scale(block_tree_sum_256(partial, red), n, p.eps);
+        for (uint32_t u = 0; u < HELD; ++u) partial += chunk_squares(held[u]);   // + 0 for chunks past the end
+        for (uint32_t c = HELD * THREADS + t; c < chunks; c += THREADS)
+            partial += chunk_squares(summed(c));
+        sum_squares = block_tree_sum_256(partial, red);
+    } else {
+        // rounds of THREADS chunks: thread t of the first 256 adds the squares of chunks t, t + 256, ... of the
+        // round in that order (+ 0 for chunks past the end, which leaves a sum of squares as it is)
+        auto add_round = [&](float sq) {
+            squares[t] = sq;
+            __syncthreads();
+            if (t < kNormThreads) {
+#pragma unroll
+                for (uint32_t u = 0; u < THREADS / kNormThreads; ++u) partial += squares[u * kNormThreads + t];
+            }
+            __syncthreads();
+        };
+#pragma unroll
+        for (uint32_t u = 0; u < HELD; ++u) {
+            if (u * THREADS < chunks) add_round(chunk_squares(held[u]));   // uniform
+        }
+        for (uint32_t base = HELD * THREADS; base < chunks; base += THREADS) {
+            const uint32_t c = base + t;
+            add_round(c < chunks ? chunk_squares(summed(c)) : 0.0f);
+        }
+        if (t < kNormThreads) {   // the first four waves: block_tree_sum_256's tree
+            const float s = wave_sum(partial);
+            if ((t & 63u) == 0) red[t >> 6] = s;
+        }
+        __syncthreads();
+        sum_squares = (red[0] + red[1]) + (red[2] + red[3]);
+    }
+    const float scale = rms_scale(sum_squares, n, p.eps);
 
     // All lanes walk the same trips: the quantizer's lane exchanges need wave-uniform control flow
     // (cols % 32 == 0 there, so the eight lanes of a block are in or out together).
@@ -105,13 +163,13 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const NormParams
         }
     };
 #pragma unroll
-    for (uint32_t u = 0; u < kHeld; ++u) {
-        if (u * kNormThreads < chunks) emit(u * kNormThreads + t, held[u], wheld[u]);   // uniform
+    for (uint32_t u = 0; u < HELD; ++u) {
+        if (u * THREADS < chunks) emit(u * THREADS + t, held[u], wheld[u]);   // uniform
     }
-    for (uint32_t base = kHeld * kNormThreads; base < chunks; base += kNormThreads) {
+    for (uint32_t base = HELD * THREADS; base < chunks; base += THREADS) {
         const uint32_t c = base + t;
         const bool live = c < chunks;
-        emit(c, live ? load_chunk<VEC>(x, c, n) : zero, live ? load_chunk<VEC>(p.weight, c, n) : zero);
+        emit(c, live ? load_chunk<VEC>(ADD ? sum_out : x, c, n) : zero, live ? load_chunk<VEC>(p.weight, c, n) : zero);
     }
 }
 
@@ -122,16 +180,28 @@ int launch(const char *what, const NormParams &p, uint32_t batch, void *stream) 
     if (batch == 0 || p.cols == 0) return Q8MI_OK;
     if (batch > 0x7fffffffu) return fail(Q8MI_REJECTED, "%s: batch %u too large for one launch", what, batch);
     const bool quant = p.y != nullptr;
+    const bool add = p.addend != nullptr;
     const bool vec = p.cols % 4 == 0 && aligned16(p.x) && aligned16(p.weight) && p.stride_x % 4 == 0 &&
-                     (p.out == nullptr || (aligned16(p.out) && p.stride_out % 4 == 0));
+                     (p.out == nullptr || (aligned16(p.out) && p.stride_out % 4 == 0)) &&
+                     (!add || (aligned16(p.addend) && aligned16(p.sum_out)));
     hipStream_t s = as_stream(stream);
-    if (quant) {
-        if (vec) rms_norm_kernel<true, true><<<batch, kNormThreads, 0, s>>>(p);
-        else rms_norm_kernel<false, true><<<batch, kNormThreads, 0, s>>>(p);
-    } else {
-        if (vec) rms_norm_kernel<true, false><<<batch, kNormThreads, 0, s>>>(p);
-        else rms_norm_kernel<false, false><<<batch, kNormThreads, 0, s>>>(p);
-    }
+    auto run = [&](auto vec_tag, auto quant_tag, auto add_tag) {
+        constexpr bool V = decltype(vec_tag)::value, Q = decltype(quant_tag)::value, A = decltype(add_tag)::value;
+        if (batch <= kWideMaxBatch && p.cols > 4 * kNormThreads)
+            rms_norm_kernel<V, Q, A, kWideThreads><<<batch, kWideThreads, 0, s>>>(p);
+        else
+            rms_norm_kernel<V, Q, A, kNormThreads><<<batch, kNormThreads, 0, s>>>(p);
+    };
+    auto by_add = [&](auto vec_tag, auto quant_tag) {
+        if (add) run(vec_tag, quant_tag, std::true_type{});
+        else run(vec_tag, quant_tag, std::false_type{});
+    };
+    auto by_quant = [&](auto vec_tag) {
+        if (quant) by_add(vec_tag, std::true_type{});
+        else by_add(vec_tag, std::false_type{});
+    };
+    if (vec) by_quant(std::true_type{});
+    else by_quant(std::false_type{});
     return check_launch(what);
 }
 
@@ -158,4 +228,19 @@ extern "C" int q8mi_rms_norm_quantize_q8_1(const float *x, const float *weight, 
     p.x = x; p.weight = weight; p.out = normalized; p.y = static_cast<uint8_t *>(y);
     p.cols = cols; p.stride_x = stride_x_row; p.stride_out = stride_normalized_row; p.eps = eps;
     return launch("rms_norm_quantize_q8_1", p, batch, stream);
+}
+
+extern "C" int q8mi_add_rms_norm(const float *a, const float *b, float *sum, const float *weight, float *normalized,
+                                 void *y_q8_1, uint32_t batch, uint32_t cols, uint32_t stride_row,
+                                 uint32_t stride_normalized_row, float eps, void *stream) {
+    if (a == nullptr || b == nullptr || sum == nullptr) return fail(Q8MI_REJECTED, "add_rms_norm: null pointer");
+    if (normalized == nullptr && y_q8_1 == nullptr) return fail(Q8MI_REJECTED, "add_rms_norm: no output");
+    if (y_q8_1 != nullptr && cols % kQK != 0)
+        return fail(Q8MI_REJECTED, "add_rms_norm: cols %u not a multiple of 32 (Q8_1 output)", cols);
+    if (normalized != nullptr && (normalized == a || normalized == b || normalized == sum))
+        return fail(Q8MI_REJECTED, "add_rms_norm: the normalised rows must not overlap the addends or the sum");
+    NormParams p{};
+    p.x = a; p.addend = b; p.sum_out = sum; p.weight = weight; p.out = normalized; p.y = static_cast<uint8_t *>(y_q8_1);
+    p.cols = cols; p.stride_x = stride_row; p.stride_out = stride_normalized_row; p.eps = eps;
+    return launch("add_rms_norm", p, batch, stream);
 }

@@ -26,7 +26,8 @@
 //     up to eight rows also leave the rows' Q8_1 blocks in the scratch, and the operator called
 //     next reads them instead of quantizing again; a one-row rms_norm is held back one call and
 //     runs inside the GEMV when that call is a batch-1 projection of its output (PendingNorm
-//     in the header).  Same bits either way.
+//     in the header); an fp32 add / add_n is held back one call and runs inside the rms_norm_batch
+//     of its sum when that is the next call (PendingAdd).  Same bits either way.
 #include "hip_q8_backend.hpp"
 
 #include <cstdio>
@@ -151,6 +152,7 @@ DeviceStatus HipQ8Backend::end_capture() {
 
 DeviceStatus HipQ8Backend::replay_graph() {
     if (!graph_exec_) return {false, "replay_graph: nothing captured"};
+    if (auto st = flush_norm(); !st.ok) return st;   // eager work still held back comes before the graph
     return hip_status(hipGraphLaunch(graph_exec_, stream_), "hip graph launch");
 }
 
@@ -276,7 +278,16 @@ DeviceStatus HipQ8Backend::quantize_q8_1(const float *x, uint32_t batch, uint32_
 }
 
 // Runs the norm that rms_norm_batch held back, with the quantizer in the same pass.
+DeviceStatus HipQ8Backend::flush_add() {
+    if (!pending_add_.active) return {};
+    const PendingAdd p = pending_add_;
+    pending_add_.active = false;
+    if (q8mi_add(p.out, p.a, p.b, p.count, 0, stream_) != Q8MI_OK) return failed("add");
+    return launch_status("hip add");
+}
+
 DeviceStatus HipQ8Backend::flush_norm() {
+    if (auto st = flush_add(); !st.ok) return st;
     if (!pending_.active) return {};
     const PendingNorm n = pending_;
     pending_.active = false;
@@ -290,6 +301,10 @@ DeviceStatus HipQ8Backend::flush_norm() {
 
 void HipQ8Backend::released(const void *ptr) {
     if (ptr == quantized_.src) forget_quantized();
+    if (pending_add_.active) {
+        if (ptr == pending_add_.out) pending_add_.active = false;   // nobody can read the sum any more
+        else if (ptr == pending_add_.a || ptr == pending_add_.b) (void)flush_add();
+    }
     if (!pending_.active) return;
     if (ptr == pending_.out) pending_.active = false;
     else if (ptr == pending_.x || ptr == pending_.weight) (void)flush_norm();
@@ -465,10 +480,12 @@ DeviceStatus HipQ8Backend::q8_0_matmul(DeviceTensor &out, const DeviceWeight &we
 
 // norm (already applied or to be applied inside the first launch) + projections of up to eight rows:
 // shared by rms_norm_q8_0_matmul_fanout and by a fan-out that follows a held-back one-row norm.
-// xin: the rows before the norm; nrm: where the normalised rows go.
+// xin: the rows before the norm; nrm: where the normalised rows go; add: a held-back add whose sum xin is
+// (batch >= 2), to run inside the norm's launch.
 DeviceStatus HipQ8Backend::fanout_normed(float *nrm, const float *xin, const float *nwp, float eps,
                                          DeviceTensor *const *outs, const DeviceWeight *const *weights,
-                                         const uint32_t *out_strides, uint32_t fanout, uint32_t batch, uint32_t cols) {
+                                         const uint32_t *out_strides, uint32_t fanout, uint32_t batch, uint32_t cols,
+                                         const PendingAdd *add) {
     auto group = [&](uint32_t i0, const uint8_t *(&wp)[4], float *(&op)[4], uint32_t (&r)[4], uint32_t (&s)[4]) {
         for (uint32_t k = 0; k < 4; ++k) { wp[k] = nullptr; op[k] = nullptr; r[k] = 0; s[k] = 0; }
         for (uint32_t i = i0; i < fanout && i < i0 + 4; ++i) {
@@ -498,8 +515,12 @@ DeviceStatus HipQ8Backend::fanout_normed(float *nrm, const float *xin, const flo
     }
     if (first == 0) {
         if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(batch, cols), "q8_1 scratch alloc"); !st.ok) return st;
-        if (q8mi_rms_norm_quantize_q8_1(xin, nwp, nrm, q8_1_.ptr, batch, cols, cols, cols, eps, stream_) != Q8MI_OK)
+        if (add != nullptr) {
+            if (q8mi_add_rms_norm(add->a, add->b, add->out, nwp, nrm, q8_1_.ptr, batch, cols, cols, cols, eps, stream_) != Q8MI_OK)
+                return failed("add_rms_norm");
+        } else if (q8mi_rms_norm_quantize_q8_1(xin, nwp, nrm, q8_1_.ptr, batch, cols, cols, cols, eps, stream_) != Q8MI_OK) {
             return failed("rms_norm_quantize_q8_1");
+        }
         quantized = true;
     }
     for (uint32_t i0 = first; i0 < fanout; i0 += 4) {
@@ -595,13 +616,31 @@ DeviceStatus HipQ8Backend::rms_norm_batch(DeviceTensor &out, const DeviceTensor 
     if (w.format != DeviceWeightFormat::F32 || w.cols < n) return {false, "rms_norm_batch: norm weight is not fp32 [n]"};
     if (T(x).count < static_cast<uint64_t>(batch) * n || T(out).count < static_cast<uint64_t>(batch) * n)
         return {false, "rms_norm_batch: tensor smaller than batch * n"};
-    if (auto st = flush_norm(); !st.ok) return st;
-    wrote(T(out).ptr);
     const float *xin = T(x).f32();
     const float *nwp = reinterpret_cast<const float *>(w.ptr);
     float *nrm = T(out).f32();
     auto aligned16 = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    if (norm_shortcuts_ && batch == 1 && n % 256 == 0 && n <= 6144 && nrm != xin && aligned16(xin) && aligned16(nwp) && aligned16(nrm)) {
+    const bool hold_back = norm_shortcuts_ && batch == 1 && n % 256 == 0 && n <= 6144 && nrm != xin && aligned16(xin) &&
+                           aligned16(nwp) && aligned16(nrm);
+    // the add that produced these rows is still held back: one launch for add, norm (and quantizer)
+    if (pending_add_.active && !hold_back && xin == pending_add_.out &&
+        pending_add_.count == static_cast<uint64_t>(batch) * n && nrm != pending_add_.out && nrm != pending_add_.a &&
+        nrm != pending_add_.b) {
+        const PendingAdd pa = pending_add_;
+        pending_add_.active = false;
+        forget_quantized();
+        const bool quant = batch <= 8 && n % 32 == 0;
+        if (quant)
+            if (auto st = ensure(q8_1_, ported::q8_1_scratch_bytes(batch, n), "q8_1 scratch alloc"); !st.ok) return st;
+        if (q8mi_add_rms_norm(pa.a, pa.b, pa.out, nwp, nrm, quant ? q8_1_.ptr : nullptr, batch, n, n, n, eps, stream_) !=
+            Q8MI_OK)
+            return failed("add_rms_norm");
+        if (quant) quantized_ = QuantizedRows{nrm, batch, n, n};
+        return launch_status("hip add + rms_norm_batch");
+    }
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(T(out).ptr);
+    if (hold_back) {
         pending_ = PendingNorm{true, xin, nwp, nrm, n, eps};
         return {};
     }
@@ -634,7 +673,6 @@ DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized,
                                                        const DeviceWeight &norm_weight, uint32_t batch,
                                                        uint32_t in_stride, float eps) {
     if (fanout == 0 || batch == 0) return {};
-    if (auto st = flush_norm(); !st.ok) return st;
     const auto &nw = W(norm_weight);
     const uint32_t cols = in_stride;
     bool fast = batch <= 8 && cols % 32 == 0 && !T(x).is_bf16() && !T(normalized).is_bf16() &&
@@ -650,9 +688,19 @@ DeviceStatus HipQ8Backend::rms_norm_q8_0_matmul_fanout(DeviceTensor &normalized,
         if (auto st = rms_norm_batch(normalized, x, norm_weight, batch, in_stride, eps); !st.ok) return st;
         return q8_0_matmul_fanout(outs, weights, out_strides, fanout, normalized, batch, in_stride);
     }
-    wrote(T(normalized).ptr);
-    return fanout_normed(T(normalized).f32(), T(x).f32(), reinterpret_cast<const float *>(nw.ptr), eps, outs, weights,
-                         out_strides, fanout, batch, cols);
+    // a held-back add whose sum these rows are (the add_n that ends the layer before): inside the norm's launch
+    PendingAdd add;
+    float *nrm = T(normalized).f32();
+    if (pending_add_.active && batch >= 2 && T(x).f32() == pending_add_.out &&
+        pending_add_.count == static_cast<uint64_t>(batch) * cols && nrm != pending_add_.out && nrm != pending_add_.a &&
+        nrm != pending_add_.b) {
+        add = pending_add_;
+        pending_add_.active = false;
+    }
+    if (auto st = flush_norm(); !st.ok) return st;
+    wrote(nrm);
+    return fanout_normed(nrm, T(x).f32(), reinterpret_cast<const float *>(nw.ptr), eps, outs, weights, out_strides, fanout,
+                         batch, cols, add.active ? &add : nullptr);
 }
 
 // src/kernels_cuda.cu:14818-14862: elementwise out = a + b over the first `count` elements; the
@@ -672,6 +720,10 @@ DeviceStatus HipQ8Backend::add_n(DeviceTensor &out, const DeviceTensor &a, const
     }
     if (auto st = flush_norm(); !st.ok) return st;
     wrote(o.ptr);
+    if (norm_shortcuts_ && !o.is_bf16() && count > 0) {   // held back for the norm that may follow
+        pending_add_ = PendingAdd{true, o.f32(), aa.f32(), bb.f32(), count};
+        return {};
+    }
     if (q8mi_add(o.ptr, aa.ptr, bb.ptr, count, o.is_bf16() ? 1 : 0, stream_) != Q8MI_OK) return failed("add");
     return launch_status("hip add");
 }

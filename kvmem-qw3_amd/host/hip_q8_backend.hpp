@@ -75,15 +75,16 @@ public:
     DeviceStatus begin() { return {}; }
     DeviceStatus end();           // drains the exec stream (src/kernels_cuda.cu:9807-9823)
     DeviceStatus synchronize();
-    // The two shortcuts behind rms_norm_batch (a one-row norm held back for the projection that
-    // reads it; the Q8_1 blocks a 2..8-row norm leaves for the projections that follow) rely on this
-    // backend seeing every write to the tensors involved.  A host that lets other code write those
-    // tensors between the norm and the projection (kernels of its own on exec_stream(), views that
-    // alias them) either calls invalidate_norm_state() before such a write or turns the shortcuts
-    // off; results are the same bits either way, only the launch count changes.
+    // The shortcuts around rms_norm_batch (a one-row norm held back for the projection that reads
+    // it; the Q8_1 blocks a 2..8-row norm leaves for the projections that follow; an fp32 add / add_n
+    // held back for the norm that reads its sum) rely on this backend seeing every read and write of
+    // the tensors involved.  A host that lets other code touch those tensors in between (kernels of
+    // its own on exec_stream(), views that alias them) either calls invalidate_norm_state() before
+    // such an access or turns the shortcuts off; results are the same bits either way, only the
+    // launch count changes.
     void set_norm_shortcuts(bool on);
     bool norm_shortcuts() const { return norm_shortcuts_; }
-    DeviceStatus invalidate_norm_state();   // runs a held-back norm, forgets the cached blocks
+    DeviceStatus invalidate_norm_state();   // runs a held-back add or norm, forgets the cached blocks
     // Called by the destructors of this backend's tensors and weights, before they free `ptr`: a
     // held-back norm that reads it runs now, one that only writes it is dropped (nobody can read
     // the result), cached blocks of its rows are forgotten.
@@ -272,6 +273,16 @@ private:
         uint32_t cols = 0;
         float eps = 0.0f;
     };
+    // An fp32 add / add_n whose launch is held back until the next call: when that call is the
+    // rms_norm_batch of exactly the rows it sums (the batched layer loop's add_n + rms_norm_batch,
+    // src/qwen_executor.cpp:6642-6668), add, norm and quantizer run as one launch; any other call
+    // runs the add first.  Never active together with a PendingNorm.
+    struct PendingAdd {
+        bool active = false;
+        float *out = nullptr;
+        const float *a = nullptr, *b = nullptr;
+        uint64_t count = 0;
+    };
     // What the Q8_1 scratch holds: the blocks of `batch` rows of `cols` floats at `src`, written by
     // the norm that produced those rows.  Valid only until the next call that writes a tensor or
     // the scratch: the projections that follow a norm read them instead of quantizing again.
@@ -279,7 +290,8 @@ private:
         const float *src = nullptr;
         uint32_t batch = 0, cols = 0, stride = 0;
     };
-    DeviceStatus flush_norm();
+    DeviceStatus flush_norm();   // runs whatever is held back (an add, or a norm)
+    DeviceStatus flush_add();
     void forget_quantized() { quantized_ = QuantizedRows{}; }
     bool absorbs_norm(const float *x, uint32_t cols, const void *out0) const;
     DeviceStatus ensure(Scratch &s, size_t need, const char *what);
@@ -293,12 +305,13 @@ private:
     DeviceStatus quantize_d4(const float *x, uint32_t batch, uint32_t cols, uint32_t stride);
     DeviceStatus fanout_normed(float *nrm, const float *xin, const float *nwp, float eps, DeviceTensor *const *outs,
                                const DeviceWeight *const *weights, const uint32_t *out_strides, uint32_t fanout,
-                               uint32_t batch, uint32_t cols);
+                               uint32_t batch, uint32_t cols, const PendingAdd *add = nullptr);
     DeviceStatus gemv_route(float *out, const DeviceWeight &w, const float *x, uint32_t batch, uint32_t in_stride,
                             uint32_t out_stride);
 
     hipStream_t stream_ = nullptr;
     PendingNorm pending_;
+    PendingAdd pending_add_;
     bool norm_shortcuts_ = true;
     std::shared_ptr<Owner> owner_;
     QuantizedRows quantized_;

@@ -72,6 +72,7 @@ SIGNATURES = {
                                   _u32, _u32, _u32, _u32, _u32, _vp]),
     "q8mi_rms_norm": (_int, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_float, _vp]),
     "q8mi_rms_norm_quantize_q8_1": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_float, _vp]),
+    "q8mi_add_rms_norm": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_float, _vp]),
     "q8mi_nqgemv": (_int, [_vp, _vp, _vp, C.c_float, _vp, _vp, _int, _u32, _u32, _u32, _vp]),
     "q8mi_nqgemv_silu_mul": (_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _u32, _u32, _u32, _vp]),
     "q8mi_nqgemv_fanout4": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,

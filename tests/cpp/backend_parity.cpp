@@ -680,6 +680,138 @@ void case_norm_reuse(qw3::HipQ8Backend &b) {
     }
 }
 
+// add / add_n held back for the norm of its sum (the batched layer loop's add_n + rms_norm_batch):
+// the sum, the normalised rows and the projection behind them are the bits of the separate
+// launches, whatever call comes next.
+void case_add_held_back(qw3::HipQ8Backend &b) {
+    std::string d;
+    const uint32_t cols = 2048, rows = 640;
+    const float eps = 1e-6f;
+    const HostWeight w = make_weight(rows, cols, 701);
+    auto dw = b.weight_q8_0(w.gguf.data(), rows, cols, "w");
+    auto nwv = normal_vec(cols, 704, 0.4f);
+    for (auto &f : nwv) f += 1.0f;
+    auto nw = b.weight_f32(nwv.data(), cols, "norm.weight");
+    auto bits_equal = [](const std::vector<float> &a, const std::vector<float> &c) {
+        return a.size() == c.size() && std::memcmp(a.data(), c.data(), a.size() * 4) == 0;
+    };
+    for (uint32_t batch : {1u, 2u, 8u, 9u, 40u}) {
+        const size_t n = static_cast<size_t>(batch) * cols;
+        const auto hv = normal_vec(n, 710 + batch, 2.0f), dv = normal_vec(n, 720 + batch, 0.7f);
+        std::vector<float> sum(n), nref(n);
+        for (size_t i = 0; i < n; ++i) sum[i] = hv[i] + dv[i];
+        q8o_rms_norm(sum.data(), nwv.data(), nref.data(), batch, cols, cols, cols, eps);
+        std::vector<float> ref, mag;
+        oracle_linear(w, nref.data(), batch, cols, rows, ref, mag);
+        auto delta = upload_f32(b, dv);
+        auto norm = b.tensor_f32(n, "n");
+        auto out = b.tensor_f32(static_cast<size_t>(batch) * rows, "o");
+        std::vector<float> first_out;
+        for (int shortcuts = 1; shortcuts >= 0; --shortcuts) {
+            b.set_norm_shortcuts(shortcuts != 0);
+            auto h = upload_f32(b, hv);
+            bool ok = require(b.zero_tensor(*norm), "zero") && require(b.add_n(*h, *h, *delta, n), "add_n in place") &&
+                      require(b.rms_norm_batch(*norm, *h, *nw, batch, cols, eps), "norm of the sum") &&
+                      require(b.q8_0_matmul(*out, *dw, *norm, batch, cols, rows), "projection");
+            ok = ok && bits_equal(download_f32(b, *h), sum) && bits_equal(download_f32(b, *norm), nref);
+            const auto got = download_f32(b, *out);
+            if (batch <= 8) ok = ok && close_fp32(got, ref, mag, batch, rows, rows, d);
+            if (shortcuts) first_out = got;
+            else ok = ok && bits_equal(got, first_out);
+            report(("add_then_norm_batch" + std::to_string(batch) + (shortcuts ? "" : "_shortcuts_off")).c_str(), ok, d);
+        }
+        b.set_norm_shortcuts(true);
+        // the same in front of the fused norm + fan-out operator (the add_n that ends a layer, then the next layer's first call)
+        std::vector<float> first_fan;
+        for (int shortcuts = 1; shortcuts >= 0; --shortcuts) {
+            b.set_norm_shortcuts(shortcuts != 0);
+            auto h = upload_f32(b, hv);
+            qw3::DeviceTensor *outs[1] = {out.get()};
+            const qw3::DeviceWeight *ws[1] = {dw.get()};
+            const uint32_t strides[1] = {rows};
+            bool ok = require(b.zero_tensor(*norm), "zero") && require(b.zero_tensor(*out), "zero") &&
+                      require(b.add_n(*h, *h, *delta, n), "add_n in place") &&
+                      require(b.rms_norm_q8_0_matmul_fanout(*norm, outs, ws, strides, 1, *h, *nw, batch, cols, eps), "norm + fan-out of the sum");
+            ok = ok && bits_equal(download_f32(b, *h), sum) && bits_equal(download_f32(b, *norm), nref);
+            const auto got = download_f32(b, *out);
+            if (batch <= 8) ok = ok && close_fp32(got, ref, mag, batch, rows, rows, d);
+            if (shortcuts) first_fan = got;
+            else ok = ok && bits_equal(got, first_fan);
+            report(("add_then_norm_fanout_batch" + std::to_string(batch) + (shortcuts ? "" : "_shortcuts_off")).c_str(), ok, d);
+        }
+        b.set_norm_shortcuts(true);
+    }
+    {
+        const uint32_t batch = 4;
+        const size_t n = static_cast<size_t>(batch) * cols;
+        const auto hv = normal_vec(n, 731, 2.0f), dv = normal_vec(n, 732, 0.7f);
+        std::vector<float> sum(n), nref(n), nplain(n);
+        for (size_t i = 0; i < n; ++i) sum[i] = hv[i] + dv[i];
+        q8o_rms_norm(sum.data(), nwv.data(), nref.data(), batch, cols, cols, cols, eps);
+        q8o_rms_norm(hv.data(), nwv.data(), nplain.data(), batch, cols, cols, cols, eps);
+        auto delta = upload_f32(b, dv);
+        // out of place, and read back right away: the add runs before the copy
+        auto h = upload_f32(b, hv);
+        auto s = b.tensor_f32(n, "s");
+        bool ok = require(b.add(*s, *h, *delta), "add") && bits_equal(download_f32(b, *s), sum) && bits_equal(download_f32(b, *h), hv);
+        // the norm of another tensor comes next: the add runs first, the norm is that tensor's
+        auto norm = b.tensor_f32(n, "n");
+        ok = ok && require(b.add_n(*s, *h, *delta, n), "add_n") && require(b.rms_norm_batch(*norm, *h, *nw, batch, cols, eps), "norm of h") &&
+             bits_equal(download_f32(b, *norm), nplain) && bits_equal(download_f32(b, *s), sum);
+        // fewer elements than the norm covers: no fusion, rows past the count keep their values
+        auto h2 = upload_f32(b, hv);
+        std::vector<float> part = hv;
+        for (size_t i = 0; i < n - cols; ++i) part[i] = sum[i];
+        std::vector<float> npart(n);
+        q8o_rms_norm(part.data(), nwv.data(), npart.data(), batch, cols, cols, cols, eps);
+        ok = ok && require(b.add_n(*h2, *h2, *delta, n - cols), "add_n of three rows") &&
+             require(b.rms_norm_batch(*norm, *h2, *nw, batch, cols, eps), "norm of four") && bits_equal(download_f32(b, *h2), part) &&
+             bits_equal(download_f32(b, *norm), npart);
+        // the norm writes over the addend: separate launches, add first
+        auto h3 = upload_f32(b, hv);
+        auto d3 = upload_f32(b, dv);
+        ok = ok && require(b.add_n(*h3, *h3, *d3, n), "add_n") && require(b.rms_norm_batch(*d3, *h3, *nw, batch, cols, eps), "norm into the addend") &&
+             bits_equal(download_f32(b, *h3), sum) && bits_equal(download_f32(b, *d3), nref);
+        report("add_held_back_other_calls_next", ok);
+
+        // tensors destroyed while the add is held back
+        auto h4 = upload_f32(b, hv);
+        auto d4 = upload_f32(b, dv);
+        ok = require(b.add_n(*h4, *h4, *d4, n), "add_n");
+        d4.reset();                                   // the addend goes: the add runs first
+        ok = ok && bits_equal(download_f32(b, *h4), sum);
+        auto gone = b.tensor_f32(n, "gone");
+        ok = ok && require(b.add(*gone, *h4, *delta), "add into a tensor about to go");
+        gone.reset();
+        ok = ok && require(b.synchronize(), "sync") && bits_equal(download_f32(b, *h4), sum);
+        report("add_held_back_tensors_destroyed", ok);
+
+        // under capture: add + norm + projection as a graph, replays equal the eager run
+        auto h5 = upload_f32(b, hv);
+        auto out = b.tensor_f32(static_cast<size_t>(batch) * rows, "o");
+        auto body = [&]() {
+            return b.add_n(*h5, *h5, *delta, n).ok && b.rms_norm_batch(*norm, *h5, *nw, batch, cols, eps).ok &&
+                   b.q8_0_matmul(*out, *dw, *norm, batch, cols, rows).ok;
+        };
+        ok = body() && require(b.synchronize(), "sync");
+        const auto eager = download_f32(b, *out);
+        ok = ok && bits_equal(download_f32(b, *h5), sum);
+        ok = ok && b.begin_capture() && body();
+        ok = require(b.end_capture(), "end_capture") && ok;
+        for (int rep = 0; rep < 3 && ok; ++rep) {
+            ok = require(b.copy_bytes_from_host(*h5, 0, hv.data(), n * 4), "reset h") && require(b.zero_tensor(*out), "zero") &&
+                 require(b.replay_graph(), "replay") && require(b.synchronize(), "sync");
+            ok = ok && bits_equal(download_f32(b, *out), eager) && bits_equal(download_f32(b, *h5), sum);
+        }
+        // an add left pending when the capture ends is part of the graph
+        ok = ok && b.begin_capture() && b.add_n(*h5, *h5, *delta, n).ok;
+        ok = require(b.end_capture(), "end_capture") && ok;
+        ok = ok && require(b.copy_bytes_from_host(*h5, 0, hv.data(), n * 4), "reset h") && require(b.replay_graph(), "replay") &&
+             bits_equal(download_f32(b, *h5), sum);
+        report("add_held_back_under_capture", ok);
+    }
+}
+
 void case_argmax(qw3::HipQ8Backend &b) {
     std::string d;
     const uint32_t n = 248320;
@@ -1045,7 +1177,7 @@ int main(int argc, char **argv) {
     struct Case { const char *name; void (*fn)(qw3::HipQ8Backend &); };
     const Case cases[] = {
         {"closed_form", case_closed_form}, {"matvec", case_matvec_family}, {"matmul", case_matmul},
-        {"matmul_add", case_matmul_add_batched}, {"silu_mul", case_silu_mul}, {"norm_reuse", case_norm_reuse},
+        {"matmul_add", case_matmul_add_batched}, {"silu_mul", case_silu_mul}, {"norm_reuse", case_norm_reuse}, {"add_held_back", case_add_held_back},
         {"argmax", case_argmax}, {"get_rows", case_get_rows}, {"gguf", case_gguf}, {"lm_head", case_lm_head_verify}, {"rms_norm", case_rms_norm}, {"graph", case_graph_replay},
     };
     for (const auto &c : cases) {

@@ -30,7 +30,7 @@ def u32(a):
 
 
 @pytest.mark.parametrize("n", [1, 3, 4, 31, 257, 1024, 1027, 5120, 6144, 6148, 17408, 40000])
-@pytest.mark.parametrize("batch", [1, 5])
+@pytest.mark.parametrize("batch", [1, 5, 70])
 def test_rms_norm_bits(gpu, oracle, n, batch):
     L = gpu.lib()
     stride = n + (8 if n % 4 == 0 else 3)
@@ -62,7 +62,7 @@ def test_rms_norm_unaligned_pointers_and_padded_output(gpu, oracle):
 
 
 @pytest.mark.parametrize("cols", [32, 256, 5120, 6144, 8192, 17408])
-@pytest.mark.parametrize("batch", [1, 6])
+@pytest.mark.parametrize("batch", [1, 6, 67])
 def test_rms_norm_quantize_bits(gpu, oracle, cols, batch):
     L = gpu.lib()
     stride = cols + 16
@@ -252,3 +252,57 @@ def test_rms_norm_non_finite_rows(gpu, oracle):
     gd, rd = gy[:, :4].copy().view(np.float16), ry[:, :4].copy().view(np.float16)
     assert np.array_equal(np.isnan(gd), np.isnan(rd))
     assert np.array_equal(gd[~np.isnan(rd)], rd[~np.isnan(rd)])
+
+
+@pytest.mark.parametrize("cols,batch,in_place", [(5120, 1, True), (5120, 8, True), (5120, 5, False), (6144, 3, True),
+                                                 (8192, 2, True), (17408, 4, True), (40000, 2, False), (256, 7, True),
+                                                 (1027, 3, True), (6148, 2, False), (5120, 300, True)])
+def test_add_rms_norm_is_add_then_norm(gpu, oracle, cols, batch, in_place):
+    """sum = a + b, then the norm (and the quantizer) of sum, in one launch: the bits of q8mi_add followed
+    by q8mi_rms_norm / q8mi_rms_norm_quantize_q8_1, and of the oracle's chain; in place (sum = a) and out
+    of place, rows held in registers and rows read twice, vector and scalar loads."""
+    L = gpu.lib()
+    a, w = rows_of(cols, batch, seed=7 * cols + batch)
+    b, _ = rows_of(cols, batch, seed=11 * cols + batch)
+    if cols % 32 == 0:
+        a[0, :32] = 0.0
+        b[0, :32] = 0.0      # an all-zero block after the add
+    ref_sum = (a + b).astype(np.float32)
+    ref_n = oracle.rms_norm(ref_sum, w, EPS)
+    dw, db = dev(w), dev(b)
+    quant = cols % 32 == 0
+    nbytes = L.q8mi_q8_1_scratch_bytes(batch, cols) if quant else 16
+    for with_normalized in ((True, False) if quant else (True,)):
+        da = dev(a)
+        dsum = da if in_place else hip.DeviceBuffer(4 * batch * cols).fill(0xee)
+        nrm = hip.DeviceBuffer(4 * batch * cols).fill(0xee)
+        y = hip.DeviceBuffer(nbytes).fill(0xee)
+        ok(L.q8mi_add_rms_norm(da.ptr, db.ptr, dsum.ptr, dw.ptr, nrm.ptr if with_normalized else NULL,
+                               y.ptr if quant else NULL, batch, cols, cols, cols, EPS, NULL), "add_rms_norm")
+        hip.synchronize()
+        assert np.array_equal(dsum.download(np.uint32), u32(ref_sum).reshape(-1)), "the sum"
+        if not in_place:
+            assert np.array_equal(da.download(np.uint32), u32(a).reshape(-1)), "a is left alone"
+        if with_normalized:
+            assert np.array_equal(nrm.download(np.uint32), u32(ref_n).reshape(-1)), "the normalised rows"
+        if quant:
+            rc, ref_y = oracle.quantize_q8_1(ref_n)
+            assert rc == 0 and np.array_equal(y.download(np.uint8), ref_y), "the Q8_1 blocks"
+    # the two launches it replaces
+    da2 = dev(a)
+    nrm2 = hip.DeviceBuffer(4 * batch * cols)
+    ok(L.q8mi_add(da2.ptr, da2.ptr, db.ptr, batch * cols, 0, NULL), "add")
+    ok(L.q8mi_rms_norm(da2.ptr, dw.ptr, nrm2.ptr, batch, cols, cols, cols, EPS, NULL), "rms_norm")
+    hip.synchronize()
+    assert np.array_equal(da2.download(np.uint32), u32(ref_sum).reshape(-1))
+    assert np.array_equal(nrm2.download(np.uint32), u32(ref_n).reshape(-1))
+
+
+def test_add_rms_norm_rejections(gpu):
+    L = gpu.lib()
+    b, c, d = hip.DeviceBuffer(4096), hip.DeviceBuffer(4096), hip.DeviceBuffer(4096)
+    assert L.q8mi_add_rms_norm(b.ptr, c.ptr, b.ptr, c.ptr, NULL, NULL, 1, 64, 64, 64, EPS, NULL) == q8mi.REJECTED   # no output
+    assert L.q8mi_add_rms_norm(b.ptr, c.ptr, b.ptr, c.ptr, b.ptr, NULL, 1, 64, 64, 64, EPS, NULL) == q8mi.REJECTED  # normalised over the sum
+    assert L.q8mi_add_rms_norm(b.ptr, c.ptr, b.ptr, c.ptr, NULL, d.ptr, 1, 48, 48, 48, EPS, NULL) == q8mi.REJECTED  # Q8_1 of 48 columns
+    assert L.q8mi_add_rms_norm(NULL, c.ptr, b.ptr, c.ptr, d.ptr, NULL, 1, 64, 64, 64, EPS, NULL) == q8mi.REJECTED
+    ok(L.q8mi_add_rms_norm(b.ptr, c.ptr, b.ptr, c.ptr, d.ptr, NULL, 0, 64, 64, 64, EPS, NULL), "empty batch")
