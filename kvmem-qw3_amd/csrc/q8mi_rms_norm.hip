@@ -103,8 +103,22 @@ __global__ __launch_bounds__(THREADS) void rms_norm_kernel(const NormParams p) {
 #pragma unroll
     for (uint32_t u = 0; u < HELD; ++u) {
         const uint32_t c = u * THREADS + t;
-        held[u] = c < chunks ? summed(c) : zero;
+        held[u] = c < chunks ? load_chunk<VEC>(x, c, n) : zero;
         wheld[u] = c < chunks ? load_chunk<VEC>(p.weight, c, n) : zero;
+    }
+    if constexpr (ADD) {   // all loads of the held chunks before the first store (which may be to x itself)
+        Float4 aheld[HELD];
+#pragma unroll
+        for (uint32_t u = 0; u < HELD; ++u) {
+            const uint32_t c = u * THREADS + t;
+            aheld[u] = c < chunks ? load_chunk<VEC>(addend, c, n) : zero;
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < HELD; ++u) {
+            const uint32_t c = u * THREADS + t;
+            held[u].x += aheld[u].x; held[u].y += aheld[u].y; held[u].z += aheld[u].z; held[u].w += aheld[u].w;
+            if (c < chunks) store_chunk<VEC>(sum_out, c, n, held[u]);
+        }
     }
     float sum_squares;
     if constexpr (THREADS == kNormThreads) {
