@@ -531,7 +531,15 @@ int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     // four 29.4; fan-out (4096 pairs) one 8.7, two 9.0, four 9.0.  At batch 2: SwiGLU two 30.8, four 30.2;
     // fan-out two 9.5, four 9.3; 5120 x 6144 (2560 pairs) two 8.0, four 8.2.  At batch 3: SwiGLU four 32.7,
     // eight 32.0; 5120 x 6144 four 9.2, eight 10.8.
-    if (NSTEPS / WAVES >= 3) ps.ppw = 2;   // rows of three and more steps per wave (15 and 17 KiB)
+    // Rows of three and more steps per wave (15 and 17 KiB): two pairs, or as many as leave exactly two
+    // workgroups per CU when the pairs divide that way (5120 x 17408: five pairs 16.3 us against 16.6 at
+    // batch 1, 17.0 against 18.2 at batch 2; 4096 x 17408: four pairs 13.6 against 13.9 and 14.3 against 15.4;
+    // 5120 x 15360: 15.6 against 15.5 and 16.5 against 17.9).
+    if (NSTEPS / WAVES >= 3) {
+        const uint32_t two_per_cu = 2u * static_cast<uint32_t>(device_cu_count());
+        const uint32_t even = ps.pairs / two_per_cu;
+        ps.ppw = (ps.pairs % two_per_cu == 0 && even >= 2 && even <= kKsplitMaxPairs) ? even : 2;
+    }
     else if (M == 1) ps.ppw = ps.pairs >= 8192 ? 2 : 1;
     else if (M == 2) ps.ppw = ps.pairs >= 4096 ? 4 : 2;
     else ps.ppw = ps.pairs >= 8192 ? 8 : 4;
