@@ -72,6 +72,7 @@ def shared_row_cases(seed, n):
         out.append((int(rng.integers(1, 300)), 1024 * kib, 2))
     out += [(700, 2048, 3), (431, 3072, 4), (9000, 2048, 4), (17001, 1024, 2), (300, 1024, 3)]   # 1 .. 3 KiB at batch 2 .. 4
     out += [(700, 7168, 3), (333, 12288, 4), (50, 3328, 2), (50, 2560, 1)]   # lengths and batches other kernels serve
+    out += [(5120, 15360, 2), (3072, 17408, 1), (2048, 17408, 2)]   # long rows whose pairs leave two workgroups per CU
     return out
 
 
