@@ -327,9 +327,13 @@ int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
     p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
     p.x_bytes = mfma_x_lds_bytes(p.nb, batch, MG, HS);
     p.interleave = kGemvInterleave;
-    // the streaming hint pays on long streams only (measured at batch 4: 2 x 17408 x 5120 36.2 -> 33.6 us,
-    // 5120 x 17408 22.0 -> 20.6 us, but 8192 x 5120 11.7 -> 12.5 us and 5120 x 6144 10.1 -> 10.8 us)
-    constexpr uint64_t kStreamFrom = 64ull * 1000 * 1000;
+    // The streaming hint on the weight loads.  Launches timed back to back on their own gain from it on long
+    // streams only (batch 4: 2 x 17408 x 5120 36.2 -> 33.6 us, 5120 x 17408 22.0 -> 20.6 us, but 8192 x 5120
+    // 11.7 -> 12.5 us and 5120 x 6144 10.1 -> 10.8 us).  In a layer's sequence of launches it pays on those two
+    // as well: with the hint on the fan-out and the O projection too, the eight-launch layer step takes 88.1 us
+    // instead of 90.3 at batch 6 and 89.9 instead of 92.1 at batch 8 -- weights a launch leaves in the caches
+    // are in the way of the launches behind it.  So every launch of a megabyte and more carries it.
+    constexpr uint64_t kStreamFrom = 1ull * 1000 * 1000;
     const bool streaming = (SILU ? 2ull : 1ull) * p.total_rows * p.nb * 34 >= kStreamFrom;
     const uint32_t grid = p.units < cus ? p.units : cus;
     const uint32_t nitems = (p.nb + kMfmaItemBlocks - 1) / kMfmaItemBlocks;
