@@ -661,6 +661,31 @@ def bench_batch_sweep(q8mi, hip, step, layers, steps):
     return sweep
 
 
+def bench_small_launch_cost(q8mi, hip, synth, layers, reps=400):
+    """What a small launch costs behind a large one on the same stream: the batch-8 down projection back to
+    back on its own, followed by a 4 KB read, and followed by the batch-8 quantizer of 5120 columns
+    (microseconds per repetition).  A kernel trace shows such a small dispatch open for 4 to 5 us, because it
+    is open while the launch in front of it drains; what it adds to the sequence is the difference here."""
+    L, ok = q8mi.lib(), q8mi.ok
+    st = DecodeStep(q8mi, hip, m=8)
+    ok(L.q8mi_quantize_q8_1(st.ffn.ptr, st.y17408.ptr, 8, FFN, FFN, None), "quantize ffn")
+    sink, small = hip.DeviceBuffer(64), hip.DeviceBuffer(4096)
+    down = lambda i: ok(L.q8mi_gemv_add(layers[i % len(layers)].w["down"].ptr, st.y17408.ptr, st.h.ptr, HIDDEN, FFN, 8,
+                                        HIDDEN, None), "down")
+    def with_read(i):
+        down(i)
+        synth.ok(synth.lib().q8sup_probe_read(small.ptr, 4096, 2, sink.ptr, None), "probe_read")
+    def with_quantizer(i):
+        down(i)
+        ok(L.q8mi_quantize_q8_1(st.x.ptr, st.y5120.ptr, 8, HIDDEN, HIDDEN, None), "quantize x")
+    out = {}
+    for name, fn in (("down_m8_alone_us", down), ("followed_by_a_4kb_read_us", with_read),
+                     ("followed_by_the_m8_quantizer_us", with_quantizer)):
+        settle(hip, fn, ms=10.0)
+        out[name] = round(time_loop(hip, fn, reps, 20) * 1e3, 2)
+    return out
+
+
 def bench_lm_head(q8mi, hip, synth, reps=100):
     """Fused LM head (5120 x 248320) + argmax + accept at M = 1, 2, 4, 6, 8."""
     L, ok = q8mi.lib(), q8mi.ok
@@ -762,7 +787,8 @@ def main():
     if args.only == "sweep":
         layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
         print(json.dumps({"gemv_layer_gbps_by_m": bench_batch_sweep(q8mi, hip, DecodeStep(q8mi, hip, m=1), layers,
-                                                                     max(args.steps // 2, 300))}))
+                                                                     max(args.steps // 2, 300)),
+                          "small_launch_behind_a_large_one": bench_small_launch_cost(q8mi, hip, synth, layers)}))
         return
     counter_calibration(synth, hip)
     layers = [Layer(synth, hip, seed=s + 1) for s in range(args.copies)]
@@ -816,6 +842,7 @@ def main():
         result["graph_replay"] = {"ms_per_step": round(ms_graph, 5), "steps_per_graph": per_graph,
                                   "gbps": round(step_bytes / (ms_graph * 1e-3) / 1e9, 1)}
         result["gemv_layer_gbps_by_m"] = bench_batch_sweep(q8mi, hip, step, layers, max(args.steps // 2, 300))
+        result["small_launch_behind_a_large_one"] = bench_small_launch_cost(q8mi, hip, synth, layers)
         # the layer's two RMS norms in front of the fan-out and the SwiGLU: inside those launches, or on their own
         norms = {}
         for name, one in (("norms_inside_the_gemv_5_launches", True), ("norm_quantizer_kernels_7_launches", False)):
