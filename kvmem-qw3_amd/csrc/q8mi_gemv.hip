@@ -318,16 +318,19 @@ int launch_m(const GemvParams &p, hipStream_t stream) {
 
 constexpr uint64_t kMfmaShallowMaxRows = 65536;
 
-// One workgroup of 512 threads (768 on short rows, below) per CU: its waves split the items of its units
+// One workgroup of 512 threads (768 where measured better, below) per CU: its waves split the items of its units
 // evenly, so a matrix only needs as many 4-row units as there are CUs to keep the chip busy.
 template <int MG, bool SILU, bool HS, bool D4, int DEPTH, int THREADS = 512>   // 256 and 1024 threads are 10..35 % slower at batch 4 and 8
 int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
-    if constexpr (THREADS == 512 && MG == 2 && !SILU && !D4 && !HS && DEPTH == 1) {
-        // Rows of up to six items at five to eight activation rows (the fan-out and the O projection of a verify
-        // step): a wave's share is four or five items, one memory round trip each, and twelve waves make it three
-        // or four (layer step at batch 6 / 8: 88.6 / 90.0 -> 88.0 / 89.5 us; ten waves 88.1 / 89.7, fourteen
-        // 89.0 / 90.3).  On long rows and on the SwiGLU twelve waves lose (35.1 against 32.6 us).
-        if (p.nb <= 6 * kMfmaItemBlocks) return launch_mfma_depth<MG, SILU, HS, D4, DEPTH, 768>(p, batch, stream);
+    if constexpr (THREADS == 512 && MG == 2 && !SILU && !D4 && DEPTH == 1) {
+        // Five to eight activation rows, every form but the SwiGLU: twelve waves.  A wave's share of a short-row
+        // launch (the fan-out and the O projection of a verify step) is then three or four items -- one memory
+        // round trip each -- instead of four or five, and eight instead of eleven on the down projection.  Layer
+        // step at batch 6 / 8 with twelve waves on the short rows: 88.6 / 90.0 -> 88.0 / 89.5 us (ten waves 88.1 /
+        // 89.7, fourteen 89.0 / 90.3); on the down projection as well: 87.4 / 88.7.  The SwiGLU loses with twelve
+        // (35.1 against 32.6 us), the down projection of three and four rows is the same either way.  A shape whose parked sums do not fit with twelve waves takes eight.
+        const int rc = launch_mfma_depth<MG, SILU, HS, D4, DEPTH, 768>(p, batch, stream);
+        if (rc != Q8MI_REJECTED) return rc;
     }
     const uint32_t cus = static_cast<uint32_t>(device_cu_count());
     p.units = SILU ? (p.total_rows + 1) / 2 : (p.total_rows + 3) / 4;
