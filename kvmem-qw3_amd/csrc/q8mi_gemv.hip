@@ -318,10 +318,17 @@ int launch_m(const GemvParams &p, hipStream_t stream) {
 
 constexpr uint64_t kMfmaShallowMaxRows = 65536;
 
-// One workgroup of 512 threads (768 where measured better, below) per CU: its waves split the items of its units
+// One workgroup of 512 threads (448 or 768 where measured better, below) per CU: its waves split the items of its units
 // evenly, so a matrix only needs as many 4-row units as there are CUs to keep the chip busy.
 template <int MG, bool SILU, bool HS, bool D4, int DEPTH, int THREADS = 512>   // 256 and 1024 threads are 10..35 % slower at batch 4 and 8
 int launch_mfma_depth(GemvParams p, uint32_t batch, hipStream_t stream) {
+    if constexpr (THREADS == 512 && MG == 1 && SILU && !D4 && DEPTH == 1) {
+        // The SwiGLU at three and four activation rows: seven waves (layer step at batch 3 / 4: 80.2 / 83.1 ->
+        // 79.7 / 82.5 us; six waves 80.8 / 83.8; at five to eight rows eight waves stay ahead, 87.0 / 88.4 against
+        // 87.8 / 89.1 with seven).
+        const int rc = launch_mfma_depth<MG, SILU, HS, D4, DEPTH, 448>(p, batch, stream);
+        if (rc != Q8MI_REJECTED) return rc;
+    }
     if constexpr (THREADS == 512 && MG == 2 && !SILU && !D4 && DEPTH == 1) {
         // Five to eight activation rows, every form but the SwiGLU: twelve waves.  A wave's share of a short-row
         // launch (the fan-out and the O projection of a verify step) is then three or four items -- one memory
