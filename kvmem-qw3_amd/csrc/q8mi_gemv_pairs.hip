@@ -542,7 +542,7 @@ int launch_ksplit(const GemvParams &p, PairSpace ps, hipStream_t stream) {
     }
     else if (M == 1) ps.ppw = ps.pairs >= 8192 ? 2 : 1;
     else if (M == 2) ps.ppw = ps.pairs >= 4096 ? 4 : 2;
-    else ps.ppw = ps.pairs >= 8192 ? 8 : 4;
+    else ps.ppw = ps.pairs >= 8192 ? 8 : ps.pairs >= 4096 ? 4 : 2;   // 5120 x 6144 (2560 pairs), two against four: 8.4 / 8.8 us at batch 3, 9.4 / 9.8 at batch 4
     const uint32_t grid = (ps.pairs + ps.ppw - 1) / ps.ppw;
     if (p.mode == kSiluMul) gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES, true><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
     else gemv_pairs_ksplit_kernel<M, NSTEPS, WAVES, false><<<grid, WAVES * kWave, 0, stream>>>(p, ps);
